@@ -1,0 +1,190 @@
+#!/usr/bin/env python3
+"""Benchmark of the tile-wise-sparse GEMM engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+
+A step is one TW GEMM  C = A * (B (.) mask)  over one batch of synthetic input that
+is already resident in HBM.  The default workload is VGG16 conv4_2 as an im2col GEMM
+(M=12544, K=4608, N=512, G=128, 75 % tile-wise sparsity, fp16 in / fp32 accumulate).
+Prints ONE JSON line: effective TFLOP/s (dense flops / time), with the speedup over the
+same kernel on the 0 %-sparse plan, the roofline of the kernel and the CPU baseline
+(NumPy masked dense matmul, the reference's CPU path) timed on this box's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
+
+
+def make_workload(name):
+    from tilesparsity_amd import workloads as W
+    table = {
+        "vgg16_conv4_2": W.vgg16_conv4_2,
+        "bert_base_ffn": W.bert_base_ffn,
+        "nmt_lstm_gates": W.nmt_lstm_gates,
+        "bert_large_ffn1_50": lambda: W.bert_large_ffn(1, 0.50),
+        "bert_large_ffn1_75": lambda: W.bert_large_ffn(1, 0.25),
+        "bert_large_ffn1_90": lambda: W.bert_large_ffn(1, 0.10),
+        "bert_large_ffn2_50": lambda: W.bert_large_ffn(2, 0.50),
+        "bert_large_ffn2_75": lambda: W.bert_large_ffn(2, 0.25),
+        "bert_large_ffn2_90": lambda: W.bert_large_ffn(2, 0.10),
+        "imbalance_stress": W.imbalance_stress,
+    }
+    return table[name]()
+
+
+def time_plan(plan, bufs, M, steps, warmup, torch):
+    """Average seconds per launch over `steps` back-to-back launches, timed with events on
+    the stream the kernel runs on; buffers rotate so that A and C come from HBM."""
+    stream = torch.cuda.current_stream()
+    s = stream.cuda_stream
+    n = len(bufs)
+    for i in range(warmup):
+        a, c = bufs[i % n]
+        plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    for i in range(steps):
+        a, c = bufs[i % n]
+        plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+    stop.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20):
+    from tilesparsity_amd import twgemm as tw
+    from tilesparsity_amd import workloads as W
+    M, K, N, G, dtype, tiles = wl["M"], wl["K"], wl["N"], wl["G"], wl["dtype"], wl["tiles"]
+    A, B = wl["values"]()
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    # K-major operands: A^T [K, M], C^T [N, M]
+    At = torch.from_numpy(A).cuda().to(tdt).t().contiguous()
+    per_set = (At.numel() + N * M) * 2
+    n_sets = max(2, min(8, -(-rotate_bytes // per_set)))
+    bufs = [(At if i == 0 else At.clone(), torch.zeros((N, M), dtype=tdt, device="cuda"))
+            for i in range(n_sets)]
+    sparse = tw.Plan.create(K, N, dtype, tiles, B)
+    dense = tw.Plan.dense(K, N, G, dtype, B)
+    t_sparse = time_plan(sparse, bufs, M, steps, warmup, torch)
+    t_dense = time_plan(dense, bufs, M, max(3, steps // 4), max(2, warmup // 4), torch)
+    sparse.destroy()
+    dense.destroy()
+    fk, fd = W.flops_kept(M, tiles), W.flops_dense(M, K, N)
+    by = W.algorithmic_bytes(M, K, N, tiles)
+    res = dict(
+        workload=wl["name"], M=M, K=K, N=N, G=G, dtype=dtype, seed=wl["seed"], n_tiles=len(tiles),
+        us_sparse=t_sparse * 1e6, us_dense=t_dense * 1e6,
+        effective_tflops=fd / t_sparse / 1e12, actual_tflops=fk / t_sparse / 1e12,
+        dense_tflops=fd / t_dense / 1e12, speedup_vs_dense=t_dense / t_sparse,
+        mfma_util_kept=fk / t_sparse / 1e12 / MFMA_PEAK_TFLOPS,
+        mfma_util_dense_run=fd / t_dense / 1e12 / MFMA_PEAK_TFLOPS,
+        algorithmic_bytes=by, hbm_gbs=by / t_sparse / 1e9, rotating_buffer_sets=n_sets,
+        kept_flops=fk, dense_flops=fd)
+    del bufs, At
+    torch.cuda.empty_cache()
+    return res, (A, B)
+
+
+def cpu_baseline(wl, A, B, budget_s=20.0):
+    """The reference's CPU path, y = x @ (kernel * mask) in fp32 (mask_dense,
+    Pruning/BERT/utils/modeling.py:992-1007), timed with NumPy's BLAS on the host cores."""
+    from oracle import tw_oracle
+    M, K, N = wl["M"], wl["K"], wl["N"]
+    mask = tw_oracle.plan_mask(K, N, wl["tiles"]).astype(np.float32)
+    rows = M
+    t0 = time.perf_counter()
+    tw_oracle.mask_dense(A[:min(M, 256)], B, mask)          # warm-up / probe
+    probe = time.perf_counter() - t0
+    if probe * (M / min(M, 256)) * 5 > budget_s:             # bound the sample
+        rows = max(256, int(M * budget_s / (probe * (M / min(M, 256)) * 5)) // 8 * 8)
+    x = np.ascontiguousarray(A[:rows])
+    tw_oracle.mask_dense(x, B, mask)
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < 10 and (len(times) < 3 or time.perf_counter() < t_end):
+        t0 = time.perf_counter()
+        tw_oracle.mask_dense(x, B, mask)
+        times.append(time.perf_counter() - t0)
+    t = float(np.median(times))
+    try:
+        cores = len(os.sched_getaffinity(0))
+    except AttributeError:
+        cores = os.cpu_count()
+    env_threads = os.environ.get("OMP_NUM_THREADS")
+    threads = min(cores, int(env_threads)) if env_threads else cores
+    return dict(value=2.0 * rows * K * N / t / 1e12, unit="TFLOP/s (dense flops, fp32)",
+                cores=threads, kind="port",
+                sample="numpy x @ (kernel*mask), %d of %d rows of the same workload, mask multiply "
+                       "inside the timed region, median of %d runs (%.3f s each)"
+                       % (rows, M, len(times), t))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="vgg16_conv4_2")
+    ap.add_argument("--all", action="store_true", help="also run the other configurations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine and this benchmark use exactly one GPU; "
+              "--gpus %d is not supported (run with --gpus 1)" % args.gpus, file=sys.stderr)
+        return 2
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        return 1
+    from tilesparsity_amd import twgemm as tw
+    tw.lib()  # fails loudly if the HIP library has not been built
+
+    wl = make_workload(args.workload)
+    res, (A, B) = run_workload(wl, args.steps, args.warmup, torch)
+    out = {
+        "metric": "effective TFLOP/s (dense flops / time) at 75% TW sparsity, G=128",
+        "value": res["effective_tflops"], "unit": "TFLOP/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["us_sparse"] * 1e-3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": wl["dtype"], "data": "synthetic",
+        "config": {"workload": "%s M=%d K=%d N=%d G=%d, %d tiles, seed %d" % (
+            wl["name"], wl["M"], wl["K"], wl["N"], wl["G"], len(wl["tiles"]), wl["seed"])},
+        "speedup_vs_dense_plan": res["speedup_vs_dense"],
+        "actual_tflops": res["actual_tflops"], "dense_plan_tflops": res["dense_tflops"],
+        "mfma_utilisation_kept_flops": res["mfma_util_kept"],
+        "mfma_utilisation_dense_run": res["mfma_util_dense_run"],
+        "us_sparse": res["us_sparse"], "us_dense": res["us_dense"],
+        "roofline": {"bound": "hbm", "achieved": res["hbm_gbs"], "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": res["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wl, A, B)
+    del A, B
+    if args.all:
+        others = {}
+        for name in ("bert_base_ffn", "nmt_lstm_gates", "bert_large_ffn1_50", "bert_large_ffn1_75",
+                     "bert_large_ffn1_90", "bert_large_ffn2_50", "bert_large_ffn2_75",
+                     "bert_large_ffn2_90", "imbalance_stress"):
+            r, _ = run_workload(make_workload(name), args.steps, args.warmup, torch)
+            others[name] = {k: r[k] for k in ("us_sparse", "us_dense", "effective_tflops",
+                                              "actual_tflops", "dense_tflops", "speedup_vs_dense",
+                                              "mfma_util_kept", "hbm_gbs", "dtype")}
+            print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
+        out["other_workloads"] = others
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

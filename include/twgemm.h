@@ -1,0 +1,216 @@
+/*
+ * twgemm.h - C ABI of libtwgemm.so, a tile-wise-sparse (TW) GEMM engine for AMD
+ * MI355X (gfx950).
+ *
+ *     C = alpha * A * (B (.) mask) + beta * C
+ *
+ * A[M,K] dense activations, B[K,N] a TW-pruned weight: B is split into column
+ * tiles; every tile keeps its own ascending list of K rows (kept_k) and of
+ * columns (kept_n, relative to the tile's first column).  A *plan* owns the
+ * tile table, the index lists and the compacted weight in device memory; the
+ * caller owns A and C (device memory).
+ *
+ * This boundary replaces the host code of the reference's perf driver,
+ * StreamMaskedGEMM/perf/basic_nn.cu; each entry point names the reference
+ * lines it stands in for.  "Relative offsets" are the reference's mask
+ * arrays: offset[i] = kept[i] - i.
+ *
+ * Conventions
+ *   - every function returns TW_OK (0) or a negative tw_status; nothing throws
+ *     across this boundary; tw_last_error() holds a message for the calling
+ *     thread's last failure.
+ *   - "host" pointers are ordinary memory, "device" pointers are HIP device
+ *     memory of the current device.
+ *   - tw_gemm is asynchronous with respect to `stream` (a hipStream_t passed as
+ *     void*, NULL = the default stream), allocates nothing and never
+ *     synchronises the device.
+ */
+#ifndef TWGEMM_H
+#define TWGEMM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TWGEMM_VERSION 100 /* major*10000 + minor*100 + patch */
+
+typedef struct tw_plan tw_plan;
+
+typedef enum tw_status {
+    TW_OK = 0,
+    TW_ERR_NULL = -1,       /* a required pointer is NULL */
+    TW_ERR_SHAPE = -2,      /* M < 0, K/N/G <= 0, bad leading dimension ... */
+    TW_ERR_TILE_TABLE = -3, /* tiles do not cover [0,N) exactly once, in order */
+    TW_ERR_INDEX_LIST = -4, /* list not strictly ascending or out of range */
+    TW_ERR_DTYPE = -5,      /* unknown element type */
+    TW_ERR_LAYOUT = -6,     /* unknown layout / pruned-column mode */
+    TW_ERR_ALIGNMENT = -7,  /* pointer or leading dimension not 16-byte aligned */
+    TW_ERR_NOT_TW = -8,     /* the 0/1 mask is not a tile-wise pattern for this G */
+    TW_ERR_DEVICE = -9,     /* HIP runtime failure (message has the HIP error) */
+    TW_ERR_ALLOC = -10,     /* host or device allocation failed */
+    TW_ERR_BUFFER = -11     /* caller-provided buffer too small */
+} tw_status;
+
+typedef enum tw_dtype {
+    TW_F16 = 0, /* IEEE half in, fp32 accumulate, half out */
+    TW_BF16 = 1 /* bfloat16 in, fp32 accumulate, bfloat16 out */
+} tw_dtype;
+
+typedef enum tw_layout {
+    /* The reference's layout (basic_nn.cu:418,423-425): A is column-major M x K,
+     * i.e. element (m,k) at A[k*lda + m]; C is column-major M x N, element (m,n)
+     * at C[n*ldc + m].  A gathered K row is one contiguous M-vector. */
+    TW_LAYOUT_KMAJOR = 0,
+    /* Element (m,k) at A[m*lda + k]; element (m,n) at C[m*ldc + n]. */
+    TW_LAYOUT_ROWMAJOR = 1
+} tw_layout;
+
+typedef enum tw_pruned_cols {
+    /* pruned C columns are never written (the reference's scatter epilogue,
+     * cutlass/gemm/mma_epilogue.h:286) */
+    TW_PRUNED_UNTOUCHED = 0,
+    /* pruned C columns receive beta*C (exact zero when beta == 0), which is
+     * what the product with the masked weight yields */
+    TW_PRUNED_ZERO = 1
+} tw_pruned_cols;
+
+/* ---- library ---------------------------------------------------------------- */
+
+int tw_version(void);
+/* Message of the calling thread's most recent failure ("" if none). */
+const char *tw_last_error(void);
+const char *tw_status_string(int status);
+
+/* ---- integer helpers (host) ---------------------------------------------------- */
+
+/* 0/1 keep vector -> relative offsets kept[i]-i; *n_kept receives the count.
+ * offsets must hold n ints.  Replaces convert_mask_to_offset,
+ * Pruning/BERT/utils/MyHook.py:66-74, and the tail of mask_gen,
+ * basic_nn.cu:713-716.  Any mask byte other than 0 or 1 is TW_ERR_INDEX_LIST. */
+int tw_mask_to_offsets(const uint8_t *mask, int n, int32_t *offsets, int *n_kept);
+
+/* Relative offsets -> ascending kept indices (i + offset[i], basic_nn.cu:154).
+ * Fails with TW_ERR_INDEX_LIST unless the result is strictly ascending in
+ * [0, limit). */
+int tw_offsets_to_kept(const int32_t *offsets, int n_kept, int limit, int32_t *kept);
+
+/* Tile partition of TestCutlassGemm, basic_nn.cu:836-885: block_num =
+ * ceil(N_pruned/n_dim) tiles of n_dim kept columns over N/block_num original
+ * columns (the last tile takes the remainders), K_cal = K_pruned everywhere,
+ * off_B = K * sum(N_ori), off_C = M * sum(N_ori).  Arrays must hold max_tiles
+ * entries (TW_ERR_BUFFER otherwise).  The reference's cap of 32 tiles (:74,:837)
+ * does not apply. */
+int tw_tile_partition(int M, int N, int K, int N_pruned, int K_pruned, int n_dim,
+                      int max_tiles, int *block_num, int32_t *N_ori, int32_t *N_cal,
+                      int32_t *K_cal, int64_t *off_B, int64_t *off_C);
+
+/* ---- plans -------------------------------------------------------------------- */
+
+/* Build a plan from an explicit tile table and index lists (all host memory).
+ *   tile_col0[t], tile_width[t]   tiles must cover [0,N) in order, without gaps
+ *   kept_k_ptr[n_tiles+1], kept_k_idx[]   CSR-style lists of kept K rows
+ *   kept_n_ptr[n_tiles+1], kept_n_idx[]   kept columns relative to tile_col0[t]
+ *   B   fp32 row-major [K,N]: the unpruned (or already masked) weight
+ * The weight is compacted and cast on the device (round to nearest even).
+ * Replaces mask_gen + gen_masked_stream_weight + float_to_half,
+ * basic_nn.cu:697-718, 757-769, 122-137, 891-914. */
+int tw_plan_create(int K, int N, int dtype, int n_tiles,
+                   const int32_t *tile_col0, const int32_t *tile_width,
+                   const int32_t *kept_k_ptr, const int32_t *kept_k_idx,
+                   const int32_t *kept_n_ptr, const int32_t *kept_n_idx,
+                   const float *B, tw_plan **out);
+
+/* The 0 %-sparse plan: tiles of G columns, every row and column kept.  Running
+ * tw_gemm on it is the dense baseline of the same kernel (the role of
+ * Cutlass_Gemm_NN, basic_nn.cu:315-375, 1006-1007). */
+int tw_plan_create_dense(int K, int N, int G, int dtype, const float *B, tw_plan **out);
+
+/* Build a plan from a dense 0/1 mask [K,N] (host, row-major, one byte per
+ * element) split every G original columns: the mask -> kept lists -> offsets ->
+ * compaction pre-pass runs as integer HIP kernels.  A row of a tile is kept iff
+ * any of its mask bytes is non-zero, a column likewise; a mask that is not the
+ * outer product of the two per tile is TW_ERR_NOT_TW.  This is the hand-off
+ * from the pruning side (mask-o of mask_dense, Pruning/BERT/utils/modeling.py:1000;
+ * exportPrunedModel, Pruning/BERT/utils/MyHook.py:54-89). */
+int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask,
+                      const float *B, tw_plan **out);
+
+/* Build a plan from the operands of the reference's Stream_Gemm_NN
+ * (basic_nn.cu:378-393): B_stream is the compacted weight in DEVICE memory in
+ * the layout of gen_masked_stream_weight (:757-769; tile t column-major with
+ * ld = K at element off_B[t]), already in `dtype`; mask_n[t] / mask_k[t] are
+ * DEVICE arrays of N_cal[t] / K_cal[t] relative offsets; off_C[t] = M * first
+ * original column of tile t. */
+int tw_plan_from_stream_operands(int M, int N, int K, int dtype, const void *B_stream,
+                                 int block_num, const int32_t *N_cal, const int32_t *K_cal,
+                                 const int32_t *const *mask_n, const int32_t *const *mask_k,
+                                 const int64_t *off_B, const int64_t *off_C, tw_plan **out);
+
+/* info[] receives: 0 K, 1 N, 2 dtype, 3 n_tiles, 4 sum K_t, 5 sum N_t,
+ * 6 sum K_t*N_t (kept weight elements), 7 packed weight bytes on the device,
+ * 8 max K_t, 9 max N_t, 10 number of empty tiles (K_t*N_t == 0),
+ * 11 total width of all tiles (== N).  n_info <= 12 entries are written. */
+int tw_plan_info(const tw_plan *plan, int64_t *info, int n_info);
+
+/* Read a plan back to host memory for bit-exact checks.  Any pointer may be
+ * NULL.  Sizes: tile_col0/tile_width n_tiles; kept_*_ptr n_tiles+1;
+ * kept_k_idx/mask_k_rel sum K_t; kept_n_idx/mask_n_rel sum N_t; B_stream K*N
+ * 16-bit patterns in the layout of gen_masked_stream_weight (basic_nn.cu:757-769)
+ * after the cast of float_to_half (:995), zeros in unused slots. */
+int tw_plan_export(const tw_plan *plan, int32_t *tile_col0, int32_t *tile_width,
+                   int32_t *kept_k_ptr, int32_t *kept_k_idx, int32_t *mask_k_rel,
+                   int32_t *kept_n_ptr, int32_t *kept_n_idx, int32_t *mask_n_rel,
+                   uint16_t *B_stream);
+
+int tw_plan_destroy(tw_plan *plan);
+
+/* ---- the GEMM ------------------------------------------------------------------ */
+
+/* C = alpha * A * (B (.) mask) + beta * C through one persistent grouped kernel.
+ * Replaces Stream_Gemm_NN (basic_nn.cu:378-445) and the masked kernel it launches
+ * per tile (cutlass/gemm/gemm.h:84-100, gemm_mainloop.h:230-338, gathered A load
+ * tile_iterator.h:786-816, column-scatter epilogue mma_epilogue.h:174-290).
+ *   A, C       device pointers of the plan's dtype, 16-byte aligned
+ *   a_layout   TW_LAYOUT_KMAJOR (lda >= M) or TW_LAYOUT_ROWMAJOR (lda >= K)
+ *   c_layout   TW_LAYOUT_KMAJOR (ldc >= M) or TW_LAYOUT_ROWMAJOR (ldc >= N)
+ *   lda, ldc   in elements, multiples of 8
+ *   M          rows of A and C; 0 is a no-op
+ *   beta       C is read only when beta != 0, and only on kept columns
+ *   pruned_cols  tw_pruned_cols
+ * Immutable plan: may be called concurrently from several host threads on
+ * distinct streams (up to 256 launches of one plan in flight at once). */
+int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda,
+            void *C, int c_layout, int64_t ldc, int M, float alpha, float beta,
+            int pruned_cols, void *stream);
+
+/* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument
+ * meaning: A column-major M x K (lda = M), B the compacted stream weight, C
+ * column-major M x N (ldc = M), all DEVICE memory of `dtype`; mask_n/mask_k host
+ * arrays of device pointers to relative offsets.  Builds a transient plan,
+ * runs tw_gemm on `stream`, synchronises that stream and frees the plan. */
+int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A,
+                      const void *B, float beta, void *C, int block_num,
+                      const int32_t *N_cal, const int32_t *K_cal,
+                      const int32_t *const *mask_n, const int32_t *const *mask_k,
+                      const int64_t *off_B, const int64_t *off_C, void *stream);
+
+/* Elementwise fp32 -> dtype cast on the device, round to nearest even
+ * (float_to_half, basic_nn.cu:122-137, without its off-by-one bound). */
+int tw_cast_f32(const float *src, void *dst, int64_t n, int dtype, void *stream);
+
+/* Row gather / scatter of the reference's in-binary oracle, on the device, for
+ * 16-bit elements: dst[i][j] = src[i + mask[i]][j] (deleteRow,
+ * basic_nn.cu:141-157, 196-208) and dst[i + mask[i]][j] = src[i][j] (insertRow,
+ * :178-194, 224-236).  mask is a device array of `rows` relative offsets. */
+int tw_delete_row(const void *matrix, void *matrix_2, int rows, int columns,
+                  const int32_t *mask, void *stream);
+int tw_insert_row(void *matrix, const void *matrix_2, int rows, int columns,
+                  const int32_t *mask, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TWGEMM_H */

@@ -1,0 +1,291 @@
+"""GPU parity of the TW GEMM against the CPU oracle, through the C ABI.
+
+Tolerance (stated by the task): max relative error <= 1e-2 for fp16 and <= 2e-2 for
+bf16, measured as max |C - C_ref| / max(|C_ref|, 1e-2 * rms(C_ref)) against the
+oracle's fp64 dense matmul of the masked weight on the same 16-bit inputs.  Integer
+outcomes (which columns are written, untouched sentinels) are checked bit-exactly.
+"""
+import numpy as np
+import pytest
+
+from tests.helpers import from_device_bits, random_tiles, to_device_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f16": 1e-2, "bf16": 2e-2}
+SENTINEL = 0x1234  # 16-bit pattern pre-filled into C
+
+
+def round_up(v, m):
+    return (v + m - 1) // m * m
+
+
+def run_gemm(tw, oracle, plan, A, dtype, N, alpha=1.0, beta=0.0, C0=None, pruned=0, pad=0):
+    """A: fp32 [M,K] -> device K-major 16-bit; returns (C as fp32 [M,N], raw C bits [N,ldc])."""
+    import torch
+    M, K = A.shape
+    lda = round_up(M, 8) + pad
+    ldc = round_up(M, 8) + pad
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    Cb = np.full((N, ldc), SENTINEL, np.uint16)
+    if C0 is not None:
+        Cb[:, :M] = oracle.cast_bits(C0, dtype).reshape(M, N).T
+    dA = to_device_bits(At, (K, lda))
+    dC = to_device_bits(Cb, (N, ldc))
+    plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
+              pruned_cols=pruned, stream=torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    bits = from_device_bits(dC)
+    return oracle.bits_to_f32(bits[:, :M], dtype).reshape(N, M).T.copy(), bits
+
+
+def reference(oracle, A, B, tiles, dtype, alpha=1.0, beta=0.0, C0=None):
+    Aq, Bq = oracle.quantize(A, dtype), oracle.quantize(B, dtype)
+    Cq = None if C0 is None else oracle.quantize(C0, dtype)
+    return oracle.tw_gemm_reference(Aq, Bq, tiles, alpha, beta, Cq)
+
+
+def kept_columns(tiles, N):
+    keep = np.zeros(N, bool)
+    for t in tiles:
+        keep[np.asarray(t["kept_n"], np.int64) + t["col0"]] = True
+    return keep
+
+
+CASES = [
+    # M,  K,   N,   G,  k_keep n_keep empty
+    (128, 64, 128, 128, 0.5, 1.0, 0),
+    (256, 128, 256, 128, 0.25, 1.0, 0),
+    (100, 96, 200, 128, 0.3, 0.9, 0),     # ragged M, ragged last tile, K_t not multiples of 32
+    (8, 40, 64, 64, 0.5, 0.8, 0),         # tiny M, G = 64 kernel
+    (520, 300, 320, 64, 0.2, 0.8, 3),     # G = 64, empty tiles
+    (333, 257, 384, 128, 0.25, 0.9, 4),   # M not a multiple of 8
+    (1024, 768, 512, 128, 0.25, 1.0, 0),
+    (64, 512, 130, 128, 0.1, 0.5, 0),     # last tile 2 columns wide
+    (257, 64, 96, 32, 0.5, 0.75, 2),      # G = 32
+    (192, 200, 512, 256, 0.3, 0.9, 0),    # tiles wider than one work unit
+]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("case", CASES)
+def test_gemm_matches_oracle(tw, oracle, case, dtype):
+    M, K, N, G, kk, nk, empty = case
+    rng = np.random.default_rng(hash(case) % (2 ** 31))
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=kk, n_keep=nk, empty_every=empty)
+    print("case", case, dtype, flush=True)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        C, bits = run_gemm(tw, oracle, plan, A, dtype, N, pad=8)
+    ref = reference(oracle, A, B, tiles, dtype)
+    keep = kept_columns(tiles, N)
+    err = oracle.rel_error(C[:, keep], ref[:, keep])
+    assert err <= TOL[dtype], err
+    # pruned columns and the padding rows beyond M were never written
+    assert np.all(bits[~keep, :] == SENTINEL)
+    assert np.all(bits[:, M:] == SENTINEL)
+    # the reference's own acceptance rule (basic_nn.cu:771-798, err 1e-2) on the kept part
+    big = np.abs(ref[:, keep]) > 0.05
+    assert oracle.checkout(np.where(big, C[:, keep], 0), np.where(big, ref[:, keep], 0),
+                           err=2e-2 if dtype == "bf16" else 1e-2) == 0
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_alpha_beta_and_zero_mode(tw, oracle, dtype):
+    rng = np.random.default_rng(21)
+    M, K, N, G = 200, 160, 256, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.7)
+    keep = kept_columns(tiles, N)
+    C0q = oracle.quantize(C0, dtype)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        # beta != 0: C read only on kept columns, pruned ones untouched (bit-exact)
+        C, bits = run_gemm(tw, oracle, plan, A, dtype, N, alpha=0.5, beta=-1.5, C0=C0)
+        ref = reference(oracle, A, B, tiles, dtype, 0.5, -1.5, C0)
+        assert oracle.rel_error(C[:, keep], ref[:, keep]) <= TOL[dtype]
+        assert np.array_equal(C[:, ~keep], C0q[:, ~keep])
+        # zero mode, beta == 0: pruned columns become exact zeros
+        C, bits = run_gemm(tw, oracle, plan, A, dtype, N, alpha=2.0, C0=C0, pruned=tw.PRUNED_ZERO)
+        ref = reference(oracle, A, B, tiles, dtype, 2.0)
+        assert oracle.rel_error(C[:, keep], ref[:, keep]) <= TOL[dtype]
+        assert np.all(bits[~keep, :M] == 0)
+        assert np.all(bits[:, M:] == SENTINEL)
+        # zero mode with beta: pruned columns receive beta * C, the full product's value
+        C, _ = run_gemm(tw, oracle, plan, A, dtype, N, alpha=1.0, beta=0.5, C0=C0,
+                        pruned=tw.PRUNED_ZERO)
+        full = oracle.quantize(A, dtype).astype(np.float64) @ oracle.masked_dense_weight(
+            oracle.quantize(B, dtype), tiles).astype(np.float64) + 0.5 * C0q
+        assert oracle.rel_error(C, full) <= TOL[dtype]
+
+
+def test_gemm_degenerate_plans(tw, oracle):
+    rng = np.random.default_rng(22)
+    M, K, N, G = 96, 64, 256, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    e = np.zeros(0, np.int32)
+    # tile 0 keeps columns but no K row -> zeros there; tile 1 keeps no column -> untouched
+    tiles = [dict(col0=0, width=128, kept_k=e, kept_n=np.arange(0, 128, 3, dtype=np.int32)),
+             dict(col0=128, width=128, kept_k=np.arange(K, dtype=np.int32), kept_n=e)]
+    with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+        assert plan.info()["empty_tiles"] == 2
+        C, bits = run_gemm(tw, oracle, plan, A, "f16", N)
+        keep = kept_columns(tiles, N)
+        assert np.all(bits[keep, :M] == 0) and np.all(bits[~keep, :] == SENTINEL)
+        # M == 0 is a no-op
+        plan.gemm(0, 0, 0)
+    # identity weight: C is the gathered A columns, exactly
+    K = N = 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    kk = np.sort(rng.choice(K, 37, replace=False)).astype(np.int32)
+    one = [dict(col0=0, width=N, kept_k=kk, kept_n=np.arange(N, dtype=np.int32))]
+    with tw.Plan.create(K, N, "f16", one, np.eye(K, dtype=np.float32)) as plan:
+        C, _ = run_gemm(tw, oracle, plan, A, "f16", N)
+    expect = np.zeros((M, N), np.float32)
+    expect[:, kk] = oracle.quantize(A, "f16")[:, kk]
+    assert np.array_equal(C, expect)
+
+
+def test_dense_plan_equals_plain_gemm(tw, oracle):
+    import torch
+    rng = np.random.default_rng(23)
+    M, K, N, G = 512, 384, 640, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    with tw.Plan.dense(K, N, G, "f16", B) as plan:
+        C, _ = run_gemm(tw, oracle, plan, A, "f16", N)
+    Aq, Bq = oracle.quantize(A, "f16"), oracle.quantize(B, "f16")
+    assert oracle.rel_error(C, Aq.astype(np.float64) @ Bq.astype(np.float64)) <= TOL["f16"]
+    # a library routine on the same inputs (hipBLASLt/rocBLAS through torch)
+    lib = (torch.from_numpy(Aq).cuda().half() @ torch.from_numpy(Bq).cuda().half()).float().cpu().numpy()
+    assert oracle.rel_error(C, lib) <= TOL["f16"]
+
+
+def test_fused_equals_gather_dense_scatter_bitwise(tw, oracle):
+    """The reference's first self-check (basic_nn.cu:1081, tolerance 1e-10 = exact): the
+    fused masked GEMM equals gather rows -> dense GEMM on the compact tile -> scatter,
+    run through the engine's own kernel and its deleteRow / insertRow kernels."""
+    import torch
+    rng = np.random.default_rng(24)
+    M, K, N, G, dtype = 264, 320, 384, 128, "f16"
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.3, n_keep=0.8)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        _, fused = run_gemm(tw, oracle, plan, A, dtype, N)
+    At = oracle.cast_bits(A, dtype).reshape(M, K).T.copy()
+    dA = to_device_bits(At, (K, M))
+    out = np.full((N, M), SENTINEL, np.uint16)
+    for t in tiles:
+        kt, nt = len(t["kept_k"]), len(t["kept_n"])
+        rel_k = torch.from_numpy(t["kept_k"] - np.arange(kt, dtype=np.int32)).cuda()
+        rel_n = torch.from_numpy(t["kept_n"] - np.arange(nt, dtype=np.int32)).cuda()
+        dA2 = torch.zeros((kt, M), dtype=torch.int16, device="cuda")
+        tw.delete_row(dA.data_ptr(), dA2.data_ptr(), kt, M, rel_k.data_ptr())
+        comp = B[np.ix_(t["kept_k"], t["kept_n"] + t["col0"])]
+        dC2 = torch.zeros((nt, M), dtype=torch.int16, device="cuda")
+        with tw.Plan.dense(kt, nt, max(nt, 1), dtype, comp) as dense:
+            dense.gemm(dA2.data_ptr(), dC2.data_ptr(), M)
+            torch.cuda.synchronize()
+        dCt = to_device_bits(out[t["col0"]:t["col0"] + t["width"]], (t["width"], M))
+        tw.insert_row(dCt.data_ptr(), dC2.data_ptr(), nt, M, rel_n.data_ptr())
+        torch.cuda.synchronize()
+        out[t["col0"]:t["col0"] + t["width"]] = from_device_bits(dCt)
+    assert np.array_equal(fused[:, :M], out)
+
+
+def test_tile_order_does_not_change_a_bit(tw, oracle):
+    """Work-queue order must not matter: the same tiles with kept-K counts arranged so
+    that the queue sorts them differently give bit-identical columns."""
+    rng = np.random.default_rng(25)
+    M, K, N, G, dtype = 300, 256, 512, 128, "f16"
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.3, n_keep=0.9)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        _, base = run_gemm(tw, oracle, plan, A, dtype, N)
+    # reverse the column-tile order of the weight (and of the plan): each tile's columns
+    # must come out identical, at their new position
+    perm = list(reversed(range(len(tiles))))
+    B2 = np.concatenate([B[:, tiles[i]["col0"]:tiles[i]["col0"] + G] for i in perm], axis=1)
+    tiles2 = [dict(col0=j * G, width=G, kept_k=tiles[i]["kept_k"], kept_n=tiles[i]["kept_n"])
+              for j, i in enumerate(perm)]
+    with tw.Plan.create(K, N, dtype, tiles2, B2) as plan:
+        _, moved = run_gemm(tw, oracle, plan, A, dtype, N)
+    for j, i in enumerate(perm):
+        assert np.array_equal(moved[j * G:(j + 1) * G], base[i * G:(i + 1) * G])
+
+
+def test_repeated_launches_and_slot_reuse(tw, oracle):
+    """More launches than ticket slots on one plan: every launch must see a re-armed queue."""
+    import torch
+    rng = np.random.default_rng(26)
+    M, K, N, G, dtype = 136, 96, 256, 128, "f16"
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.5, n_keep=0.9)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        _, first = run_gemm(tw, oracle, plan, A, dtype, N)
+        At = oracle.cast_bits(A, dtype).reshape(M, K).T.copy()
+        dA = to_device_bits(At, (K, M))
+        dC = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+        for _ in range(600):
+            plan.gemm(dA.data_ptr(), dC.data_ptr(), M,
+                      stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        keep = kept_columns(tiles, N)
+        assert np.array_equal(from_device_bits(dC)[keep], first[keep, :M])
+
+
+def test_gemm_argument_errors(tw):
+    import torch
+    K, N, M = 64, 128, 64
+    with tw.Plan.dense(K, N, 128, "f16", np.zeros((K, N), np.float32)) as plan:
+        a = torch.zeros((K, M), dtype=torch.int16, device="cuda")
+        c = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+        for kwargs, status in ((dict(lda=M - 8), tw.ERR_SHAPE), (dict(ldc=M + 4), tw.ERR_ALIGNMENT),
+                               (dict(a_layout=5), tw.ERR_LAYOUT), (dict(pruned_cols=3), tw.ERR_LAYOUT)):
+            with pytest.raises(tw.TwError) as e:
+                plan.gemm(a.data_ptr(), c.data_ptr(), M, **kwargs)
+            assert e.value.status == status
+        with pytest.raises(tw.TwError) as e:
+            plan.gemm(a.data_ptr() + 2, c.data_ptr(), M)
+        assert e.value.status == tw.ERR_ALIGNMENT
+        with pytest.raises(tw.TwError) as e:
+            plan.gemm(0, c.data_ptr(), M)
+        assert e.value.status == tw.ERR_NULL
+        with pytest.raises(tw.TwError) as e:
+            plan.gemm(a.data_ptr(), c.data_ptr(), -1)
+        assert e.value.status == tw.ERR_SHAPE
+
+
+def test_stream_gemm_nn_drop_in(tw, oracle):
+    """The reference's own problem (`test_basic_nn 64 768 256 384 128`, its rand() stream)
+    driven through the Stream_Gemm_NN-shaped entry point with the reference's operands."""
+    import torch
+    M, N, K, Np, Kp = 64, 768, 256, 384, 128
+    A, B, tiles, part = oracle.ref_compat_problem(M, N, K, Np, Kp)
+    dtype = "f16"
+    dA = to_device_bits(oracle.cast_bits(A, dtype).reshape(M, K).T.copy(), (K, M))
+    dB = to_device_bits(oracle.cast_bits(oracle.stream_weight(B, tiles), dtype), (K * N,))
+    dC = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+    mk = [torch.from_numpy(t["mask_k"]).cuda() for t in tiles]
+    mn = [torch.from_numpy(t["mask_n"]).cuda() for t in tiles]
+    tw.stream_gemm_nn(M, N, K, dtype, 1.0, dA.data_ptr(), dB.data_ptr(), 0.0, dC.data_ptr(),
+                      part["N_cal"], part["K_cal"], [x.data_ptr() for x in mn],
+                      [x.data_ptr() for x in mk], part["off_B"], part["off_C"])
+    C = oracle.bits_to_f32(from_device_bits(dC), dtype).reshape(N, M).T
+    ref = reference(oracle, A, B, tiles, dtype)
+    assert oracle.rel_error(C, ref) <= TOL[dtype]
+    # and a plan built from those operands exports the same lists and weight bits
+    with tw.Plan.from_stream_operands(M, N, K, dtype, dB.data_ptr(), part["N_cal"], part["K_cal"],
+                                      [x.data_ptr() for x in mn], [x.data_ptr() for x in mk],
+                                      part["off_B"], part["off_C"]) as plan:
+        got, Bs = plan.export()
+        for g, t in zip(got, tiles):
+            assert np.array_equal(g["kept_k"], t["kept_k"]) and np.array_equal(g["mask_n"], t["mask_n"])
+        assert np.array_equal(Bs, from_device_bits(dB))

@@ -1,0 +1,112 @@
+"""GPU parity of the integer pre-pass (mask -> kept lists -> relative offsets ->
+compaction) and of the small boundary kernels, bit-exact against the oracle."""
+import numpy as np
+import pytest
+
+from tests.helpers import from_device_bits, random_tiles, to_device_bits
+
+pytestmark = pytest.mark.gpu
+
+
+def check_export(oracle, plan, tiles, B, dtype):
+    got, Bs = plan.export()
+    assert len(got) == len(tiles)
+    for g, t in zip(got, tiles):
+        assert g["col0"] == t["col0"] and g["width"] == t["width"]
+        assert np.array_equal(g["kept_k"], t["kept_k"])
+        assert np.array_equal(g["kept_n"], t["kept_n"])
+        # relative offsets: kept[i] - i, and the oracle's mask -> offsets routine
+        assert np.array_equal(g["mask_k"], t["kept_k"] - np.arange(len(t["kept_k"])))
+        assert np.array_equal(g["mask_n"], t["kept_n"] - np.arange(len(t["kept_n"])))
+    K, N = B.shape
+    assert np.array_equal(g["mask_k"], oracle.mask_to_offsets(
+        np.isin(np.arange(K), tiles[-1]["kept_k"]).astype(np.uint8)))
+    # compacted weight, reference stream layout, after the 16-bit cast: bit-exact
+    expect = oracle.cast_bits(oracle.stream_weight(B, tiles), dtype)
+    assert np.array_equal(Bs, expect)
+
+
+@pytest.mark.parametrize("K,N,G,dtype", [(64, 128, 32, "f16"), (100, 200, 64, "bf16"),
+                                         (257, 300, 128, "f16"), (768, 512, 128, "bf16"),
+                                         (33, 40, 64, "f16")])
+def test_plan_create_compaction_bit_exact(tw, oracle, K, N, G, dtype):
+    rng = np.random.default_rng(K * 1000 + N)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.3, n_keep=0.8, empty_every=4)
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        check_export(oracle, plan, tiles, B, dtype)
+        inf = plan.info()
+        assert inf["sum_k"] == sum(len(t["kept_k"]) for t in tiles)
+        assert inf["kept_elems"] == sum(len(t["kept_k"]) * len(t["kept_n"]) for t in tiles)
+        assert inf["total_width"] == N
+
+
+@pytest.mark.parametrize("K,N,G,dtype", [(64, 128, 32, "f16"), (300, 520, 128, "bf16"),
+                                         (1000, 77, 64, "f16"), (768, 3072, 128, "f16")])
+def test_plan_from_mask_bit_exact(tw, oracle, K, N, G, dtype):
+    rng = np.random.default_rng(K + N)
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.25, n_keep=0.9, empty_every=5)
+    mask = oracle.plan_mask(K, N, tiles)
+    expect = oracle.plan_from_mask(mask, G)   # empty tiles lose their lists, as a mask cannot hold them
+    with tw.Plan.from_mask(mask, G, dtype, B) as plan:
+        check_export(oracle, plan, expect, B, dtype)
+
+
+def test_plan_from_mask_rejects_non_tw_mask(tw):
+    K, N, G = 64, 128, 32
+    mask = np.zeros((K, N), np.uint8)
+    mask[::2, :16] = 1
+    mask[5, 3] = 1          # an element outside the (rows x columns) product
+    mask[0, 1] = 0          # and a hole inside it
+    with pytest.raises(tw.TwError) as e:
+        tw.Plan.from_mask(mask, G, "f16", np.zeros((K, N), np.float32))
+    assert e.value.status == tw.ERR_NOT_TW
+    mask[5, 3] = 0
+    mask[0, 1] = 1
+    tw.Plan.from_mask(mask, G, "f16", np.zeros((K, N), np.float32)).destroy()
+
+
+def test_dense_plan(tw, oracle):
+    K, N, G = 96, 200, 64
+    B = np.random.default_rng(9).standard_normal((K, N)).astype(np.float32)
+    with tw.Plan.dense(K, N, G, "f16", B) as plan:
+        tiles, Bs = plan.export()
+        assert [t["width"] for t in tiles] == [64, 64, 64, 8]
+        assert all(len(t["kept_k"]) == K and len(t["kept_n"]) == t["width"] for t in tiles)
+        # all kept: the stream layout is simply B transposed
+        assert np.array_equal(Bs.reshape(N, K), oracle.cast_bits(B.T, "f16").reshape(N, K))
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_cast_kernel_bit_exact(tw, oracle, dtype):
+    import torch
+    rng = np.random.default_rng(11)
+    x = (rng.standard_normal(100003) * 10.0 ** rng.integers(-8, 6, 100003)).astype(np.float32)
+    x[:8] = [0.0, -0.0, np.inf, -np.inf, 65504.0, 65520.0, 1e-8, 3e-5]
+    src = torch.from_numpy(x).cuda()
+    dst = torch.full((x.size + 1,), 0x5555, dtype=torch.int16, device="cuda")
+    tw.cast_f32(src.data_ptr(), dst.data_ptr(), x.size, dtype)
+    torch.cuda.synchronize()
+    got = from_device_bits(dst)
+    assert np.array_equal(got[:-1], oracle.cast_bits(x, dtype))
+    assert got[-1] == 0x5555    # no write past the end (the reference's bound is off by one)
+
+
+def test_delete_insert_row_kernels(tw):
+    import torch
+    rng = np.random.default_rng(12)
+    rows, cols = 300, 77
+    src = rng.integers(0, 65536, (rows, cols)).astype(np.uint16)
+    kept = np.sort(rng.choice(rows, 120, replace=False)).astype(np.int32)
+    rel = torch.from_numpy(kept - np.arange(120, dtype=np.int32)).cuda()
+    d_src = to_device_bits(src, (rows, cols))
+    d_out = torch.zeros((120, cols), dtype=torch.int16, device="cuda")
+    tw.delete_row(d_src.data_ptr(), d_out.data_ptr(), 120, cols, rel.data_ptr())
+    d_back = torch.zeros((rows, cols), dtype=torch.int16, device="cuda")
+    tw.insert_row(d_back.data_ptr(), d_out.data_ptr(), 120, cols, rel.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(from_device_bits(d_out), src[kept])
+    expect = np.zeros_like(src)
+    expect[kept] = src[kept]
+    assert np.array_equal(from_device_bits(d_back), expect)

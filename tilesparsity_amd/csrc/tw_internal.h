@@ -1,0 +1,116 @@
+// Internal declarations shared by the host code and the HIP kernels of libtwgemm.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <string>
+#include <vector>
+
+#include "twgemm.h"
+
+namespace tw {
+
+// Geometry shared by the pack kernel and the GEMM kernels.
+constexpr int kMfmaN = 32;    // columns of one MFMA block (packing granularity in n)
+constexpr int kMfmaK = 16;    // k extent of one v_mfma_f32_32x32x16
+constexpr int kBlockK = 32;   // k rows staged per main-loop step; K_t is padded to this
+constexpr int kMaxUnitN = 128; // compact columns handled by one work item
+constexpr int kTicketSlots = 256;
+
+// One schedulable piece of a tile: at most kMaxUnitN compact columns.
+// 48 bytes; read with scalar loads.
+struct UnitDev {
+    int32_t col0;     // first original column of the tile in C
+    int32_t k_kept;   // K_t
+    int32_t k_pad;    // K_t rounded up to kBlockK
+    int32_t n_cnt;    // compact columns in this unit
+    int32_t nb0;      // first 32-column block of the tile's packed weight used here
+    int32_t nb_cnt;   // 32-column blocks in this unit
+    int32_t kk_off;   // offset of the tile's kept_k list
+    int32_t kn_off;   // offset of this unit's first compact column in kept_n
+    int64_t b_off;    // element offset of the tile's packed weight
+    int32_t tile;     // owning tile
+    int32_t pad_;
+};
+
+// Zero-fill work for TW_PRUNED_ZERO: the pruned columns of one tile.
+struct TileDev {
+    int32_t col0;
+    int32_t n_pruned; // pruned original columns in the tile
+    int32_t pn_off;   // offset into pruned_n
+    int32_t pad_;
+};
+
+struct GemmArgs {
+    const UnitDev *units;   // sorted by k_kept descending
+    const TileDev *tiles;
+    const int32_t *kept_k;
+    const int32_t *kept_n;
+    const int32_t *pruned_n;
+    const void *Bp;
+    const void *A;
+    void *C;
+    int64_t lda, ldc;
+    int32_t M;
+    int32_t n_mblk;       // ceil(M / BM)
+    int32_t n_gemm_items; // n_units * n_mblk
+    int32_t n_items;      // + n_zero_tiles * n_mblk when zero-filling
+    int32_t n_zero_tiles; // tiles with pruned columns (first entries of `tiles`)
+    float alpha, beta;
+    int32_t *ticket;      // [0] next item, [1] finished workgroups
+};
+
+} // namespace tw
+
+struct tw_plan {
+    int K = 0, N = 0, dtype = 0, n_tiles = 0;
+    int device = 0;
+    // host copies
+    std::vector<int32_t> tile_col0, tile_width, kept_k_ptr, kept_k_idx, kept_n_ptr, kept_n_idx;
+    std::vector<int32_t> k_pad, n_pad;
+    std::vector<int64_t> b_off; // element offset of each tile's packed weight
+    int64_t packed_elems = 0;
+    int n_units = 0, n_zero_tiles = 0, max_unit_n = 0;
+    // device
+    int32_t *d_kept_k = nullptr, *d_kept_n = nullptr, *d_rel_k = nullptr, *d_rel_n = nullptr;
+    int32_t *d_pruned_n = nullptr;
+    tw::UnitDev *d_units = nullptr;
+    tw::TileDev *d_tiles = nullptr;
+    void *d_Bp = nullptr;
+    int32_t *d_tickets = nullptr; // kTicketSlots pairs
+    mutable unsigned next_slot = 0;
+    int cu_count = 0;
+};
+
+namespace tw {
+
+void set_error(const char *fmt, ...);
+int fail(int status, const char *fmt, ...);
+
+#define TW_HIP(call)                                                                     \
+    do {                                                                                 \
+        hipError_t e_ = (call);                                                          \
+        if (e_ != hipSuccess)                                                            \
+            return ::tw::fail(TW_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(e_)); \
+    } while (0)
+
+// validation shared by the plan builders (host only)
+int validate_lists(int K, int N, int n_tiles, const int32_t *tile_col0, const int32_t *tile_width,
+                   const int32_t *kept_k_ptr, const int32_t *kept_k_idx,
+                   const int32_t *kept_n_ptr, const int32_t *kept_n_idx);
+
+// fills the host-side geometry (k_pad, n_pad, b_off, packed_elems) of a plan whose
+// lists are set, uploads lists/units/tiles and allocates the packed weight (zeroed).
+int finalize_plan_geometry(tw_plan *p);
+
+// device pack: packed weight from a row-major fp32 [K,N] device buffer
+int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s);
+// device pack: packed weight from the reference's compacted stream layout (16-bit, device)
+int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStream_t s);
+// device unpack: compacted stream layout (K*N 16-bit, zero elsewhere) from the packed weight
+int unpack_to_stream(const tw_plan *p, uint16_t *d_Bs, hipStream_t s);
+
+} // namespace tw

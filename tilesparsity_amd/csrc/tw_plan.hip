@@ -1,0 +1,863 @@
+// Plan construction for libtwgemm: the integer mask -> kept lists -> relative
+// offsets -> compaction pre-pass (HIP kernels), the MFMA-ordered weight packing,
+// and the read-back used for bit-exact checks.
+//
+// Packed weight of tile t (K_t x N_t compact, padded to k_pad x n_pad):
+//   for 32-column block nb, 16-row step k16, lane l (0..63), e (0..7):
+//     Bp[b_off + ((nb * (k_pad/16) + k16) * 64 + l) * 8 + e]
+//        = compact[k16*16 + (l/32)*8 + e][nb*32 + l%32]      (0 outside K_t x N_t)
+// i.e. each wave fetches one MFMA B operand with a single 16-byte load per lane,
+// 1 KiB contiguous per wave.
+#include "tw_internal.h"
+
+#include <algorithm>
+#include <cstring>
+#include <mutex>
+
+namespace tw {
+
+struct PackTile {
+    int32_t col0, k_kept, n_kept, k_pad, n_pad, kk_off, kn_off, pad_;
+    int64_t b_off;
+    int64_t src_off; // stream layout only: element offset of the tile in B_stream
+};
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f)
+{
+    uint32_t x = __float_as_uint(f);
+    if ((x & 0x7F800000u) == 0x7F800000u && (x & 0x007FFFFFu))
+        return (uint16_t)((x >> 16) | 0x0040u);
+    x += 0x7FFFu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+}
+
+__device__ __forceinline__ uint16_t f32_to_f16_rne(float f)
+{
+    _Float16 h = (_Float16)f; // v_cvt_f16_f32, round to nearest even
+    return __builtin_bit_cast(uint16_t, h);
+}
+
+__device__ __forceinline__ uint16_t cast16(float f, int dtype)
+{
+    return dtype == TW_BF16 ? f32_to_bf16_rne(f) : f32_to_f16_rne(f);
+}
+
+// ---------------------------------------------------------------------------------
+// packing
+
+__global__ void pack_dense_kernel(const PackTile *tiles, const int32_t *kept_k,
+                                  const int32_t *kept_n, const float *B, int N, int dtype,
+                                  uint16_t *Bp)
+{
+    const PackTile t = tiles[blockIdx.y];
+    const int64_t groups = (int64_t)t.k_pad * t.n_pad / 8;
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= groups)
+        return;
+    const int lane = (int)(g & 63);
+    const int64_t blk = g >> 6;
+    const int ksteps = t.k_pad / kMfmaK;
+    const int k16 = (int)(blk % ksteps);
+    const int nb = (int)(blk / ksteps);
+    const int n = nb * kMfmaN + (lane & 31);
+    const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
+    uint16_t v[8];
+    int col = -1;
+    if (n < t.n_kept)
+        col = t.col0 + kept_n[t.kn_off + n];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int kk = kk0 + e;
+        float f = 0.0f;
+        if (col >= 0 && kk < t.k_kept)
+            f = B[(int64_t)kept_k[t.kk_off + kk] * N + col];
+        v[e] = cast16(f, dtype);
+    }
+    uint4 out;
+    out.x = v[0] | ((uint32_t)v[1] << 16);
+    out.y = v[2] | ((uint32_t)v[3] << 16);
+    out.z = v[4] | ((uint32_t)v[5] << 16);
+    out.w = v[6] | ((uint32_t)v[7] << 16);
+    *reinterpret_cast<uint4 *>(Bp + t.b_off + g * 8) = out;
+}
+
+// Source is the reference's compacted layout: tile column j, row i at
+// Bs[src_off + j*K + i] (gen_masked_stream_weight, basic_nn.cu:765).
+__global__ void pack_stream_kernel(const PackTile *tiles, const uint16_t *Bs, int K, uint16_t *Bp)
+{
+    const PackTile t = tiles[blockIdx.y];
+    const int64_t groups = (int64_t)t.k_pad * t.n_pad / 8;
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= groups)
+        return;
+    const int lane = (int)(g & 63);
+    const int64_t blk = g >> 6;
+    const int ksteps = t.k_pad / kMfmaK;
+    const int k16 = (int)(blk % ksteps);
+    const int nb = (int)(blk / ksteps);
+    const int n = nb * kMfmaN + (lane & 31);
+    const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
+    uint16_t v[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int kk = kk0 + e;
+        v[e] = (n < t.n_kept && kk < t.k_kept) ? Bs[t.src_off + (int64_t)n * K + kk] : (uint16_t)0;
+    }
+    uint4 out;
+    out.x = v[0] | ((uint32_t)v[1] << 16);
+    out.y = v[2] | ((uint32_t)v[3] << 16);
+    out.z = v[4] | ((uint32_t)v[5] << 16);
+    out.w = v[6] | ((uint32_t)v[7] << 16);
+    *reinterpret_cast<uint4 *>(Bp + t.b_off + g * 8) = out;
+}
+
+// Inverse of the packing into the reference's compacted layout at K*col0.
+__global__ void unpack_stream_kernel(const PackTile *tiles, const uint16_t *Bp, int K, uint16_t *Bs)
+{
+    const PackTile t = tiles[blockIdx.y];
+    const int64_t groups = (int64_t)t.k_pad * t.n_pad / 8;
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= groups)
+        return;
+    const int lane = (int)(g & 63);
+    const int64_t blk = g >> 6;
+    const int ksteps = t.k_pad / kMfmaK;
+    const int k16 = (int)(blk % ksteps);
+    const int nb = (int)(blk / ksteps);
+    const int n = nb * kMfmaN + (lane & 31);
+    const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
+    if (n >= t.n_kept)
+        return;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int kk = kk0 + e;
+        if (kk < t.k_kept)
+            Bs[(int64_t)(t.col0 + n) * K + kk] = Bp[t.b_off + g * 8 + e];
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// mask -> flags -> lists  (integer pre-pass)
+
+// rowflag[t*K + k] = any byte of mask[k][t*G .. t*G+w) is non-zero
+__global__ void row_flags_kernel(const uint8_t *mask, int K, int N, int G, int n_tiles,
+                                 uint8_t *rowflag)
+{
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)K * n_tiles)
+        return;
+    const int t = (int)(idx % n_tiles);
+    const int k = (int)(idx / n_tiles);
+    const int c0 = t * G;
+    const int w = min(G, N - c0);
+    const uint8_t *row = mask + (int64_t)k * N + c0;
+    uint32_t any = 0;
+    for (int j = 0; j < w; ++j)
+        any |= row[j];
+    rowflag[(int64_t)t * K + k] = any ? 1 : 0;
+}
+
+// colflag[c] |= any of mask[k][c] over a 64-row slab (colflag holds 32-bit words)
+__global__ void col_flags_kernel(const uint8_t *mask, int K, int N, uint32_t *colflag)
+{
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= N)
+        return;
+    const int k0 = blockIdx.y * 64;
+    const int k1 = min(K, k0 + 64);
+    uint32_t any = 0;
+    for (int k = k0; k < k1; ++k)
+        any |= mask[(int64_t)k * N + c];
+    if (any)
+        atomicOr(&colflag[c], 1u);
+}
+
+// counts the elements where mask != rowflag & colflag (a TW mask has none)
+__global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, int G,
+                                   const uint8_t *rowflag, const uint32_t *colflag,
+                                   unsigned long long *mismatch)
+{
+    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (int64_t)K * N)
+        return;
+    const int c = (int)(idx % N);
+    const int k = (int)(idx / N);
+    const int t = c / G;
+    const bool m = mask[idx] != 0;
+    const bool e = rowflag[(int64_t)t * K + k] && colflag[c];
+    if (m != e)
+        atomicAdd(mismatch, 1ull);
+}
+
+// counts[t] = kept rows of tile t, counts[n_tiles + t] = kept columns of tile t
+__global__ void count_flags_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K, int N,
+                                   int G, int n_tiles, int32_t *counts)
+{
+    __shared__ int s_sum[2];
+    const int t = blockIdx.x;
+    if (threadIdx.x == 0) {
+        s_sum[0] = 0;
+        s_sum[1] = 0;
+    }
+    __syncthreads();
+    int rk = 0, ck = 0;
+    for (int k = threadIdx.x; k < K; k += blockDim.x)
+        rk += rowflag[(int64_t)t * K + k];
+    const int c0 = t * G, w = min(G, N - c0);
+    for (int j = threadIdx.x; j < w; j += blockDim.x)
+        ck += colflag[c0 + j] ? 1 : 0;
+    atomicAdd(&s_sum[0], rk);
+    atomicAdd(&s_sum[1], ck);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        counts[t] = s_sum[0];
+        counts[n_tiles + t] = s_sum[1];
+    }
+}
+
+// Ordered compaction of one flag vector by one 256-thread block: writes the
+// ascending kept indices and the relative offsets kept[i] - i.
+__device__ void block_compact(const uint8_t *flag8, const uint32_t *flag32, int n, int32_t *kept,
+                              int32_t *rel)
+{
+    __shared__ int s_wave[4];
+    __shared__ int s_base;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    if (threadIdx.x == 0)
+        s_base = 0;
+    __syncthreads();
+    for (int i0 = 0; i0 < n; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        bool f = false;
+        if (i < n)
+            f = flag8 ? flag8[i] != 0 : flag32[i] != 0;
+        const unsigned long long b = __ballot(f);
+        const int before = __popcll(b & ((1ull << lane) - 1ull));
+        if (lane == 0)
+            s_wave[wave] = __popcll(b);
+        __syncthreads();
+        int off = s_base;
+        for (int w = 0; w < wave; ++w)
+            off += s_wave[w];
+        if (f) {
+            kept[off + before] = i;
+            rel[off + before] = i - (off + before);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0)
+            s_base += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+        __syncthreads();
+    }
+}
+
+// grid (n_tiles, 2): y == 0 rows, y == 1 columns
+__global__ void __launch_bounds__(256)
+    compact_lists_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K, int N, int G,
+                         const int32_t *k_ptr, const int32_t *n_ptr, int32_t *kept_k,
+                         int32_t *rel_k, int32_t *kept_n, int32_t *rel_n)
+{
+    const int t = blockIdx.x;
+    if (blockIdx.y == 0) {
+        block_compact(rowflag + (int64_t)t * K, nullptr, K, kept_k + k_ptr[t], rel_k + k_ptr[t]);
+    } else {
+        const int c0 = t * G, w = min(G, N - c0);
+        block_compact(nullptr, colflag + c0, w, kept_n + n_ptr[t], rel_n + n_ptr[t]);
+    }
+}
+
+// ---------------------------------------------------------------------------------
+
+static int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+static std::vector<PackTile> pack_tiles(const tw_plan *p, const int64_t *src_off)
+{
+    std::vector<PackTile> v(p->n_tiles);
+    for (int t = 0; t < p->n_tiles; ++t) {
+        PackTile &q = v[t];
+        q.col0 = p->tile_col0[t];
+        q.k_kept = p->kept_k_ptr[t + 1] - p->kept_k_ptr[t];
+        q.n_kept = p->kept_n_ptr[t + 1] - p->kept_n_ptr[t];
+        q.k_pad = p->k_pad[t];
+        q.n_pad = p->n_pad[t];
+        q.kk_off = p->kept_k_ptr[t];
+        q.kn_off = p->kept_n_ptr[t];
+        q.pad_ = 0;
+        q.b_off = p->b_off[t];
+        q.src_off = src_off ? src_off[t] : 0;
+    }
+    return v;
+}
+
+static int64_t max_groups(const tw_plan *p)
+{
+    int64_t g = 0;
+    for (int t = 0; t < p->n_tiles; ++t)
+        g = std::max<int64_t>(g, (int64_t)p->k_pad[t] * p->n_pad[t] / 8);
+    return g;
+}
+
+template <typename T> static int upload(T **dst, const std::vector<T> &src)
+{
+    *dst = nullptr;
+    size_t bytes = std::max<size_t>(src.size(), 1) * sizeof(T);
+    if (hipMalloc((void **)dst, bytes) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes failed", bytes);
+    if (!src.empty())
+        TW_HIP(hipMemcpy(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice));
+    return TW_OK;
+}
+
+int finalize_plan_geometry(tw_plan *p)
+{
+    const int nt = p->n_tiles;
+    p->k_pad.assign(nt, 0);
+    p->n_pad.assign(nt, 0);
+    p->b_off.assign(nt, 0);
+    int64_t off = 0;
+    std::vector<UnitDev> units;
+    std::vector<TileDev> ztiles;
+    std::vector<int32_t> pruned_n;
+    p->max_unit_n = 0;
+    for (int t = 0; t < nt; ++t) {
+        const int kt = p->kept_k_ptr[t + 1] - p->kept_k_ptr[t];
+        const int ntk = p->kept_n_ptr[t + 1] - p->kept_n_ptr[t];
+        p->k_pad[t] = ntk > 0 ? round_up(kt, kBlockK) : 0;
+        p->n_pad[t] = kt > 0 ? round_up(ntk, kMfmaN) : 0;
+        if (p->k_pad[t] == 0 || p->n_pad[t] == 0) {
+            // nothing to multiply; kept columns (if any) still receive alpha*0 + beta*C
+            p->k_pad[t] = 0;
+            p->n_pad[t] = ntk > 0 ? round_up(ntk, kMfmaN) : 0;
+        }
+        p->b_off[t] = off;
+        off += (int64_t)p->k_pad[t] * p->n_pad[t];
+        off = (off + 511) / 512 * 512; // keep every tile 1 KiB aligned
+        for (int nc0 = 0; nc0 < ntk; nc0 += kMaxUnitN) {
+            UnitDev u;
+            u.col0 = p->tile_col0[t];
+            u.k_kept = kt;
+            u.k_pad = p->k_pad[t];
+            u.n_cnt = std::min(kMaxUnitN, ntk - nc0);
+            u.nb0 = nc0 / kMfmaN;
+            u.nb_cnt = (u.n_cnt + kMfmaN - 1) / kMfmaN;
+            u.kk_off = p->kept_k_ptr[t];
+            u.kn_off = p->kept_n_ptr[t] + nc0;
+            u.b_off = p->b_off[t];
+            u.tile = t;
+            u.pad_ = 0;
+            units.push_back(u);
+            p->max_unit_n = std::max(p->max_unit_n, u.n_cnt);
+        }
+        if (ntk < p->tile_width[t]) {
+            TileDev z;
+            z.col0 = p->tile_col0[t];
+            z.n_pruned = p->tile_width[t] - ntk;
+            z.pn_off = (int32_t)pruned_n.size();
+            z.pad_ = 0;
+            const int32_t *kn = p->kept_n_idx.data() + p->kept_n_ptr[t];
+            int j = 0;
+            for (int c = 0; c < p->tile_width[t]; ++c) {
+                if (j < ntk && kn[j] == c)
+                    ++j;
+                else
+                    pruned_n.push_back(c);
+            }
+            ztiles.push_back(z);
+        }
+    }
+    // work queue order: heaviest kept-K first, ties keep a tile's pieces adjacent
+    std::stable_sort(units.begin(), units.end(),
+                     [](const UnitDev &a, const UnitDev &b) { return a.k_kept > b.k_kept; });
+    p->packed_elems = off;
+    p->n_units = (int)units.size();
+    p->n_zero_tiles = (int)ztiles.size();
+
+    int st;
+    if (!p->d_kept_k) {
+        std::vector<int32_t> rel_k(p->kept_k_idx.size()), rel_n(p->kept_n_idx.size());
+        for (int t = 0; t < nt; ++t) {
+            for (int i = p->kept_k_ptr[t]; i < p->kept_k_ptr[t + 1]; ++i)
+                rel_k[i] = p->kept_k_idx[i] - (i - p->kept_k_ptr[t]);
+            for (int i = p->kept_n_ptr[t]; i < p->kept_n_ptr[t + 1]; ++i)
+                rel_n[i] = p->kept_n_idx[i] - (i - p->kept_n_ptr[t]);
+        }
+        if ((st = upload(&p->d_kept_k, p->kept_k_idx)) || (st = upload(&p->d_kept_n, p->kept_n_idx)) ||
+            (st = upload(&p->d_rel_k, rel_k)) || (st = upload(&p->d_rel_n, rel_n)))
+            return st;
+    }
+    if ((st = upload(&p->d_units, units)) || (st = upload(&p->d_tiles, ztiles)) ||
+        (st = upload(&p->d_pruned_n, pruned_n)))
+        return st;
+    size_t bp_bytes = std::max<int64_t>(p->packed_elems, 8) * 2;
+    if (hipMalloc(&p->d_Bp, bp_bytes) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the packed weight failed", bp_bytes);
+    TW_HIP(hipMemset(p->d_Bp, 0, bp_bytes));
+    if (hipMalloc((void **)&p->d_tickets, sizeof(int32_t) * 2 * kTicketSlots) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of the ticket slots failed");
+    TW_HIP(hipMemset(p->d_tickets, 0, sizeof(int32_t) * 2 * kTicketSlots));
+    hipDeviceProp_t prop;
+    TW_HIP(hipGetDevice(&p->device));
+    TW_HIP(hipGetDeviceProperties(&prop, p->device));
+    p->cu_count = prop.multiProcessorCount;
+    return TW_OK;
+}
+
+int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s)
+{
+    const int64_t mg = max_groups(p);
+    if (mg == 0)
+        return TW_OK;
+    std::vector<PackTile> pt = pack_tiles(p, nullptr);
+    PackTile *d_pt = nullptr;
+    int st = upload(&d_pt, pt);
+    if (st)
+        return st;
+    dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
+    hipLaunchKernelGGL(pack_dense_kernel, grid, dim3(256), 0, s, d_pt, p->d_kept_k, p->d_kept_n,
+                       d_B, p->N, p->dtype, (uint16_t *)p->d_Bp);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(s);
+    hipFree(d_pt);
+    if (e != hipSuccess)
+        return fail(TW_ERR_DEVICE, "weight packing kernel failed: %s", hipGetErrorString(e));
+    return TW_OK;
+}
+
+int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStream_t s)
+{
+    const int64_t mg = max_groups(p);
+    if (mg == 0)
+        return TW_OK;
+    std::vector<PackTile> pt = pack_tiles(p, off_B);
+    PackTile *d_pt = nullptr;
+    int st = upload(&d_pt, pt);
+    if (st)
+        return st;
+    dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
+    hipLaunchKernelGGL(pack_stream_kernel, grid, dim3(256), 0, s, d_pt, (const uint16_t *)d_Bs,
+                       p->K, (uint16_t *)p->d_Bp);
+    hipError_t e = hipGetLastError();
+    if (e == hipSuccess)
+        e = hipStreamSynchronize(s);
+    hipFree(d_pt);
+    if (e != hipSuccess)
+        return fail(TW_ERR_DEVICE, "stream-weight packing kernel failed: %s", hipGetErrorString(e));
+    return TW_OK;
+}
+
+int unpack_to_stream(const tw_plan *p, uint16_t *d_Bs, hipStream_t s)
+{
+    TW_HIP(hipMemsetAsync(d_Bs, 0, (size_t)p->K * p->N * 2, s));
+    const int64_t mg = max_groups(p);
+    if (mg > 0) {
+        std::vector<PackTile> pt = pack_tiles(p, nullptr);
+        PackTile *d_pt = nullptr;
+        int st = upload(&d_pt, pt);
+        if (st)
+            return st;
+        dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
+        hipLaunchKernelGGL(unpack_stream_kernel, grid, dim3(256), 0, s, d_pt,
+                           (const uint16_t *)p->d_Bp, p->K, d_Bs);
+        hipError_t e = hipGetLastError();
+        if (e == hipSuccess)
+            e = hipStreamSynchronize(s);
+        hipFree(d_pt);
+        if (e != hipSuccess)
+            return fail(TW_ERR_DEVICE, "unpack kernel failed: %s", hipGetErrorString(e));
+    }
+    TW_HIP(hipStreamSynchronize(s));
+    return TW_OK;
+}
+
+static void free_plan(tw_plan *p)
+{
+    if (!p)
+        return;
+    hipFree(p->d_kept_k);
+    hipFree(p->d_kept_n);
+    hipFree(p->d_rel_k);
+    hipFree(p->d_rel_n);
+    hipFree(p->d_pruned_n);
+    hipFree(p->d_units);
+    hipFree(p->d_tiles);
+    hipFree(p->d_Bp);
+    hipFree(p->d_tickets);
+    delete p;
+}
+
+static int check_dtype(int dtype)
+{
+    if (dtype != TW_F16 && dtype != TW_BF16)
+        return fail(TW_ERR_DTYPE, "dtype %d is neither TW_F16 nor TW_BF16", dtype);
+    return TW_OK;
+}
+
+// uploads a host fp32 [K,N] weight and packs it
+static int pack_host_weight(tw_plan *p, const float *B)
+{
+    if (p->packed_elems == 0)
+        return TW_OK;
+    float *d_B = nullptr;
+    size_t bytes = (size_t)p->K * p->N * sizeof(float);
+    if (hipMalloc((void **)&d_B, bytes) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the weight upload failed", bytes);
+    hipError_t e = hipMemcpy(d_B, B, bytes, hipMemcpyHostToDevice);
+    int st = e == hipSuccess ? pack_from_dense(p, d_B, nullptr)
+                             : fail(TW_ERR_DEVICE, "weight upload failed: %s", hipGetErrorString(e));
+    hipFree(d_B);
+    return st;
+}
+
+} // namespace tw
+
+using namespace tw;
+
+extern "C" {
+
+int tw_plan_create(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                   const int32_t *tile_width, const int32_t *kept_k_ptr, const int32_t *kept_k_idx,
+                   const int32_t *kept_n_ptr, const int32_t *kept_n_idx, const float *B,
+                   tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    int st = check_dtype(dtype);
+    if (st)
+        return st;
+    st = validate_lists(K, N, n_tiles, tile_col0, tile_width, kept_k_ptr, kept_k_idx, kept_n_ptr,
+                        kept_n_idx);
+    if (st)
+        return st;
+    if (!B)
+        return fail(TW_ERR_NULL, "B is NULL");
+    tw_plan *p = new (std::nothrow) tw_plan;
+    if (!p)
+        return fail(TW_ERR_ALLOC, "out of host memory");
+    p->K = K;
+    p->N = N;
+    p->dtype = dtype;
+    p->n_tiles = n_tiles;
+    p->tile_col0.assign(tile_col0, tile_col0 + n_tiles);
+    p->tile_width.assign(tile_width, tile_width + n_tiles);
+    p->kept_k_ptr.assign(kept_k_ptr, kept_k_ptr + n_tiles + 1);
+    p->kept_n_ptr.assign(kept_n_ptr, kept_n_ptr + n_tiles + 1);
+    p->kept_k_idx.assign(kept_k_idx, kept_k_idx + kept_k_ptr[n_tiles]);
+    p->kept_n_idx.assign(kept_n_idx, kept_n_idx + kept_n_ptr[n_tiles]);
+    if ((st = finalize_plan_geometry(p)) || (st = pack_host_weight(p, B))) {
+        free_plan(p);
+        return st;
+    }
+    *out = p;
+    return TW_OK;
+}
+
+int tw_plan_create_dense(int K, int N, int G, int dtype, const float *B, tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (K <= 0 || N <= 0 || G <= 0)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d G=%d must all be positive", K, N, G);
+    const int nt = (N + G - 1) / G;
+    std::vector<int32_t> col0(nt), width(nt), kp(nt + 1), np(nt + 1), ki, ni;
+    ki.reserve((size_t)nt * K);
+    ni.reserve(N);
+    kp[0] = np[0] = 0;
+    for (int t = 0; t < nt; ++t) {
+        col0[t] = t * G;
+        width[t] = std::min(G, N - t * G);
+        for (int k = 0; k < K; ++k)
+            ki.push_back(k);
+        for (int c = 0; c < width[t]; ++c)
+            ni.push_back(c);
+        kp[t + 1] = (int32_t)ki.size();
+        np[t + 1] = (int32_t)ni.size();
+    }
+    return tw_plan_create(K, N, dtype, nt, col0.data(), width.data(), kp.data(), ki.data(),
+                          np.data(), ni.data(), B, out);
+}
+
+int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const float *B,
+                      tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    int st = check_dtype(dtype);
+    if (st)
+        return st;
+    if (K <= 0 || N <= 0 || G <= 0)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d G=%d must all be positive", K, N, G);
+    if (!mask || !B)
+        return fail(TW_ERR_NULL, "mask or B is NULL");
+    const int nt = (N + G - 1) / G;
+
+    uint8_t *d_mask = nullptr, *d_rowflag = nullptr;
+    uint32_t *d_colflag = nullptr;
+    unsigned long long *d_mismatch = nullptr;
+    int32_t *d_counts = nullptr, *d_kptr = nullptr, *d_nptr = nullptr;
+    tw_plan *p = nullptr;
+    auto cleanup = [&]() {
+        hipFree(d_mask);
+        hipFree(d_rowflag);
+        hipFree(d_colflag);
+        hipFree(d_mismatch);
+        hipFree(d_counts);
+        hipFree(d_kptr);
+        hipFree(d_nptr);
+    };
+#define TW_TRY(call)                                                                       \
+    do {                                                                                   \
+        hipError_t e_ = (call);                                                            \
+        if (e_ != hipSuccess) {                                                            \
+            cleanup();                                                                     \
+            free_plan(p);                                                                  \
+            return fail(TW_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(e_));     \
+        }                                                                                  \
+    } while (0)
+
+    const size_t mask_bytes = (size_t)K * N;
+    TW_TRY(hipMalloc((void **)&d_mask, mask_bytes));
+    TW_TRY(hipMalloc((void **)&d_rowflag, (size_t)nt * K));
+    TW_TRY(hipMalloc((void **)&d_colflag, sizeof(uint32_t) * N));
+    TW_TRY(hipMalloc((void **)&d_mismatch, sizeof(unsigned long long)));
+    TW_TRY(hipMalloc((void **)&d_counts, sizeof(int32_t) * 2 * nt));
+    TW_TRY(hipMemcpy(d_mask, mask, mask_bytes, hipMemcpyHostToDevice));
+    TW_TRY(hipMemset(d_colflag, 0, sizeof(uint32_t) * N));
+    TW_TRY(hipMemset(d_mismatch, 0, sizeof(unsigned long long)));
+
+    {
+        const int64_t n_rt = (int64_t)K * nt;
+        hipLaunchKernelGGL(row_flags_kernel, dim3((unsigned)((n_rt + 255) / 256)), dim3(256), 0,
+                           nullptr, d_mask, K, N, G, nt, d_rowflag);
+        hipLaunchKernelGGL(col_flags_kernel, dim3((N + 255) / 256, (K + 63) / 64), dim3(256), 0,
+                           nullptr, d_mask, K, N, d_colflag);
+        const int64_t n_el = (int64_t)K * N;
+        hipLaunchKernelGGL(validate_tw_kernel, dim3((unsigned)((n_el + 255) / 256)), dim3(256), 0,
+                           nullptr, d_mask, K, N, G, d_rowflag, d_colflag, d_mismatch);
+        hipLaunchKernelGGL(count_flags_kernel, dim3(nt), dim3(256), 0, nullptr, d_rowflag,
+                           d_colflag, K, N, G, nt, d_counts);
+        TW_TRY(hipGetLastError());
+    }
+    unsigned long long mismatch = 0;
+    std::vector<int32_t> counts(2 * nt);
+    TW_TRY(hipMemcpy(&mismatch, d_mismatch, sizeof(mismatch), hipMemcpyDeviceToHost));
+    TW_TRY(hipMemcpy(counts.data(), d_counts, sizeof(int32_t) * 2 * nt, hipMemcpyDeviceToHost));
+    if (mismatch != 0) {
+        cleanup();
+        return fail(TW_ERR_NOT_TW,
+                    "%llu mask elements differ from (row kept) & (column kept) for G=%d", mismatch,
+                    G);
+    }
+
+    p = new (std::nothrow) tw_plan;
+    if (!p) {
+        cleanup();
+        return fail(TW_ERR_ALLOC, "out of host memory");
+    }
+    p->K = K;
+    p->N = N;
+    p->dtype = dtype;
+    p->n_tiles = nt;
+    p->tile_col0.resize(nt);
+    p->tile_width.resize(nt);
+    p->kept_k_ptr.assign(nt + 1, 0);
+    p->kept_n_ptr.assign(nt + 1, 0);
+    for (int t = 0; t < nt; ++t) {
+        p->tile_col0[t] = t * G;
+        p->tile_width[t] = std::min(G, N - t * G);
+        p->kept_k_ptr[t + 1] = p->kept_k_ptr[t] + counts[t];
+        p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + counts[nt + t];
+    }
+    const size_t sk = std::max(p->kept_k_ptr[nt], 1), sn = std::max(p->kept_n_ptr[nt], 1);
+    TW_TRY(hipMalloc((void **)&d_kptr, sizeof(int32_t) * (nt + 1)));
+    TW_TRY(hipMalloc((void **)&d_nptr, sizeof(int32_t) * (nt + 1)));
+    TW_TRY(hipMemcpy(d_kptr, p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
+    TW_TRY(hipMemcpy(d_nptr, p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
+    TW_TRY(hipMalloc((void **)&p->d_kept_k, sizeof(int32_t) * sk));
+    TW_TRY(hipMalloc((void **)&p->d_rel_k, sizeof(int32_t) * sk));
+    TW_TRY(hipMalloc((void **)&p->d_kept_n, sizeof(int32_t) * sn));
+    TW_TRY(hipMalloc((void **)&p->d_rel_n, sizeof(int32_t) * sn));
+    hipLaunchKernelGGL(compact_lists_kernel, dim3(nt, 2), dim3(256), 0, nullptr, d_rowflag,
+                       d_colflag, K, N, G, d_kptr, d_nptr, p->d_kept_k, p->d_rel_k, p->d_kept_n,
+                       p->d_rel_n);
+    TW_TRY(hipGetLastError());
+    p->kept_k_idx.resize(p->kept_k_ptr[nt]);
+    p->kept_n_idx.resize(p->kept_n_ptr[nt]);
+    if (!p->kept_k_idx.empty())
+        TW_TRY(hipMemcpy(p->kept_k_idx.data(), p->d_kept_k, sizeof(int32_t) * p->kept_k_idx.size(),
+                         hipMemcpyDeviceToHost));
+    if (!p->kept_n_idx.empty())
+        TW_TRY(hipMemcpy(p->kept_n_idx.data(), p->d_kept_n, sizeof(int32_t) * p->kept_n_idx.size(),
+                         hipMemcpyDeviceToHost));
+    cleanup();
+#undef TW_TRY
+    st = validate_lists(K, N, nt, p->tile_col0.data(), p->tile_width.data(), p->kept_k_ptr.data(),
+                        p->kept_k_idx.data(), p->kept_n_ptr.data(), p->kept_n_idx.data());
+    if (!st)
+        st = finalize_plan_geometry(p);
+    if (!st)
+        st = pack_host_weight(p, B);
+    if (st) {
+        free_plan(p);
+        return st;
+    }
+    *out = p;
+    return TW_OK;
+}
+
+int tw_plan_from_stream_operands(int M, int N, int K, int dtype, const void *B_stream,
+                                 int block_num, const int32_t *N_cal, const int32_t *K_cal,
+                                 const int32_t *const *mask_n, const int32_t *const *mask_k,
+                                 const int64_t *off_B, const int64_t *off_C, tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    int st = check_dtype(dtype);
+    if (st)
+        return st;
+    if (M <= 0 || N <= 0 || K <= 0 || block_num <= 0)
+        return fail(TW_ERR_SHAPE, "M=%d N=%d K=%d block_num=%d must all be positive", M, N, K,
+                    block_num);
+    if (!B_stream || !N_cal || !K_cal || !mask_n || !mask_k || !off_B || !off_C)
+        return fail(TW_ERR_NULL, "an operand pointer is NULL");
+    std::vector<int32_t> col0(block_num), width(block_num), kp(block_num + 1, 0),
+        np(block_num + 1, 0), ki, ni;
+    for (int t = 0; t < block_num; ++t) {
+        if (off_C[t] % M != 0)
+            return fail(TW_ERR_TILE_TABLE, "off_C[%d] = %lld is not a multiple of M", t,
+                        (long long)off_C[t]);
+        col0[t] = (int32_t)(off_C[t] / M);
+        if (N_cal[t] < 0 || K_cal[t] < 0 || K_cal[t] > K)
+            return fail(TW_ERR_SHAPE, "tile %d: N_cal=%d K_cal=%d", t, N_cal[t], K_cal[t]);
+        if ((N_cal[t] > 0 && !mask_n[t]) || (K_cal[t] > 0 && !mask_k[t]))
+            return fail(TW_ERR_NULL, "mask pointer of tile %d is NULL", t);
+    }
+    for (int t = 0; t < block_num; ++t) {
+        const int next = t + 1 < block_num ? col0[t + 1] : N;
+        width[t] = next - col0[t];
+        if (width[t] <= 0 || N_cal[t] > width[t])
+            return fail(TW_ERR_TILE_TABLE, "tile %d: width %d, N_cal %d", t, width[t], N_cal[t]);
+        if (off_B[t] < 0 || off_B[t] + (int64_t)std::max(N_cal[t] - 1, 0) * K + K_cal[t] >
+                                (int64_t)K * N)
+            return fail(TW_ERR_SHAPE, "off_B[%d] = %lld leaves the K*N weight buffer", t,
+                        (long long)off_B[t]);
+        std::vector<int32_t> rel_k(K_cal[t]), rel_n(N_cal[t]);
+        if (K_cal[t])
+            TW_HIP(hipMemcpy(rel_k.data(), mask_k[t], sizeof(int32_t) * K_cal[t],
+                             hipMemcpyDeviceToHost));
+        if (N_cal[t])
+            TW_HIP(hipMemcpy(rel_n.data(), mask_n[t], sizeof(int32_t) * N_cal[t],
+                             hipMemcpyDeviceToHost));
+        size_t k0 = ki.size(), n0 = ni.size();
+        ki.resize(k0 + K_cal[t]);
+        ni.resize(n0 + N_cal[t]);
+        if ((st = tw_offsets_to_kept(rel_k.data(), K_cal[t], K, ki.data() + k0)) ||
+            (st = tw_offsets_to_kept(rel_n.data(), N_cal[t], width[t], ni.data() + n0)))
+            return st;
+        kp[t + 1] = (int32_t)ki.size();
+        np[t + 1] = (int32_t)ni.size();
+    }
+    st = validate_lists(K, N, block_num, col0.data(), width.data(), kp.data(), ki.data(), np.data(),
+                        ni.data());
+    if (st)
+        return st;
+    tw_plan *p = new (std::nothrow) tw_plan;
+    if (!p)
+        return fail(TW_ERR_ALLOC, "out of host memory");
+    p->K = K;
+    p->N = N;
+    p->dtype = dtype;
+    p->n_tiles = block_num;
+    p->tile_col0 = col0;
+    p->tile_width = width;
+    p->kept_k_ptr = kp;
+    p->kept_n_ptr = np;
+    p->kept_k_idx = ki;
+    p->kept_n_idx = ni;
+    if ((st = finalize_plan_geometry(p)) || (st = pack_from_stream(p, B_stream, off_B, nullptr))) {
+        free_plan(p);
+        return st;
+    }
+    *out = p;
+    return TW_OK;
+}
+
+int tw_plan_info(const tw_plan *p, int64_t *info, int n_info)
+{
+    if (!p || !info)
+        return fail(TW_ERR_NULL, "plan or info is NULL");
+    int64_t v[12] = {0};
+    v[0] = p->K;
+    v[1] = p->N;
+    v[2] = p->dtype;
+    v[3] = p->n_tiles;
+    for (int t = 0; t < p->n_tiles; ++t) {
+        const int64_t kt = p->kept_k_ptr[t + 1] - p->kept_k_ptr[t];
+        const int64_t nt = p->kept_n_ptr[t + 1] - p->kept_n_ptr[t];
+        v[4] += kt;
+        v[5] += nt;
+        v[6] += kt * nt;
+        v[8] = std::max(v[8], kt);
+        v[9] = std::max(v[9], nt);
+        v[10] += (kt * nt == 0);
+        v[11] += p->tile_width[t];
+    }
+    v[7] = p->packed_elems * 2;
+    for (int i = 0; i < n_info && i < 12; ++i)
+        info[i] = v[i];
+    return TW_OK;
+}
+
+int tw_plan_export(const tw_plan *p, int32_t *tile_col0, int32_t *tile_width, int32_t *kept_k_ptr,
+                   int32_t *kept_k_idx, int32_t *mask_k_rel, int32_t *kept_n_ptr,
+                   int32_t *kept_n_idx, int32_t *mask_n_rel, uint16_t *B_stream)
+{
+    if (!p)
+        return fail(TW_ERR_NULL, "plan is NULL");
+    const int nt = p->n_tiles;
+    if (tile_col0)
+        memcpy(tile_col0, p->tile_col0.data(), sizeof(int32_t) * nt);
+    if (tile_width)
+        memcpy(tile_width, p->tile_width.data(), sizeof(int32_t) * nt);
+    if (kept_k_ptr)
+        memcpy(kept_k_ptr, p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1));
+    if (kept_n_ptr)
+        memcpy(kept_n_ptr, p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1));
+    const size_t sk = p->kept_k_idx.size(), sn = p->kept_n_idx.size();
+    // the index lists come back from the device copies the kernels read
+    if (kept_k_idx && sk)
+        TW_HIP(hipMemcpy(kept_k_idx, p->d_kept_k, sizeof(int32_t) * sk, hipMemcpyDeviceToHost));
+    if (mask_k_rel && sk)
+        TW_HIP(hipMemcpy(mask_k_rel, p->d_rel_k, sizeof(int32_t) * sk, hipMemcpyDeviceToHost));
+    if (kept_n_idx && sn)
+        TW_HIP(hipMemcpy(kept_n_idx, p->d_kept_n, sizeof(int32_t) * sn, hipMemcpyDeviceToHost));
+    if (mask_n_rel && sn)
+        TW_HIP(hipMemcpy(mask_n_rel, p->d_rel_n, sizeof(int32_t) * sn, hipMemcpyDeviceToHost));
+    if (B_stream) {
+        uint16_t *d_Bs = nullptr;
+        const size_t bytes = (size_t)p->K * p->N * 2;
+        if (hipMalloc((void **)&d_Bs, bytes) != hipSuccess)
+            return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes failed", bytes);
+        int st = unpack_to_stream(p, d_Bs, nullptr);
+        hipError_t e = hipSuccess;
+        if (!st)
+            e = hipMemcpy(B_stream, d_Bs, bytes, hipMemcpyDeviceToHost);
+        hipFree(d_Bs);
+        if (st)
+            return st;
+        if (e != hipSuccess)
+            return fail(TW_ERR_DEVICE, "read-back failed: %s", hipGetErrorString(e));
+    }
+    return TW_OK;
+}
+
+int tw_plan_destroy(tw_plan *plan)
+{
+    free_plan(plan);
+    return TW_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,338 @@
+"""ctypes binding of libtwgemm.so and the host-side mirror of the reference's
+TW-GEMM driver interface (StreamMaskedGEMM/perf/basic_nn.cu).
+
+The names follow the reference: ``mask_to_offsets`` (convert_mask_to_offset,
+Pruning/BERT/utils/MyHook.py:66-74), ``tile_partition`` (basic_nn.cu:836-885),
+``Plan`` (the per-tile mask_k / mask_n / compacted weight that
+basic_nn.cu:891-914 builds), ``Plan.gemm`` / ``stream_gemm_nn`` (Stream_Gemm_NN,
+basic_nn.cu:378-445).  Device memory is passed as raw pointers (integers), e.g.
+``torch.Tensor.data_ptr()``; this module itself does not import torch.
+
+There is no CPU fallback: if the HIP library is missing, loading fails loudly.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "libtwgemm.so")
+
+F16, BF16 = 0, 1
+KMAJOR, ROWMAJOR = 0, 1
+PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
+
+OK = 0
+ERR_NULL, ERR_SHAPE, ERR_TILE_TABLE, ERR_INDEX_LIST, ERR_DTYPE = -1, -2, -3, -4, -5
+ERR_LAYOUT, ERR_ALIGNMENT, ERR_NOT_TW, ERR_DEVICE, ERR_ALLOC, ERR_BUFFER = -6, -7, -8, -9, -10, -11
+
+_DTYPES = {"f16": F16, "fp16": F16, "half": F16, "bf16": BF16, F16: F16, BF16: BF16}
+
+# every symbol include/twgemm.h declares
+EXPORTED_SYMBOLS = (
+    "tw_version", "tw_last_error", "tw_status_string",
+    "tw_mask_to_offsets", "tw_offsets_to_kept", "tw_tile_partition",
+    "tw_plan_create", "tw_plan_create_dense", "tw_plan_from_mask",
+    "tw_plan_from_stream_operands", "tw_plan_info", "tw_plan_export", "tw_plan_destroy",
+    "tw_gemm", "tw_stream_gemm_nn", "tw_cast_f32", "tw_delete_row", "tw_insert_row",
+)
+
+
+class TwError(RuntimeError):
+    """A libtwgemm call returned a negative status."""
+
+    def __init__(self, status, message):
+        super().__init__("libtwgemm status %d: %s" % (status, message))
+        self.status = status
+        self.message = message
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library (raises if libtwgemm.so has not been built)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python -m tilesparsity_amd.build` "
+            "(there is no CPU fallback)" % LIB_PATH)
+    L = ctypes.CDLL(LIB_PATH)
+    c_int, c_i64, c_f, vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
+    i32p = ctypes.POINTER(ctypes.c_int32)
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    u8p = ctypes.POINTER(ctypes.c_uint8)
+    u16p = ctypes.POINTER(ctypes.c_uint16)
+    f32p = ctypes.POINTER(ctypes.c_float)
+    pp = ctypes.POINTER(vp)
+    sig = {
+        "tw_version": (c_int, []),
+        "tw_last_error": (ctypes.c_char_p, []),
+        "tw_status_string": (ctypes.c_char_p, [c_int]),
+        "tw_mask_to_offsets": (c_int, [u8p, c_int, i32p, ctypes.POINTER(c_int)]),
+        "tw_offsets_to_kept": (c_int, [i32p, c_int, c_int, i32p]),
+        "tw_tile_partition": (c_int, [c_int] * 7 + [ctypes.POINTER(c_int), i32p, i32p, i32p,
+                                                     i64p, i64p]),
+        "tw_plan_create": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, i32p, i32p, i32p,
+                                   i32p, f32p, pp]),
+        "tw_plan_create_dense": (c_int, [c_int, c_int, c_int, c_int, f32p, pp]),
+        "tw_plan_from_mask": (c_int, [c_int, c_int, c_int, c_int, u8p, f32p, pp]),
+        "tw_plan_from_stream_operands": (c_int, [c_int, c_int, c_int, c_int, vp, c_int, i32p,
+                                                 i32p, pp, pp, i64p, i64p, pp]),
+        "tw_plan_info": (c_int, [vp, i64p, c_int]),
+        "tw_plan_export": (c_int, [vp, i32p, i32p, i32p, i32p, i32p, i32p, i32p, i32p, u16p]),
+        "tw_plan_destroy": (c_int, [vp]),
+        "tw_gemm": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int, vp]),
+        "tw_stream_gemm_nn": (c_int, [c_int, c_int, c_int, c_int, c_f, vp, vp, c_f, vp, c_int,
+                                      i32p, i32p, pp, pp, i64p, i64p, vp]),
+        "tw_cast_f32": (c_int, [vp, vp, c_i64, c_int, vp]),
+        "tw_delete_row": (c_int, [vp, vp, c_int, c_int, vp, vp]),
+        "tw_insert_row": (c_int, [vp, vp, c_int, c_int, vp, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(L, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = L
+    return L
+
+
+def _check(status):
+    if status != OK:
+        raise TwError(status, lib().tw_last_error().decode())
+
+
+def _i32(a):
+    return np.ascontiguousarray(a, dtype=np.int32)
+
+
+def _ptr(a, ct):
+    return a.ctypes.data_as(ctypes.POINTER(ct))
+
+
+def dtype_code(dtype):
+    try:
+        return _DTYPES[dtype]
+    except KeyError:
+        raise TwError(ERR_DTYPE, "unknown dtype %r" % (dtype,))
+
+
+def version():
+    return lib().tw_version()
+
+
+# --------------------------------------------------------------------------- integer helpers
+def mask_to_offsets(mask):
+    """0/1 keep vector -> relative offsets kept[i]-i (convert_mask_to_offset)."""
+    mask = np.ascontiguousarray(mask, dtype=np.uint8)
+    out = np.empty(max(mask.size, 1), dtype=np.int32)
+    n = ctypes.c_int(0)
+    _check(lib().tw_mask_to_offsets(_ptr(mask, ctypes.c_uint8), mask.size,
+                                    _ptr(out, ctypes.c_int32), ctypes.byref(n)))
+    return out[:n.value].copy()
+
+
+def offsets_to_kept(offsets, limit):
+    """Relative offsets -> ascending kept indices in [0, limit)."""
+    offsets = _i32(offsets)
+    out = np.empty(max(offsets.size, 1), dtype=np.int32)
+    _check(lib().tw_offsets_to_kept(_ptr(offsets, ctypes.c_int32), offsets.size, limit,
+                                    _ptr(out, ctypes.c_int32)))
+    return out[:offsets.size].copy()
+
+
+def tile_partition(M, N, K, N_pruned, K_pruned, n_dim=128, max_tiles=4096):
+    """Tile partition of TestCutlassGemm (basic_nn.cu:836-885)."""
+    bn = ctypes.c_int(0)
+    N_ori = np.zeros(max_tiles, np.int32)
+    N_cal = np.zeros(max_tiles, np.int32)
+    K_cal = np.zeros(max_tiles, np.int32)
+    off_B = np.zeros(max_tiles, np.int64)
+    off_C = np.zeros(max_tiles, np.int64)
+    _check(lib().tw_tile_partition(M, N, K, N_pruned, K_pruned, n_dim, max_tiles,
+                                   ctypes.byref(bn), _ptr(N_ori, ctypes.c_int32),
+                                   _ptr(N_cal, ctypes.c_int32), _ptr(K_cal, ctypes.c_int32),
+                                   _ptr(off_B, ctypes.c_int64), _ptr(off_C, ctypes.c_int64)))
+    n = bn.value
+    return dict(block_num=n, N_ori=N_ori[:n].tolist(), N_cal=N_cal[:n].tolist(),
+                K_cal=K_cal[:n].tolist(), off_B=off_B[:n].tolist(), off_C=off_C[:n].tolist())
+
+
+def tiles_to_csr(tiles):
+    """list of tile dicts (col0, width, kept_k, kept_n) -> the six flat arrays."""
+    col0 = _i32([t["col0"] for t in tiles])
+    width = _i32([t["width"] for t in tiles])
+    kp = np.zeros(len(tiles) + 1, np.int32)
+    npt = np.zeros(len(tiles) + 1, np.int32)
+    for i, t in enumerate(tiles):
+        kp[i + 1] = kp[i] + len(t["kept_k"])
+        npt[i + 1] = npt[i] + len(t["kept_n"])
+    ki = _i32(np.concatenate([_i32(t["kept_k"]) for t in tiles])) if tiles else _i32([])
+    ni = _i32(np.concatenate([_i32(t["kept_n"]) for t in tiles])) if tiles else _i32([])
+    return col0, width, kp, ki, npt, ni
+
+
+# --------------------------------------------------------------------------- plans
+class Plan:
+    """Device-resident TW weight: tile table, kept-K / kept-N lists, packed weight."""
+
+    def __init__(self, handle, K, N, dtype):
+        self._h = ctypes.c_void_p(handle)
+        self.K, self.N, self.dtype = K, N, dtype
+
+    # -- constructors
+    @classmethod
+    def create(cls, K, N, dtype, tiles, B):
+        """From an explicit tile table (list of dicts) and the fp32 weight B[K,N]."""
+        col0, width, kp, ki, npt, ni = tiles_to_csr(tiles)
+        return cls.create_csr(K, N, dtype, col0, width, kp, ki, npt, ni, B)
+
+    @classmethod
+    def create_csr(cls, K, N, dtype, col0, width, kp, ki, npt, ni, B):
+        B = np.ascontiguousarray(B, dtype=np.float32)
+        if B.size != K * N:
+            raise TwError(ERR_SHAPE, "B has %d elements, expected K*N=%d" % (B.size, K * N))
+        col0, width, kp, ki, npt, ni = map(_i32, (col0, width, kp, ki, npt, ni))
+        h = ctypes.c_void_p()
+        i32 = ctypes.c_int32
+        _check(lib().tw_plan_create(K, N, dtype_code(dtype), col0.size, _ptr(col0, i32),
+                                    _ptr(width, i32), _ptr(kp, i32), _ptr(ki, i32),
+                                    _ptr(npt, i32), _ptr(ni, i32), _ptr(B, ctypes.c_float),
+                                    ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def dense(cls, K, N, G, dtype, B):
+        """The 0 %-sparse plan (every row and column kept)."""
+        B = np.ascontiguousarray(B, dtype=np.float32)
+        if B.size != K * N:
+            raise TwError(ERR_SHAPE, "B has %d elements, expected K*N=%d" % (B.size, K * N))
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_create_dense(K, N, G, dtype_code(dtype), _ptr(B, ctypes.c_float),
+                                          ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def from_mask(cls, mask, G, dtype, B):
+        """From a dense 0/1 mask [K,N]; the integer pre-pass runs on the GPU."""
+        mask = np.ascontiguousarray(mask, dtype=np.uint8)
+        K, N = mask.shape
+        B = np.ascontiguousarray(B, dtype=np.float32)
+        if B.size != K * N:
+            raise TwError(ERR_SHAPE, "B has %d elements, expected K*N=%d" % (B.size, K * N))
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_from_mask(K, N, G, dtype_code(dtype), _ptr(mask, ctypes.c_uint8),
+                                       _ptr(B, ctypes.c_float), ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def from_stream_operands(cls, M, N, K, dtype, B_stream_ptr, N_cal, K_cal, mask_n_ptrs,
+                             mask_k_ptrs, off_B, off_C):
+        """From the device operands of the reference's Stream_Gemm_NN."""
+        N_cal, K_cal = _i32(N_cal), _i32(K_cal)
+        off_B = np.ascontiguousarray(off_B, dtype=np.int64)
+        off_C = np.ascontiguousarray(off_C, dtype=np.int64)
+        bn = N_cal.size
+        mn = (ctypes.c_void_p * bn)(*[int(p) for p in mask_n_ptrs])
+        mk = (ctypes.c_void_p * bn)(*[int(p) for p in mask_k_ptrs])
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_from_stream_operands(
+            M, N, K, dtype_code(dtype), ctypes.c_void_p(int(B_stream_ptr)), bn,
+            _ptr(N_cal, ctypes.c_int32), _ptr(K_cal, ctypes.c_int32), mn, mk,
+            _ptr(off_B, ctypes.c_int64), _ptr(off_C, ctypes.c_int64), ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    # -- inspection
+    def info(self):
+        v = np.zeros(12, np.int64)
+        _check(lib().tw_plan_info(self._h, _ptr(v, ctypes.c_int64), 12))
+        keys = ("K", "N", "dtype", "n_tiles", "sum_k", "sum_n", "kept_elems", "packed_bytes",
+                "max_k", "max_n", "empty_tiles", "total_width")
+        return dict(zip(keys, (int(x) for x in v)))
+
+    def export(self, with_weight=True):
+        """Tile table, kept lists, relative offsets and (optionally) the compacted
+        weight in the reference's stream layout, as 16-bit patterns [K*N]."""
+        inf = self.info()
+        nt, sk, sn = inf["n_tiles"], inf["sum_k"], inf["sum_n"]
+        i32 = ctypes.c_int32
+        col0, width = np.zeros(nt, np.int32), np.zeros(nt, np.int32)
+        kp, npt = np.zeros(nt + 1, np.int32), np.zeros(nt + 1, np.int32)
+        ki, rk = np.zeros(max(sk, 1), np.int32), np.zeros(max(sk, 1), np.int32)
+        ni, rn = np.zeros(max(sn, 1), np.int32), np.zeros(max(sn, 1), np.int32)
+        Bs = np.zeros(self.K * self.N, np.uint16) if with_weight else None
+        _check(lib().tw_plan_export(
+            self._h, _ptr(col0, i32), _ptr(width, i32), _ptr(kp, i32), _ptr(ki, i32),
+            _ptr(rk, i32), _ptr(npt, i32), _ptr(ni, i32), _ptr(rn, i32),
+            _ptr(Bs, ctypes.c_uint16) if with_weight else None))
+        tiles = []
+        for t in range(nt):
+            tiles.append(dict(col0=int(col0[t]), width=int(width[t]),
+                              kept_k=ki[kp[t]:kp[t + 1]].copy(), kept_n=ni[npt[t]:npt[t + 1]].copy(),
+                              mask_k=rk[kp[t]:kp[t + 1]].copy(), mask_n=rn[npt[t]:npt[t + 1]].copy()))
+        return tiles, Bs
+
+    # -- the GEMM
+    def gemm(self, A_ptr, C_ptr, M, lda=None, ldc=None, alpha=1.0, beta=0.0,
+             a_layout=KMAJOR, c_layout=KMAJOR, pruned_cols=PRUNED_UNTOUCHED, stream=0):
+        """C = alpha * A (B (.) mask) + beta * C on device pointers; asynchronous."""
+        if lda is None:
+            lda = M if a_layout == KMAJOR else self.K
+        if ldc is None:
+            ldc = M if c_layout == KMAJOR else self.N
+        _check(lib().tw_gemm(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
+                             ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
+                             pruned_cols, ctypes.c_void_p(int(stream or 0))))
+
+    def destroy(self):
+        if self._h is not None and self._h.value:
+            lib().tw_plan_destroy(self._h)
+        self._h = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.destroy()
+
+
+def stream_gemm_nn(M, N, K, dtype, alpha, A_ptr, B_ptr, beta, C_ptr, N_cal, K_cal, mask_n_ptrs,
+                   mask_k_ptrs, off_B, off_C, stream=0):
+    """One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), device pointers."""
+    N_cal, K_cal = _i32(N_cal), _i32(K_cal)
+    off_B = np.ascontiguousarray(off_B, dtype=np.int64)
+    off_C = np.ascontiguousarray(off_C, dtype=np.int64)
+    bn = N_cal.size
+    mn = (ctypes.c_void_p * bn)(*[int(p) for p in mask_n_ptrs])
+    mk = (ctypes.c_void_p * bn)(*[int(p) for p in mask_k_ptrs])
+    _check(lib().tw_stream_gemm_nn(M, N, K, dtype_code(dtype), alpha, ctypes.c_void_p(int(A_ptr)),
+                                   ctypes.c_void_p(int(B_ptr)), beta, ctypes.c_void_p(int(C_ptr)),
+                                   bn, _ptr(N_cal, ctypes.c_int32), _ptr(K_cal, ctypes.c_int32),
+                                   mn, mk, _ptr(off_B, ctypes.c_int64), _ptr(off_C, ctypes.c_int64),
+                                   ctypes.c_void_p(int(stream or 0))))
+
+
+def cast_f32(src_ptr, dst_ptr, n, dtype, stream=0):
+    """Device fp32 -> 16-bit cast (float_to_half)."""
+    _check(lib().tw_cast_f32(ctypes.c_void_p(int(src_ptr or 0)), ctypes.c_void_p(int(dst_ptr or 0)),
+                             n, dtype_code(dtype), ctypes.c_void_p(int(stream or 0))))
+
+
+def delete_row(matrix_ptr, matrix_2_ptr, rows, columns, mask_ptr, stream=0):
+    _check(lib().tw_delete_row(ctypes.c_void_p(int(matrix_ptr or 0)),
+                               ctypes.c_void_p(int(matrix_2_ptr or 0)), rows, columns,
+                               ctypes.c_void_p(int(mask_ptr or 0)), ctypes.c_void_p(int(stream or 0))))
+
+
+def insert_row(matrix_ptr, matrix_2_ptr, rows, columns, mask_ptr, stream=0):
+    _check(lib().tw_insert_row(ctypes.c_void_p(int(matrix_ptr or 0)),
+                               ctypes.c_void_p(int(matrix_2_ptr or 0)), rows, columns,
+                               ctypes.c_void_p(int(mask_ptr or 0)), ctypes.c_void_p(int(stream or 0))))

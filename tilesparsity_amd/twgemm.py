@@ -11,7 +11,9 @@ basic_nn.cu:378-445).  Device memory is passed as raw pointers (integers), e.g.
 There is no CPU fallback: if the HIP library is missing, loading fails loudly.
 """
 import ctypes
+import importlib.util
 import os
+import sys
 
 import numpy as np
 
@@ -50,6 +52,25 @@ class TwError(RuntimeError):
 _lib = None
 
 
+def _share_torch_hip_runtime():
+    """A process must hold ONE HIP runtime.  PyTorch wheels bundle their own
+    libamdhip64 (same soname as the system one); if it is loaded after the system copy
+    that libtwgemm.so would otherwise pull in, the second runtime finds no GPU.  So when
+    PyTorch is installed but not yet imported, its runtime is loaded first and
+    libtwgemm.so binds to it by soname.  TWGEMM_SYSTEM_HIP=1 skips this."""
+    if "torch" in sys.modules or os.environ.get("TWGEMM_SYSTEM_HIP") == "1":
+        return
+    try:
+        spec = importlib.util.find_spec("torch")
+    except (ImportError, ValueError):
+        spec = None
+    if spec is None or not spec.origin:
+        return
+    path = os.path.join(os.path.dirname(spec.origin), "lib", "libamdhip64.so")
+    if os.path.exists(path):
+        ctypes.CDLL(path, mode=ctypes.RTLD_GLOBAL)
+
+
 def lib():
     """The loaded library (raises if libtwgemm.so has not been built)."""
     global _lib
@@ -59,6 +80,7 @@ def lib():
         raise ImportError(
             "%s is missing: build it with `python -m tilesparsity_amd.build` "
             "(there is no CPU fallback)" % LIB_PATH)
+    _share_torch_hip_runtime()
     L = ctypes.CDLL(LIB_PATH)
     c_int, c_i64, c_f, vp = ctypes.c_int, ctypes.c_int64, ctypes.c_float, ctypes.c_void_p
     i32p = ctypes.POINTER(ctypes.c_int32)

@@ -83,7 +83,7 @@ __device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M
 }
 
 template <int DT, int WM, int WN, bool TR>
-__global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const GemmArgs p)
+__global__ void __launch_bounds__(64 * WM * WN, 2) tw_gemm_kmajor_kernel(const GemmArgs p)
 {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = 64 * WM;
@@ -96,6 +96,10 @@ __global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const Gemm
     constexpr int STAGE = BK * PITCH;
     constexpr int CPITCH = BM + 8;
     constexpr int SMEM = (2 * STAGE > BN * CPITCH) ? 2 * STAGE : BN * CPITCH;
+    constexpr int D = BM >= 256 ? 2 : 3; // prefetch distance in steps (24-32 KiB of A in flight)
+    constexpr int R = D + 1;         // register ring slots; the main loop is unrolled R times
+    constexpr int RPW = 64 / CPR;    // staged rows covered by one wave in one pass
+    typedef int IdxVec __attribute__((ext_vector_type(RPW)));
     using E = Elem<DT>;
 
     __shared__ __align__(16) uint16_t smem[SMEM];
@@ -104,10 +108,12 @@ __global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const Gemm
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int wm = wave % WM;
-    const int wn = wave / WM;
+    const int wm = __builtin_amdgcn_readfirstlane(wave % WM);
+    const int wn = __builtin_amdgcn_readfirstlane(wave / WM);
     const int chunk = tid % CPR;
     const int rrow = tid / CPR;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const int sub = lane / CPR;
     const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
     uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
     const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
@@ -150,42 +156,20 @@ __global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const Gemm
         const int m0 = (item - ui * p.n_mblk) * BM;
         const UnitDev u = p.units[ui];
         const int nsteps = u.k_pad / BK;
-        const int32_t *const klist = p.kept_k + u.kk_off;
+        const int32_t *const klist = p.kept_k + u.kk_off; // padded to k_pad entries
         const int m_ld = m0 + chunk * 8;
+        const bool m_ok = m_ld < p.M;
+        const int m_eff = m_ok ? m_ld : 0; // a valid chunk to read when this one is beyond M
         const int ksteps16 = u.k_pad / kMfmaK;
-
-        // gathered A rows for one step -> registers (zeros beyond K_t and beyond M)
-        auto load_a = [&](int s, u32x4(&r)[PASSES]) {
+        // packed weight operand streams of this wave's two 32-column blocks; a block
+        // beyond the unit reads block 0 (its products land in columns that are not stored)
+        const uint16_t *b_base[2];
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int kk = s * BK + ps * RPP + rrow;
-                u32x4 v = {0u, 0u, 0u, 0u};
-                if (kk < u.k_kept && m_ld < p.M)
-                    v = *reinterpret_cast<const u32x4 *>(A + (int64_t)klist[kk] * p.lda + m_ld);
-                r[ps] = v;
-            }
-        };
-        auto store_a = [&](int buf, const u32x4(&r)[PASSES]) {
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps)
-                *reinterpret_cast<u32x4 *>(smem + buf * STAGE + (ps * RPP + rrow) * PITCH +
-                                           chunk * 8) = r[ps];
-        };
-        // packed weight operands of one step: [k16 step][32-column block]
-        auto load_b = [&](int s, u32x4(&r)[2][2]) {
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni) {
-                    const int nb = wn * 2 + ni;
-                    u32x4 v = {0u, 0u, 0u, 0u};
-                    if (nb < u.nb_cnt)
-                        v = *reinterpret_cast<const u32x4 *>(
-                            Bp + u.b_off +
-                            (((int64_t)(u.nb0 + nb) * ksteps16 + (s * 2 + ks)) * 64 + lane) * 8);
-                    r[ks][ni] = v;
-                }
-        };
+        for (int ni = 0; ni < 2; ++ni) {
+            const int nb = wn * 2 + ni;
+            b_base[ni] = Bp + u.b_off +
+                         ((int64_t)(u.nb0 + (nb < u.nb_cnt ? nb : 0)) * ksteps16 * 64 + lane) * 8;
+        }
 
         f32x16 acc[2][2];
 #pragma unroll
@@ -196,22 +180,53 @@ __global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const Gemm
                 for (int r = 0; r < 16; ++r)
                     acc[mi][ni][r] = 0.0f;
 
-        u32x4 a_reg[PASSES];
-        u32x4 b_cur[2][2], b_nxt[2][2];
-        if (nsteps > 0) {
-            load_a(0, a_reg);
-            load_b(0, b_cur);
-            store_a(0, a_reg);
-        }
-        __syncthreads();
-
-        for (int s = 0; s < nsteps; ++s) {
-            const bool more = s + 1 < nsteps;
-            if (more) {
-                load_a(s + 1, a_reg);
-                load_b(s + 1, b_nxt);
+        // Register ring: the loads of step s+D are issued while step s is consumed, so D
+        // steps of gathered A rows (and of packed weight operands) are in flight per
+        // workgroup.  Loads return in order, so A and B share one prefetch distance.
+        // The kept-K indices of a step are wave-uniform per 16-byte-chunk row group and come
+        // through the scalar cache one step ahead of the loads that use them.
+        auto load_idx = [&](int s, IdxVec(&ix)[PASSES]) {
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const int kkbase = s * BK + ps * RPP + wave_u * RPW;
+                ix[ps] = *reinterpret_cast<const __attribute__((address_space(4))) IdxVec *>(
+                    (uintptr_t)(klist + kkbase));
             }
-            const uint16_t *stage = smem + (s & 1) * STAGE;
+        };
+        // No lane-dependent branches here: rows beyond K_t and chunks beyond M are loaded
+        // from a valid address and replaced by zeros when they are staged (not here, so that
+        // nothing waits on a load that was just issued).
+        auto issue = [&](int s, const IdxVec(&ix)[PASSES], u32x4(&ar)[PASSES], u32x4(&br)[2][2]) {
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                int my = ix[ps][0];
+#pragma unroll
+                for (int q = 1; q < RPW; ++q)
+                    my = sub == q ? ix[ps][q] : my;
+                ar[ps] = *reinterpret_cast<const u32x4 *>(A + (int64_t)my * p.lda + m_eff);
+            }
+#pragma unroll
+            for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+                    br[ks][ni] = *reinterpret_cast<const u32x4 *>(
+                        b_base[ni] + (int64_t)(s * 2 + ks) * (64 * 8));
+        };
+        auto consume = [&](int s, int buf, const u32x4(&ar)[PASSES], const u32x4(&br)[2][2]) {
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const uint32_t keep =
+                    (s * BK + ps * RPP + rrow < u.k_kept && m_ok) ? 0xFFFFFFFFu : 0u;
+                u32x4 v = ar[ps];
+                v.x &= keep;
+                v.y &= keep;
+                v.z &= keep;
+                v.w &= keep;
+                *reinterpret_cast<u32x4 *>(smem + buf * STAGE + (ps * RPP + rrow) * PITCH +
+                                           chunk * 8) = v;
+            }
+            __syncthreads();
+            const uint16_t *stage = smem + buf * STAGE;
 #pragma unroll
             for (int ks = 0; ks < 2; ++ks) {
                 u32x4 af[2];
@@ -248,24 +263,50 @@ __global__ void __launch_bounds__(64 * WM * WN) tw_gemm_kmajor_kernel(const Gemm
                     }
                 }
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni) {
-                    if (wn * 2 + ni < u.nb_cnt) {
+                for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                        for (int mi = 0; mi < 2; ++mi)
-                            acc[mi][ni] = E::mfma(af[mi], b_cur[ks][ni], acc[mi][ni]);
+                    for (int mi = 0; mi < 2; ++mi)
+                        acc[mi][ni] = E::mfma(af[mi], br[ks][ni], acc[mi][ni]);
+            }
+        };
+
+        u32x4 a_ring[R][PASSES];
+        u32x4 b_ring[R][2][2];
+        IdxVec idx[PASSES];
+        if (nsteps > 0)
+            load_idx(0, idx);
+#pragma unroll
+        for (int j = 0; j < D; ++j) {
+            if (j < nsteps) {
+                issue(j, idx, a_ring[j], b_ring[j]);
+                load_idx(j + 1, idx); // the list is padded by one step, so this stays in bounds
+            }
+        }
+        int s0 = 0;
+        // steady state: every slot issues and consumes, no conditionals
+        for (; s0 + R + D <= nsteps; s0 += R) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                issue(s0 + r + D, idx, a_ring[(r + D) % R], b_ring[(r + D) % R]);
+                load_idx(s0 + r + D + 1, idx);
+                consume(s0 + r, r & 1, a_ring[r], b_ring[r]);
+            }
+        }
+        // drain: fewer than R + D steps remain
+        for (; s0 < nsteps; s0 += R) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const int s = s0 + r;
+                if (s < nsteps) {
+                    if (s + D < nsteps) {
+                        issue(s + D, idx, a_ring[(r + D) % R], b_ring[(r + D) % R]);
+                        load_idx(s + D + 1, idx);
                     }
+                    consume(s, r & 1, a_ring[r], b_ring[r]);
                 }
             }
-            if (more) {
-                store_a((s + 1) & 1, a_reg);
-#pragma unroll
-                for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-                        b_cur[ks][ni] = b_nxt[ks][ni];
-            }
-            __syncthreads();
         }
+        __syncthreads();
 
         // ---- epilogue ------------------------------------------------------------
         const int32_t *const nlist = p.kept_n + u.kn_off;
@@ -405,7 +446,7 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     GemmArgs a;
     a.units = plan->d_units;
     a.tiles = plan->d_tiles;
-    a.kept_k = plan->d_kept_k;
+    a.kept_k = plan->d_kept_k_pad;
     a.kept_n = plan->d_kept_n;
     a.pruned_n = plan->d_pruned_n;
     a.Bp = plan->d_Bp;

@@ -29,7 +29,7 @@ struct UnitDev {
     int32_t n_cnt;    // compact columns in this unit
     int32_t nb0;      // first 32-column block of the tile's packed weight used here
     int32_t nb_cnt;   // 32-column blocks in this unit
-    int32_t kk_off;   // offset of the tile's kept_k list
+    int32_t kk_off;   // offset of the tile's kept_k list in the padded array (k_pad entries)
     int32_t kn_off;   // offset of this unit's first compact column in kept_n
     int64_t b_off;    // element offset of the tile's packed weight
     int32_t tile;     // owning tile
@@ -77,6 +77,7 @@ struct tw_plan {
     // device
     int32_t *d_kept_k = nullptr, *d_kept_n = nullptr, *d_rel_k = nullptr, *d_rel_n = nullptr;
     int32_t *d_pruned_n = nullptr;
+    int32_t *d_kept_k_pad = nullptr; // per tile k_pad entries at 4-aligned offsets (kernel's copy)
     tw::UnitDev *d_units = nullptr;
     tw::TileDev *d_tiles = nullptr;
     void *d_Bp = nullptr;

@@ -317,6 +317,7 @@ int finalize_plan_geometry(tw_plan *p)
     std::vector<UnitDev> units;
     std::vector<TileDev> ztiles;
     std::vector<int32_t> pruned_n;
+    std::vector<int32_t> kept_k_pad; // the GEMM kernel's copy: k_pad entries per tile
     p->max_unit_n = 0;
     for (int t = 0; t < nt; ++t) {
         const int kt = p->kept_k_ptr[t + 1] - p->kept_k_ptr[t];
@@ -328,6 +329,11 @@ int finalize_plan_geometry(tw_plan *p)
             p->k_pad[t] = 0;
             p->n_pad[t] = ntk > 0 ? round_up(ntk, kMfmaN) : 0;
         }
+        const int32_t kkp_off = (int32_t)kept_k_pad.size();
+        kept_k_pad.insert(kept_k_pad.end(), p->kept_k_idx.begin() + p->kept_k_ptr[t],
+                          p->kept_k_idx.begin() + p->kept_k_ptr[t + 1]);
+        // one extra step of padding: the kernel prefetches the index list one step ahead
+        kept_k_pad.resize(kkp_off + p->k_pad[t] + kBlockK, 0);
         p->b_off[t] = off;
         off += (int64_t)p->k_pad[t] * p->n_pad[t];
         off = (off + 511) / 512 * 512; // keep every tile 1 KiB aligned
@@ -339,7 +345,7 @@ int finalize_plan_geometry(tw_plan *p)
             u.n_cnt = std::min(kMaxUnitN, ntk - nc0);
             u.nb0 = nc0 / kMfmaN;
             u.nb_cnt = (u.n_cnt + kMfmaN - 1) / kMfmaN;
-            u.kk_off = p->kept_k_ptr[t];
+            u.kk_off = kkp_off;
             u.kn_off = p->kept_n_ptr[t] + nc0;
             u.b_off = p->b_off[t];
             u.tile = t;
@@ -385,7 +391,7 @@ int finalize_plan_geometry(tw_plan *p)
             return st;
     }
     if ((st = upload(&p->d_units, units)) || (st = upload(&p->d_tiles, ztiles)) ||
-        (st = upload(&p->d_pruned_n, pruned_n)))
+        (st = upload(&p->d_pruned_n, pruned_n)) || (st = upload(&p->d_kept_k_pad, kept_k_pad)))
         return st;
     size_t bp_bytes = std::max<int64_t>(p->packed_elems, 8) * 2;
     if (hipMalloc(&p->d_Bp, bp_bytes) != hipSuccess)
@@ -478,6 +484,7 @@ static void free_plan(tw_plan *p)
     hipFree(p->d_rel_k);
     hipFree(p->d_rel_n);
     hipFree(p->d_pruned_n);
+    hipFree(p->d_kept_k_pad);
     hipFree(p->d_units);
     hipFree(p->d_tiles);
     hipFree(p->d_Bp);

@@ -13,8 +13,10 @@
 //     staged in LDS as [k][m];
 //   * the MFMA A operand (32 m x 16 k per instruction, 8 k per lane) is read
 //     from that [k][m] stage with the transposing LDS read ds_read_b64_tr_b16;
-//   * the MFMA B operand comes straight from the packed weight (already in
-//     per-lane operand order, 16 bytes per lane, 1 KiB per wave), no LDS;
+//   * the packed weight is stored per 32-row step in per-lane MFMA operand order; a
+//     step's block is one contiguous run, copied once per workgroup into LDS and read
+//     back 16 bytes per lane (every wave needs it, and the vector-memory path, not
+//     HBM, is what limits a workgroup that fetches its own copy per wave);
 //   * v_mfma_f32_32x32x16_{f16,bf16}, fp32 accumulators;
 //   * epilogue: alpha/beta in fp32, round to the 16-bit type, transpose through
 //     LDS, then scatter whole C columns (col0 + kept_n[j]) with 16-byte stores.
@@ -33,6 +35,10 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 #define TW_LDS(T) __attribute__((address_space(3))) T *
+
+#ifndef TW_A_PAD
+#define TW_A_PAD 16 // halfs of padding per staged A row
+#endif
 
 template <int DT> struct Elem;
 template <> struct Elem<TW_F16> {
@@ -82,28 +88,44 @@ __device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M
     }
 }
 
-template <int DT, int WM, int WN, bool TR>
-__global__ void __launch_bounds__(64 * WM * WN, 2) tw_gemm_kmajor_kernel(const GemmArgs p)
+// WM x WN waves of 64 x 64 outputs each: workgroup tile BM = 64*WM rows by BN = 64*WN
+// compact columns.  WGS is the number of workgroups meant to share a CU.
+// BK k rows are staged per main-loop step (a multiple of 16 that divides kBlockK); the loads
+// of the D steps after the one being multiplied are in flight.
+template <int DT, int WM, int WN, int BK, int D, int WGS>
+__global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
+    tw_gemm_kmajor_kernel(const GemmArgs p)
 {
     constexpr int NT = 64 * WM * WN;
     constexpr int BM = 64 * WM;
     constexpr int BN = 64 * WN;
-    constexpr int BK = kBlockK;
-    constexpr int CPR = BM / 8;       // 16-byte chunks per staged row / stored column
-    constexpr int RPP = NT / CPR;     // rows (columns) covered by one pass of the block
-    constexpr int PASSES = BK / RPP;
-    constexpr int PITCH = BM + 16;    // halfs; +32 B keeps the 4 rows of a transposed read apart
-    constexpr int STAGE = BK * PITCH;
+    constexpr int KS = BK / kMfmaK;      // MFMA k steps per main-loop step
+    constexpr int PKS = kBlockK / kMfmaK; // MFMA k steps per packed weight step
+    constexpr int CPR = BM / 8;          // 16-byte chunks per staged A row / stored C column
+    constexpr int RPP = NT / CPR;        // A rows (C columns) covered by one pass of the block
+    constexpr int PASSES = BK / RPP;     // A loads per thread and step
+    constexpr int BCH = BN * BK / 8;     // 16-byte chunks of packed weight per step
+    constexpr int BPASS = (BCH + NT - 1) / NT;
+    constexpr int PITCH = BM + TW_A_PAD; // halfs; the pad spreads the rows of a transposed read
+    constexpr int ASTAGE = BK * PITCH;
+    constexpr int BSTAGE = BN * BK;
     constexpr int CPITCH = BM + 8;
-    constexpr int SMEM = (2 * STAGE > BN * CPITCH) ? 2 * STAGE : BN * CPITCH;
-    constexpr int D = BM >= 256 ? 2 : 3; // prefetch distance in steps (24-32 KiB of A in flight)
-    constexpr int R = D + 1;         // register ring slots; the main loop is unrolled R times
-    constexpr int RPW = 64 / CPR;    // staged rows covered by one wave in one pass
-    typedef int IdxVec __attribute__((ext_vector_type(RPW)));
+    constexpr int PIPE = 2 * ASTAGE + 2 * BSTAGE;
+    constexpr int SMEM = PIPE > BN * CPITCH ? PIPE : BN * CPITCH;
+    static_assert(NT % CPR == 0 && BK % RPP == 0 && kBlockK % BK == 0, "tile shape");
+    static_assert(BCH % NT == 0 || BCH < NT, "weight chunks per thread");
     using E = Elem<DT>;
 
     __shared__ __align__(16) uint16_t smem[SMEM];
     __shared__ int s_item;
+#ifdef TW_EXP_TIMING
+    __shared__ unsigned long long s_ts[64 * 4];
+#define TW_STAMP(step, slot)                                                              \
+    if (item == 0 && tid == 0 && (step) >= 8 && (step) < 72)                              \
+        s_ts[((step)-8) * 4 + (slot)] = __builtin_readcyclecounter();
+#else
+#define TW_STAMP(step, slot)
+#endif
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -112,11 +134,11 @@ __global__ void __launch_bounds__(64 * WM * WN, 2) tw_gemm_kmajor_kernel(const G
     const int wn = __builtin_amdgcn_readfirstlane(wave / WM);
     const int chunk = tid % CPR;
     const int rrow = tid / CPR;
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int sub = lane / CPR;
     const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
     uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
     const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
+    uint16_t *const sA = smem;
+    uint16_t *const sB = smem + 2 * ASTAGE;
 
     for (;;) {
         if (tid == 0)
@@ -156,20 +178,30 @@ __global__ void __launch_bounds__(64 * WM * WN, 2) tw_gemm_kmajor_kernel(const G
         const int m0 = (item - ui * p.n_mblk) * BM;
         const UnitDev u = p.units[ui];
         const int nsteps = u.k_pad / BK;
-        const int32_t *const klist = p.kept_k + u.kk_off; // padded to k_pad entries
+        const int32_t *const klist = p.kept_k + u.kk_off; // padded past k_pad
         const int m_ld = m0 + chunk * 8;
         const bool m_ok = m_ld < p.M;
         const int m_eff = m_ok ? m_ld : 0; // a valid chunk to read when this one is beyond M
-        const int ksteps16 = u.k_pad / kMfmaK;
-        // packed weight operand streams of this wave's two 32-column blocks; a block
-        // beyond the unit reads block 0 (its products land in columns that are not stored)
-        const uint16_t *b_base[2];
+        // This thread's 16-byte chunks of the step's packed weight.  The weight is packed per
+        // kBlockK rows as ((step, nb, k16, lane)); chunk c of a BK-row step of this kernel is
+        // (nb = c / (KS*64), k16 = (c / 64) % KS, lane = c % 64).  A block beyond the unit
+        // reads block 0 (its products land in columns that are never stored).
+        const uint16_t *b_src[BPASS];
 #pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const int nb = wn * 2 + ni;
-            b_base[ni] = Bp + u.b_off +
-                         ((int64_t)(u.nb0 + (nb < u.nb_cnt ? nb : 0)) * ksteps16 * 64 + lane) * 8;
+        for (int bp = 0; bp < BPASS; ++bp) {
+            const int c = tid + bp * NT;
+            const int nbl = c / (KS * 64);
+            const int k16 = (c >> 6) % KS;
+            b_src[bp] = Bp + u.b_off +
+                        (((int64_t)(u.nb0 + (nbl < u.nb_cnt ? nbl : 0)) * PKS + k16) * 64 +
+                         (c & 63)) * 8;
         }
+        // element strides between consecutive BK-row steps: inside a packed step the k16
+        // index advances, across packed steps the whole block does
+        const int64_t b_pack = (int64_t)u.nblk * (PKS * 64 * 8);
+        auto b_off_of = [&](int s) -> int64_t {
+            return (int64_t)(s / (PKS / KS)) * b_pack + (int64_t)(s % (PKS / KS)) * (KS * 64 * 8);
+        };
 
         f32x16 acc[2][2];
 #pragma unroll
@@ -180,134 +212,157 @@ __global__ void __launch_bounds__(64 * WM * WN, 2) tw_gemm_kmajor_kernel(const G
                 for (int r = 0; r < 16; ++r)
                     acc[mi][ni][r] = 0.0f;
 
-        // Register ring: the loads of step s+D are issued while step s is consumed, so D
-        // steps of gathered A rows (and of packed weight operands) are in flight per
-        // workgroup.  Loads return in order, so A and B share one prefetch distance.
-        // The kept-K indices of a step are wave-uniform per 16-byte-chunk row group and come
-        // through the scalar cache one step ahead of the loads that use them.
-        auto load_idx = [&](int s, IdxVec(&ix)[PASSES]) {
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int kkbase = s * BK + ps * RPP + wave_u * RPW;
-                ix[ps] = *reinterpret_cast<const __attribute__((address_space(4))) IdxVec *>(
-                    (uintptr_t)(klist + kkbase));
-            }
+        // Pipeline over steps of BK rows.  Iteration s issues the global loads of step s+D
+        // into a free register slot, writes the registers of step s (loaded D iterations
+        // ago) to LDS buffer s&1, and after one barrier multiplies step s out of LDS.  So D
+        // steps of gathered A rows and packed weight are in flight per workgroup.
+        // Kept-K indices: every wave fetches the BK indices of a step with one coalesced
+        // load (lane l holds row l of the step) D iterations before the row loads that use
+        // them; loads return in order, so the word has landed by then without an extra wait.
+        // The row loads pick their index out of that register with a cross-lane permute.
+        auto load_idx = [&](int s, int &ix) {
+            ix = klist[s * BK + (lane & (BK - 1))];
+#ifdef TW_EXP_AWINDOW
+            ix &= 63;
+#endif
         };
         // No lane-dependent branches here: rows beyond K_t and chunks beyond M are loaded
         // from a valid address and replaced by zeros when they are staged (not here, so that
         // nothing waits on a load that was just issued).
-        auto issue = [&](int s, const IdxVec(&ix)[PASSES], u32x4(&ar)[PASSES], u32x4(&br)[2][2]) {
+        auto issue = [&](int s, int ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
 #pragma unroll
             for (int ps = 0; ps < PASSES; ++ps) {
-                int my = ix[ps][0];
-#pragma unroll
-                for (int q = 1; q < RPW; ++q)
-                    my = sub == q ? ix[ps][q] : my;
-                ar[ps] = *reinterpret_cast<const u32x4 *>(A + (int64_t)my * p.lda + m_eff);
+                const int row = __builtin_amdgcn_ds_bpermute((ps * RPP + rrow) * 4, ix);
+                ar[ps] = *reinterpret_cast<const u32x4 *>(A + (int64_t)row * p.lda + m_eff);
             }
 #pragma unroll
-            for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-                    br[ks][ni] = *reinterpret_cast<const u32x4 *>(
-                        b_base[ni] + (int64_t)(s * 2 + ks) * (64 * 8));
+            for (int bp = 0; bp < BPASS; ++bp)
+                if (BCH >= NT || tid < BCH)
+                    br[bp] = *reinterpret_cast<const u32x4 *>(b_src[bp] + b_off_of(s));
         };
-        auto consume = [&](int s, int buf, const u32x4(&ar)[PASSES], const u32x4(&br)[2][2]) {
+        auto stage = [&](int s, const u32x4(&ar)[PASSES], const u32x4(&br)[BPASS]) {
+            uint16_t *const stA = sA + (s & 1) * ASTAGE;
+            uint16_t *const stB = sB + (s & 1) * BSTAGE;
+            if (s * BK + BK > u.k_kept || m0 + BM > p.M) {
+                // edge step: rows beyond K_t and chunks beyond M become zeros
 #pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const uint32_t keep =
-                    (s * BK + ps * RPP + rrow < u.k_kept && m_ok) ? 0xFFFFFFFFu : 0u;
-                u32x4 v = ar[ps];
-                v.x &= keep;
-                v.y &= keep;
-                v.z &= keep;
-                v.w &= keep;
-                *reinterpret_cast<u32x4 *>(smem + buf * STAGE + (ps * RPP + rrow) * PITCH +
-                                           chunk * 8) = v;
-            }
-            __syncthreads();
-            const uint16_t *stage = smem + buf * STAGE;
-#pragma unroll
-            for (int ks = 0; ks < 2; ++ks) {
-                u32x4 af[2];
-#pragma unroll
-                for (int mi = 0; mi < 2; ++mi) {
-                    const int mcol = wm * 64 + mi * 32;
-                    if (TR) {
-                        // 16 lanes read a 4(k) x 16(m) block; lane L addresses row L/4,
-                        // columns 4*(L%4)..+3 and receives column L of the 4 rows.
-                        const int L = lane & 15;
-                        const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
-                        const int col = mcol + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
-                        const uint16_t *q = stage + row * PITCH + col;
-                        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
-                        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
-                            (TW_LDS(s16x4))(q + 4 * PITCH));
-                        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-                        af[mi].x = l2.x;
-                        af[mi].y = l2.y;
-                        af[mi].z = h2.x;
-                        af[mi].w = h2.y;
-                    } else {
-                        const uint16_t *q =
-                            stage + (ks * 16 + (lane >> 5) * 8) * PITCH + mcol + (lane & 31);
-                        uint32_t w[4];
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            w[e] = (uint32_t)q[(2 * e) * PITCH] |
-                                   ((uint32_t)q[(2 * e + 1) * PITCH] << 16);
-                        af[mi].x = w[0];
-                        af[mi].y = w[1];
-                        af[mi].z = w[2];
-                        af[mi].w = w[3];
-                    }
+                for (int ps = 0; ps < PASSES; ++ps) {
+                    const uint32_t keep =
+                        (s * BK + ps * RPP + rrow < u.k_kept && m_ok) ? 0xFFFFFFFFu : 0u;
+                    u32x4 v = ar[ps];
+                    v.x &= keep;
+                    v.y &= keep;
+                    v.z &= keep;
+                    v.w &= keep;
+                    *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) = v;
                 }
+            } else {
 #pragma unroll
-                for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-                    for (int mi = 0; mi < 2; ++mi)
-                        acc[mi][ni] = E::mfma(af[mi], br[ks][ni], acc[mi][ni]);
+                for (int ps = 0; ps < PASSES; ++ps)
+                    *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) =
+                        ar[ps];
             }
+#pragma unroll
+            for (int bp = 0; bp < BPASS; ++bp)
+                if (BCH >= NT || tid < BCH)
+                    *reinterpret_cast<u32x4 *>(stB + (tid + bp * NT) * 8) = br[bp];
+        };
+        auto frags = [&](int s, int ks, u32x4(&af)[2], u32x4(&bf)[2]) {
+            const uint16_t *const stA = sA + (s & 1) * ASTAGE;
+            const uint16_t *const stB = sB + (s & 1) * BSTAGE;
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi) {
+                // ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(m) block; lane L addresses
+                // row L/4, columns 4*(L%4)..+3 and receives column L of the 4 rows.
+                const int L = lane & 15;
+                const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
+                const int col = wm * 64 + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
+                const uint16_t *q = stA + row * PITCH + col;
+                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
+                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * PITCH));
+                u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                af[mi].x = l2.x;
+                af[mi].y = l2.y;
+                af[mi].z = h2.x;
+                af[mi].w = h2.y;
+            }
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+                bf[ni] = *reinterpret_cast<const u32x4 *>(
+                    stB + ((((wn * 2 + ni) * KS + ks) * 64) + lane) * 8);
+        };
+        auto mma = [&](const u32x4(&af)[2], const u32x4(&bf)[2]) {
+#ifdef TW_EXP_NOMFMA
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+                    acc[mi][ni][0] += __uint_as_float(af[mi].x ^ bf[ni].x);
+#else
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+                    acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
+#endif
         };
 
+        constexpr int R = D + 1; // register slots: step s being staged plus D steps in flight
         u32x4 a_ring[R][PASSES];
-        u32x4 b_ring[R][2][2];
-        IdxVec idx[PASSES];
-        if (nsteps > 0)
-            load_idx(0, idx);
+        u32x4 b_ring[R][BPASS];
+        int i_ring[R];
+        // one iteration; r == s % R is the register slot of step s
+        auto iteration = [&](int s, int r, bool more_loads) {
+            u32x4 af[2], bf[2];
+            if (more_loads) {
+                load_idx(s + 2 * D, i_ring[(r + 2 * D) % R]); // padded list: stays in bounds
+                issue(s + D, i_ring[(r + D) % R], a_ring[(r + D) % R], b_ring[(r + D) % R]);
+            }
+            TW_STAMP(s, 0)
+            stage(s, a_ring[r], b_ring[r]);
+            TW_STAMP(s, 1)
+            __syncthreads();
+            TW_STAMP(s, 2)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                frags(s, ks, af, bf);
+                mma(af, bf);
+            }
+            TW_STAMP(s, 3)
+        };
+
+#pragma unroll
+        for (int j = 0; j < D; ++j)
+            load_idx(j, i_ring[j % R]);
 #pragma unroll
         for (int j = 0; j < D; ++j) {
             if (j < nsteps) {
-                issue(j, idx, a_ring[j], b_ring[j]);
-                load_idx(j + 1, idx); // the list is padded by one step, so this stays in bounds
+                issue(j, i_ring[j % R], a_ring[j], b_ring[j]);
+                load_idx(j + D, i_ring[(j + D) % R]);
             }
         }
         int s0 = 0;
-        // steady state: every slot issues and consumes, no conditionals
+        // steady state: every iteration issues, stages and multiplies, no conditionals
         for (; s0 + R + D <= nsteps; s0 += R) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                issue(s0 + r + D, idx, a_ring[(r + D) % R], b_ring[(r + D) % R]);
-                load_idx(s0 + r + D + 1, idx);
-                consume(s0 + r, r & 1, a_ring[r], b_ring[r]);
-            }
+            for (int r = 0; r < R; ++r)
+                iteration(s0 + r, r, true);
         }
         // drain: fewer than R + D steps remain
         for (; s0 < nsteps; s0 += R) {
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 const int s = s0 + r;
-                if (s < nsteps) {
-                    if (s + D < nsteps) {
-                        issue(s + D, idx, a_ring[(r + D) % R], b_ring[(r + D) % R]);
-                        load_idx(s + D + 1, idx);
-                    }
-                    consume(s, r & 1, a_ring[r], b_ring[r]);
-                }
+                if (s < nsteps)
+                    iteration(s, r, s + D < nsteps);
             }
         }
         __syncthreads();
 
+#ifdef TW_EXP_TIMING
+        if (item == 0 && tid < 256)
+            reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
+#endif
         // ---- epilogue ------------------------------------------------------------
         const int32_t *const nlist = p.kept_n + u.kn_off;
 #pragma unroll
@@ -395,15 +450,29 @@ static int env_int(const char *name, int dflt)
     return v && *v ? atoi(v) : dflt;
 }
 
-template <int DT, int WM, int WN>
-static void launch_kmajor(const GemmArgs &a, int grid, bool tr, hipStream_t s)
+// Tile shapes: 0: 256 x 128 (8 waves, one workgroup per CU), 1: 128 x 128 (4 waves, two
+// per CU), 2: 512 x 64, 3: 256 x 64 (the two shapes for tiles of at most 64 kept columns).
+struct Shape {
+    int bm, wgs_per_cu;
+};
+static const Shape kShapes[4] = {{256, 1}, {128, 2}, {512, 1}, {256, 2}};
+
+template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int grid, hipStream_t s)
 {
-    if (tr)
-        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, WM, WN, true>), dim3(grid),
-                           dim3(64 * WM * WN), 0, s, a);
-    else
-        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, WM, WN, false>), dim3(grid),
-                           dim3(64 * WM * WN), 0, s, a);
+    switch (shape) {
+    case 0:
+        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 2, 64, 2, 1>), dim3(grid), dim3(512), 0, s, a);
+        break;
+    case 1:
+        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 2, 2, 32, 3, 2>), dim3(grid), dim3(256), 0, s, a);
+        break;
+    case 2:
+        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 8, 1, 32, 2, 1>), dim3(grid), dim3(512), 0, s, a);
+        break;
+    default:
+        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 1, 32, 2, 2>), dim3(grid), dim3(256), 0, s, a);
+        break;
+    }
 }
 
 } // namespace tw
@@ -441,8 +510,20 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR)
         return fail(TW_ERR_LAYOUT, "row-major operands are not implemented yet");
 
+    // Shape choice: the large tile halves the weight traffic per row of A, but needs enough
+    // work items to fill the chip; otherwise the small tile with two workgroups per CU.
     const bool narrow = plan->max_unit_n <= 64;
-    const int BM = narrow ? 256 : 128;
+    int shape = narrow ? 2 : 0;
+    {
+        const int forced = env_int("TWGEMM_SHAPE", -1);
+        const int64_t big_items =
+            (int64_t)plan->n_units * ((M + kShapes[shape].bm - 1) / kShapes[shape].bm);
+        if (forced >= 0 && forced < 4 && (forced >= 2) == narrow)
+            shape = forced;
+        else if (big_items < 2 * (int64_t)plan->cu_count)
+            shape += 1;
+    }
+    const int BM = kShapes[shape].bm;
     GemmArgs a;
     a.units = plan->d_units;
     a.tiles = plan->d_tiles;
@@ -466,25 +547,25 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     const unsigned slot =
         __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kTicketSlots;
     a.ticket = plan->d_tickets + 2 * slot;
+    a.dbg = plan->d_tickets + 2 * kTicketSlots;
 
-    const int per_cu = env_int("TWGEMM_WGS_PER_CU", 2);
-    const int grid = std::min<int64_t>(a.n_items, (int64_t)plan->cu_count * per_cu);
-    const bool tr = env_int("TWGEMM_NO_TR_READ", 0) == 0;
+    const int per_cu = env_int("TWGEMM_WGS_PER_CU", kShapes[shape].wgs_per_cu);
+    const int grid = (int)std::min<int64_t>(a.n_items, (int64_t)plan->cu_count * per_cu);
     hipStream_t s = (hipStream_t)stream;
-    if (plan->dtype == TW_F16) {
-        if (narrow)
-            launch_kmajor<TW_F16, 4, 1>(a, grid, tr, s);
-        else
-            launch_kmajor<TW_F16, 2, 2>(a, grid, tr, s);
-    } else {
-        if (narrow)
-            launch_kmajor<TW_BF16, 4, 1>(a, grid, tr, s);
-        else
-            launch_kmajor<TW_BF16, 2, 2>(a, grid, tr, s);
-    }
+    if (plan->dtype == TW_F16)
+        launch_kmajor<TW_F16>(shape, a, grid, s);
+    else
+        launch_kmajor<TW_BF16>(shape, a, grid, s);
     TW_HIP(hipGetLastError());
     return TW_OK;
 }
+
+#ifdef TW_EXP_TIMING
+int tw_exp_read_debug(const tw_plan *plan, void *host, int nbytes)
+{
+    return hipMemcpy(host, plan->d_tickets + 2 * kTicketSlots, nbytes, hipMemcpyDeviceToHost);
+}
+#endif
 
 int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A, const void *B,
                       float beta, void *C, int block_num, const int32_t *N_cal,

@@ -16,7 +16,7 @@ namespace tw {
 // Geometry shared by the pack kernel and the GEMM kernels.
 constexpr int kMfmaN = 32;    // columns of one MFMA block (packing granularity in n)
 constexpr int kMfmaK = 16;    // k extent of one v_mfma_f32_32x32x16
-constexpr int kBlockK = 32;   // k rows staged per main-loop step; K_t is padded to this
+constexpr int kBlockK = 64;   // k rows per packed weight step; K_t is padded to this
 constexpr int kMaxUnitN = 128; // compact columns handled by one work item
 constexpr int kTicketSlots = 256;
 
@@ -33,7 +33,7 @@ struct UnitDev {
     int32_t kn_off;   // offset of this unit's first compact column in kept_n
     int64_t b_off;    // element offset of the tile's packed weight
     int32_t tile;     // owning tile
-    int32_t pad_;
+    int32_t nblk;     // 32-column blocks of the whole tile (n_pad / 32)
 };
 
 // Zero-fill work for TW_PRUNED_ZERO: the pruned columns of one tile.
@@ -61,6 +61,7 @@ struct GemmArgs {
     int32_t n_zero_tiles; // tiles with pruned columns (first entries of `tiles`)
     float alpha, beta;
     int32_t *ticket;      // [0] next item, [1] finished workgroups
+    void *dbg;            // 2 KiB scratch after the ticket slots (instrumented builds only)
 };
 
 } // namespace tw

@@ -2,12 +2,12 @@
 // offsets -> compaction pre-pass (HIP kernels), the MFMA-ordered weight packing,
 // and the read-back used for bit-exact checks.
 //
-// Packed weight of tile t (K_t x N_t compact, padded to k_pad x n_pad):
-//   for 32-column block nb, 16-row step k16, lane l (0..63), e (0..7):
-//     Bp[b_off + ((nb * (k_pad/16) + k16) * 64 + l) * 8 + e]
-//        = compact[k16*16 + (l/32)*8 + e][nb*32 + l%32]      (0 outside K_t x N_t)
-// i.e. each wave fetches one MFMA B operand with a single 16-byte load per lane,
-// 1 KiB contiguous per wave.
+// Packed weight of tile t (K_t x N_t compact, padded to k_pad x n_pad, nblk = n_pad/32):
+//   for 64-row step s, 32-column block nb, k16 step ks (0..3), lane l (0..63), e (0..7):
+//     Bp[b_off + (((s * nblk + nb) * 4 + ks) * 64 + l) * 8 + e]
+//        = compact[s*64 + ks*16 + (l/32)*8 + e][nb*32 + l%32]      (0 outside K_t x N_t)
+// i.e. one MFMA B operand is 16 bytes per lane, 1 KiB contiguous per wave, and the whole
+// block a 64-row main-loop step needs is one contiguous run of nblk * 4 KiB.
 #include "tw_internal.h"
 
 #include <algorithm>
@@ -15,6 +15,8 @@
 #include <mutex>
 
 namespace tw {
+
+constexpr int kPackKS = kBlockK / kMfmaK; // MFMA k steps per packed step
 
 struct PackTile {
     int32_t col0, k_kept, n_kept, k_pad, n_pad, kk_off, kn_off, pad_;
@@ -55,10 +57,11 @@ __global__ void pack_dense_kernel(const PackTile *tiles, const int32_t *kept_k,
     if (g >= groups)
         return;
     const int lane = (int)(g & 63);
-    const int64_t blk = g >> 6;
-    const int ksteps = t.k_pad / kMfmaK;
-    const int k16 = (int)(blk % ksteps);
-    const int nb = (int)(blk / ksteps);
+    const int64_t blk = g >> 6; // ((step * nblk + nb) * kPackKS + ks)
+    const int nblk = t.n_pad / kMfmaN;
+    const int ks = (int)(blk % kPackKS);
+    const int nb = (int)((blk / kPackKS) % nblk);
+    const int k16 = (int)((blk / kPackKS) / nblk) * kPackKS + ks;
     const int n = nb * kMfmaN + (lane & 31);
     const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
     uint16_t v[8];
@@ -91,10 +94,11 @@ __global__ void pack_stream_kernel(const PackTile *tiles, const uint16_t *Bs, in
     if (g >= groups)
         return;
     const int lane = (int)(g & 63);
-    const int64_t blk = g >> 6;
-    const int ksteps = t.k_pad / kMfmaK;
-    const int k16 = (int)(blk % ksteps);
-    const int nb = (int)(blk / ksteps);
+    const int64_t blk = g >> 6; // ((step * nblk + nb) * kPackKS + ks)
+    const int nblk = t.n_pad / kMfmaN;
+    const int ks = (int)(blk % kPackKS);
+    const int nb = (int)((blk / kPackKS) % nblk);
+    const int k16 = (int)((blk / kPackKS) / nblk) * kPackKS + ks;
     const int n = nb * kMfmaN + (lane & 31);
     const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
     uint16_t v[8];
@@ -120,10 +124,11 @@ __global__ void unpack_stream_kernel(const PackTile *tiles, const uint16_t *Bp, 
     if (g >= groups)
         return;
     const int lane = (int)(g & 63);
-    const int64_t blk = g >> 6;
-    const int ksteps = t.k_pad / kMfmaK;
-    const int k16 = (int)(blk % ksteps);
-    const int nb = (int)(blk / ksteps);
+    const int64_t blk = g >> 6; // ((step * nblk + nb) * kPackKS + ks)
+    const int nblk = t.n_pad / kMfmaN;
+    const int ks = (int)(blk % kPackKS);
+    const int nb = (int)((blk / kPackKS) % nblk);
+    const int k16 = (int)((blk / kPackKS) / nblk) * kPackKS + ks;
     const int n = nb * kMfmaN + (lane & 31);
     const int kk0 = k16 * kMfmaK + (lane >> 5) * 8;
     if (n >= t.n_kept)
@@ -332,8 +337,8 @@ int finalize_plan_geometry(tw_plan *p)
         const int32_t kkp_off = (int32_t)kept_k_pad.size();
         kept_k_pad.insert(kept_k_pad.end(), p->kept_k_idx.begin() + p->kept_k_ptr[t],
                           p->kept_k_idx.begin() + p->kept_k_ptr[t + 1]);
-        // one extra step of padding: the kernel prefetches the index list one step ahead
-        kept_k_pad.resize(kkp_off + p->k_pad[t] + kBlockK, 0);
+        // padding past k_pad: the kernel prefetches the index list up to six 64-row steps ahead
+        kept_k_pad.resize(kkp_off + p->k_pad[t] + 6 * kBlockK, 0);
         p->b_off[t] = off;
         off += (int64_t)p->k_pad[t] * p->n_pad[t];
         off = (off + 511) / 512 * 512; // keep every tile 1 KiB aligned
@@ -349,7 +354,7 @@ int finalize_plan_geometry(tw_plan *p)
             u.kn_off = p->kept_n_ptr[t] + nc0;
             u.b_off = p->b_off[t];
             u.tile = t;
-            u.pad_ = 0;
+            u.nblk = p->n_pad[t] / kMfmaN;
             units.push_back(u);
             p->max_unit_n = std::max(p->max_unit_n, u.n_cnt);
         }
@@ -397,9 +402,9 @@ int finalize_plan_geometry(tw_plan *p)
     if (hipMalloc(&p->d_Bp, bp_bytes) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the packed weight failed", bp_bytes);
     TW_HIP(hipMemset(p->d_Bp, 0, bp_bytes));
-    if (hipMalloc((void **)&p->d_tickets, sizeof(int32_t) * 2 * kTicketSlots) != hipSuccess)
+    if (hipMalloc((void **)&p->d_tickets, sizeof(int32_t) * 2 * kTicketSlots + 2048) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of the ticket slots failed");
-    TW_HIP(hipMemset(p->d_tickets, 0, sizeof(int32_t) * 2 * kTicketSlots));
+    TW_HIP(hipMemset(p->d_tickets, 0, sizeof(int32_t) * 2 * kTicketSlots + 2048));
     hipDeviceProp_t prop;
     TW_HIP(hipGetDevice(&p->device));
     TW_HIP(hipGetDeviceProperties(&prop, p->device));

@@ -18,7 +18,7 @@ import sys
 import numpy as np
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "libtwgemm.so")
+LIB_PATH = os.environ.get("TWGEMM_LIB") or os.path.join(_PKG, "libtwgemm.so")
 
 F16, BF16 = 0, 1
 KMAJOR, ROWMAJOR = 0, 1

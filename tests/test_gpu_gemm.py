@@ -122,6 +122,55 @@ def test_gemm_alpha_beta_and_zero_mode(tw, oracle, dtype):
         assert oracle.rel_error(C, full) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("a_layout,c_layout", [(1, 1), (1, 0), (0, 1)])
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_gemm_row_major_layouts(tw, oracle, a_layout, c_layout, dtype):
+    """Row-major A[M,K] (lda >= K) and/or C[M,N] (ldc >= N) through the layout-generic path."""
+    import torch
+    rng = np.random.default_rng(31 + 2 * a_layout + c_layout)
+    M, K, N, G = 203, 150, 330, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.8, empty_every=3)
+    keep = kept_columns(tiles, N)
+    Ab, Cb = oracle.cast_bits(A, dtype).reshape(M, K), oracle.cast_bits(C0, dtype).reshape(M, N)
+    if a_layout == tw.ROWMAJOR:
+        lda = round_up(K, 8) + 8
+        Ah = np.zeros((M, lda), np.uint16)
+        Ah[:, :K] = Ab
+    else:
+        lda = round_up(M, 8)
+        Ah = np.zeros((K, lda), np.uint16)
+        Ah[:, :M] = Ab.T
+    for alpha, beta, pruned in ((1.0, 0.0, tw.PRUNED_UNTOUCHED), (0.5, 2.0, tw.PRUNED_ZERO)):
+        if c_layout == tw.ROWMAJOR:
+            ldc = round_up(N, 8) + 8
+            Ch = np.full((M, ldc), SENTINEL, np.uint16)
+            Ch[:, :N] = Cb
+        else:
+            ldc = round_up(M, 8)
+            Ch = np.full((N, ldc), SENTINEL, np.uint16)
+            Ch[:, :M] = Cb.T
+        dA, dC = to_device_bits(Ah, Ah.shape), to_device_bits(Ch, Ch.shape)
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
+                      a_layout=a_layout, c_layout=c_layout, pruned_cols=pruned)
+            torch.cuda.synchronize()
+        out = from_device_bits(dC)
+        got = out[:, :N] if c_layout == tw.ROWMAJOR else out[:, :M].T
+        pad = out[:, N:] if c_layout == tw.ROWMAJOR else out[:, M:]
+        assert np.all(pad == SENTINEL)
+        Cf = oracle.bits_to_f32(np.ascontiguousarray(got), dtype).reshape(M, N)
+        ref = reference(oracle, A, B, tiles, dtype, alpha, beta, C0)
+        assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
+        if pruned == tw.PRUNED_UNTOUCHED:
+            assert np.array_equal(np.ascontiguousarray(got)[:, ~keep], Cb[:, ~keep])
+        else:
+            expect = oracle.cast_bits(beta * oracle.quantize(C0, dtype)[:, ~keep], dtype)
+            assert np.array_equal(np.ascontiguousarray(got)[:, ~keep], expect.reshape(M, -1))
+
+
 def test_gemm_degenerate_plans(tw, oracle):
     rng = np.random.default_rng(22)
     M, K, N, G = 96, 64, 256, 128

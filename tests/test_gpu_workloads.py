@@ -1,0 +1,98 @@
+"""The five benchmark configurations on the GPU, at full size where memory allows.
+
+At full size the oracle is evaluated on a sample of rows (a row of C depends on the same
+row of A only, so C[rows] = A[rows] @ (B (.) mask) is exact for the sample), and
+size-independent properties are checked on the whole result: pruned columns untouched,
+linearity in A, and agreement of the two kernel shapes.
+"""
+import numpy as np
+import pytest
+
+from tests.helpers import from_device_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f16": 1e-2, "bf16": 2e-2}
+
+
+def run(tw, wl, A_dev, M, plan, alpha=1.0):
+    import torch
+    C = torch.full((wl["N"], M), 0x1234, dtype=torch.int16, device="cuda")
+    plan.gemm(A_dev.data_ptr(), C.data_ptr(), M, alpha=alpha,
+              stream=torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    return C
+
+
+def check_workload(tw, oracle, wl, sample_rows=96):
+    import torch
+    M, K, N, dtype, tiles = wl["M"], wl["K"], wl["N"], wl["dtype"], wl["tiles"]
+    A, B = wl["values"]()
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    At = torch.from_numpy(A).cuda().to(tdt).t().contiguous()
+    keep = np.zeros(N, bool)
+    for t in tiles:
+        keep[np.asarray(t["kept_n"], np.int64) + t["col0"]] = True
+    rng = np.random.default_rng(wl["seed"])
+    rows = np.sort(rng.choice(M, size=min(sample_rows, M), replace=False))
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        C = run(tw, wl, At, M, plan)
+        bits = from_device_bits(C)
+        got = oracle.bits_to_f32(np.ascontiguousarray(bits[:, rows]), dtype).reshape(N, rows.size).T
+        Aq = oracle.bits_to_f32(from_device_bits(At.view(torch.int16)[:, rows].contiguous()), dtype)
+        ref = oracle.tw_gemm_reference(Aq.reshape(K, rows.size).T, oracle.quantize(B, dtype), tiles)
+        err = oracle.rel_error(got[:, keep], ref[:, keep])
+        assert err <= TOL[dtype], (wl["name"], err)
+        assert np.all(bits[~keep] == 0x1234), "pruned columns were written"
+        # linearity: tw_gemm(2A) == 2 tw_gemm(A) exactly (scaling by 2 is exact in fp16/bf16)
+        C2 = run(tw, wl, At * 2, M, plan)
+        a = oracle.bits_to_f32(from_device_bits(C)[keep][:, :4096].copy(), dtype)
+        b = oracle.bits_to_f32(from_device_bits(C2)[keep][:, :4096].copy(), dtype)
+        fin = np.isfinite(b) & (np.abs(a) > 1e-3)
+        assert np.array_equal((2 * a)[fin], b[fin])
+    return err
+
+
+def test_config1_bert_base_ffn(tw, oracle):
+    from tilesparsity_amd import workloads as W
+    check_workload(tw, oracle, W.bert_base_ffn())
+
+
+def test_config2_vgg16_conv4_2(tw, oracle):
+    from tilesparsity_amd import workloads as W
+    check_workload(tw, oracle, W.vgg16_conv4_2())
+
+
+def test_config3_nmt_lstm_gates_50_steps(tw, oracle):
+    """Fixed plan, 50 back-to-back steps: every step must reproduce the first bit for bit."""
+    import torch
+    from tilesparsity_amd import workloads as W
+    wl = W.nmt_lstm_gates()
+    check_workload(tw, oracle, wl, sample_rows=128)
+    A, B = wl["values"]()
+    At = torch.from_numpy(A).cuda().half().t().contiguous()
+    with tw.Plan.create(wl["K"], wl["N"], "f16", wl["tiles"], B) as plan:
+        first = from_device_bits(run(tw, wl, At, wl["M"], plan))
+        C = torch.zeros((wl["N"], wl["M"]), dtype=torch.int16, device="cuda")
+        for _ in range(50):
+            plan.gemm(At.data_ptr(), C.data_ptr(), wl["M"],
+                      stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        assert np.array_equal(from_device_bits(C), first)
+
+
+@pytest.mark.parametrize("which,keep", [(1, 0.5), (1, 0.25), (1, 0.10), (2, 0.5), (2, 0.25), (2, 0.10)])
+def test_config4_bert_large_ffn_bf16(tw, oracle, which, keep):
+    from tilesparsity_amd import workloads as W
+    wl = W.bert_large_ffn(which, keep)
+    K = wl["K"]
+    assert all(len(t["kept_k"]) == int(np.floor(keep * K + 0.5)) for t in wl["tiles"])
+    check_workload(tw, oracle, wl)
+
+
+def test_config5_imbalance_stress(tw, oracle):
+    from tilesparsity_amd import workloads as W
+    wl = W.imbalance_stress()
+    kts = [len(t["kept_k"]) for t in wl["tiles"]]
+    assert kts.count(0) >= 13 and max(kts) > 2500      # empty tiles and near-dense tiles
+    check_workload(tw, oracle, wl)

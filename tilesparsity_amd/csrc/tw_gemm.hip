@@ -37,7 +37,8 @@ typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 #define TW_LDS(T) __attribute__((address_space(3))) T *
 
 #ifndef TW_A_PAD
-#define TW_A_PAD 16 // halfs of padding per staged A row
+#define TW_A_PAD 32 // halfs of padding per staged A row: 64 B, so that the 4 rows x 2 column
+                    // halves one transposed read touches fall into 8 distinct 32-byte bank groups
 #endif
 
 template <int DT> struct Elem;
@@ -415,6 +416,127 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 }
 
 // ---------------------------------------------------------------------------------
+// Layout-generic kernel: any combination of K-major / row-major A and C through element
+// strides.  One workgroup (4 waves, 128 x 128 tile, 32-row steps) per work item in queue
+// order, single-buffered.  Gathered A elements are fetched one by one with the lanes running
+// along the kept-K list (for row-major A the 32 kept columns of a row sit within a few cache
+// lines), staged as [m][k] so that an MFMA operand is a plain 16-byte LDS read.  This is the
+// functional path for the layouts the pipelined K-major kernel does not take.
+template <int DT>
+__global__ void __launch_bounds__(256, 2) tw_gemm_generic_kernel(const GemmArgs p, int64_t sa_m,
+                                                                  int64_t sa_k, int64_t sc_m,
+                                                                  int64_t sc_n)
+{
+    constexpr int BM = 128, BK = 32, KP = BK + 8; // halfs per staged row (80 B)
+    constexpr int PKS = kBlockK / kMfmaK;
+    constexpr int CP = BM + 8;
+    using E = Elem<DT>;
+    __shared__ __align__(16) uint16_t smem[128 * CP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave & 1, wn = wave >> 1;
+    const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
+    uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
+    const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
+    const int item = blockIdx.x;
+
+    if (item >= p.n_gemm_items) { // zero-fill item: pruned columns receive beta*C
+        const int z = item - p.n_gemm_items;
+        const int zt = z / p.n_mblk;
+        const int m0 = (z - zt * p.n_mblk) * BM;
+        const TileDev t = p.tiles[zt];
+        for (int e = tid; e < t.n_pruned * BM; e += 256) {
+            const int j = e % t.n_pruned, m = m0 + e / t.n_pruned;
+            if (m < p.M) {
+                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)(t.col0 + p.pruned_n[t.pn_off + j]) * sc_n;
+                *dst = p.beta != 0.0f ? (uint16_t)E::to_bits(p.beta * E::from_bits(*dst)) : (uint16_t)0;
+            }
+        }
+        return;
+    }
+    const int ui = item / p.n_mblk;
+    const int m0 = (item - ui * p.n_mblk) * BM;
+    const UnitDev u = p.units[ui];
+    const int32_t *const klist = p.kept_k + u.kk_off;
+    const int32_t *const nlist = p.kept_n + u.kn_off;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+        for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[mi][ni][r] = 0.0f;
+
+    const int kk_l = tid & 31, m_l = tid >> 5; // this thread stages column kk_l of rows m_l + 8 i
+    for (int s = 0; s < u.k_pad / BK; ++s) {
+        const int kk = s * BK + kk_l;
+        const bool k_ok = kk < u.k_kept;
+        const int64_t koff = k_ok ? (int64_t)klist[kk] * sa_k : 0;
+#pragma unroll 4
+        for (int i = 0; i < BM / 8; ++i) {
+            const int ml = m_l + 8 * i;
+            uint16_t v = 0;
+            if (k_ok && m0 + ml < p.M)
+                v = A[(int64_t)(m0 + ml) * sa_m + koff];
+            smem[ml * KP + kk_l] = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+            u32x4 af[2], bf[2];
+#pragma unroll
+            for (int mi = 0; mi < 2; ++mi)
+                af[mi] = *reinterpret_cast<const u32x4 *>(
+                    smem + (wm * 64 + mi * 32 + (lane & 31)) * KP + ks * 16 + (lane >> 5) * 8);
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                const int nb = wn * 2 + ni;
+                const int k16 = s * 2 + ks; // 16-row step; the weight is packed per kBlockK rows
+                bf[ni] = *reinterpret_cast<const u32x4 *>(
+                    Bp + u.b_off +
+                    ((((int64_t)(k16 / PKS) * u.nblk + u.nb0 + (nb < u.nb_cnt ? nb : 0)) * PKS +
+                      (k16 % PKS)) * 64 + lane) * 8);
+            }
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+                    acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
+        }
+        __syncthreads();
+    }
+    // epilogue: stage alpha*acc as fp32-rounded 16-bit [j][m], then strided stores
+    float *const sF = reinterpret_cast<float *>(smem); // 64 columns x 128 rows of fp32 per half
+    for (int half = 0; half < 2; ++half) {
+        if (wn == half) {
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const int jl = ni * 32 + (lane & 31);
+                        const int ml = wm * 64 + mi * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                        sF[jl * (BM + 1) + ml] = acc[mi][ni][r];
+                    }
+        }
+        __syncthreads();
+        for (int e = tid; e < 64 * BM; e += 256) {
+            const int jl = e & 63, ml = e >> 6;
+            const int j = half * 64 + jl, m = m0 + ml;
+            if (j < u.n_cnt && m < p.M) {
+                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)(u.col0 + nlist[j]) * sc_n;
+                float v = p.alpha * sF[jl * (BM + 1) + ml];
+                if (p.beta != 0.0f)
+                    v += p.beta * E::from_bits(*dst);
+                *dst = (uint16_t)E::to_bits(v);
+            }
+        }
+        __syncthreads();
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // small elementwise kernels of the boundary
 
 __global__ void cast_f32_kernel(const float *src, uint16_t *dst, int64_t n, int dtype)
@@ -507,8 +629,43 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
                     (long long)lda, (long long)ldc);
     if (((uintptr_t)A & 15) || ((uintptr_t)C & 15))
         return fail(TW_ERR_ALIGNMENT, "A and C must be 16-byte aligned");
-    if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR)
-        return fail(TW_ERR_LAYOUT, "row-major operands are not implemented yet");
+    if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR) {
+        // layout-generic path (element strides), 128-row blocks, one workgroup per item
+        GemmArgs a;
+        a.units = plan->d_units;
+        a.tiles = plan->d_tiles;
+        a.kept_k = plan->d_kept_k_pad;
+        a.kept_n = plan->d_kept_n;
+        a.pruned_n = plan->d_pruned_n;
+        a.Bp = plan->d_Bp;
+        a.A = A;
+        a.C = C;
+        a.lda = lda;
+        a.ldc = ldc;
+        a.M = M;
+        a.n_mblk = (M + 127) / 128;
+        a.n_gemm_items = plan->n_units * a.n_mblk;
+        a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
+        a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
+        a.alpha = alpha;
+        a.beta = beta;
+        a.ticket = nullptr;
+        a.dbg = nullptr;
+        if (a.n_items == 0)
+            return TW_OK;
+        const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
+        const int64_t sa_k = a_layout == TW_LAYOUT_KMAJOR ? lda : 1;
+        const int64_t sc_m = c_layout == TW_LAYOUT_KMAJOR ? 1 : ldc;
+        const int64_t sc_n = c_layout == TW_LAYOUT_KMAJOR ? ldc : 1;
+        if (plan->dtype == TW_F16)
+            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_F16>), dim3(a.n_items), dim3(256), 0,
+                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
+        else
+            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_BF16>), dim3(a.n_items), dim3(256), 0,
+                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
+        TW_HIP(hipGetLastError());
+        return TW_OK;
+    }
 
     // Shape choice: the large tile halves the weight traffic per row of A, but needs enough
     // work items to fill the chip; otherwise the small tile with two workgroups per CU.
@@ -520,8 +677,8 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
             (int64_t)plan->n_units * ((M + kShapes[shape].bm - 1) / kShapes[shape].bm);
         if (forced >= 0 && forced < 4 && (forced >= 2) == narrow)
             shape = forced;
-        else if (big_items < 2 * (int64_t)plan->cu_count)
-            shape += 1;
+        else if (big_items * 5 < 3 * (int64_t)plan->cu_count)
+            shape += 1; // too few large items to occupy the chip
     }
     const int BM = kShapes[shape].bm;
     GemmArgs a;

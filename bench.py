@@ -138,6 +138,10 @@ def main():
     ap.add_argument("--workload", default="vgg16_conv4_2")
     ap.add_argument("--all", action="store_true", help="also run the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB device copy (4 launches over rotating buffers), "
+                         "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
+                         "the same counters show for a copy of known size")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine and this benchmark use exactly one GPU; "
@@ -149,6 +153,17 @@ def main():
         return 1
     from tilesparsity_amd import twgemm as tw
     tw.lib()  # fails loudly if the HIP library has not been built
+
+    if args.copy_calibration:
+        n = (256 << 20) // 4
+        srcs = [torch.full((n,), float(i), dtype=torch.float32, device="cuda") for i in range(4)]
+        dsts = [torch.empty_like(x) for x in srcs]
+        torch.cuda.synchronize()
+        for x, y in zip(srcs, dsts):          # each source was written long ago: it comes from HBM
+            y.copy_(x)
+        torch.cuda.synchronize()
+        del srcs, dsts
+        torch.cuda.empty_cache()
 
     wl = make_workload(args.workload)
     res, (A, B) = run_workload(wl, args.steps, args.warmup, torch)

@@ -65,11 +65,7 @@ template <> struct Elem<TW_BF16> {
     }
     static __device__ __forceinline__ uint32_t to_bits(float f)
     {
-        uint32_t x = __float_as_uint(f);
-        if ((x & 0x7F800000u) == 0x7F800000u && (x & 0x007FFFFFu))
-            return (x >> 16) | 0x0040u;
-        x += 0x7FFFu + ((x >> 16) & 1u);
-        return x >> 16;
+        return __builtin_bit_cast(uint16_t, (__bf16)f); // v_cvt_pk_bf16_f32, nearest even
     }
     static __device__ __forceinline__ float from_bits(uint16_t h)
     {
@@ -110,7 +106,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     constexpr int PITCH = BM + TW_A_PAD; // halfs; the pad spreads the rows of a transposed read
     constexpr int ASTAGE = BK * PITCH;
     constexpr int BSTAGE = BN * BK;
-    constexpr int CPITCH = BM + 8;
+    constexpr int CPITCH = BM + 4;       // halfs; 8-byte accumulator writes of 32 lanes (one
+                                         // column each) then fall into 32 distinct bank pairs
     constexpr int PIPE = 2 * ASTAGE + 2 * BSTAGE;
     constexpr int SMEM = PIPE > BN * CPITCH ? PIPE : BN * CPITCH;
     static_assert(NT % CPR == 0 && BK % RPP == 0 && kBlockK % BK == 0, "tile shape");
@@ -118,14 +115,18 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     using E = Elem<DT>;
 
     __shared__ __align__(16) uint16_t smem[SMEM];
-    __shared__ int s_item;
+    __shared__ int s_tk[2];
 #ifdef TW_EXP_TIMING
     __shared__ unsigned long long s_ts[64 * 4];
 #define TW_STAMP(step, slot)                                                              \
     if (item == 0 && tid == 0 && (step) >= 8 && (step) < 72)                              \
         s_ts[((step)-8) * 4 + (slot)] = __builtin_readcyclecounter();
+#define TW_PHASE(k)                                                                       \
+    if (blockIdx.x == 0 && tid == 0 && n_done_items < 2)                                  \
+        s_ts[240 + n_done_items * 8 + (k)] = __builtin_readcyclecounter();
 #else
 #define TW_STAMP(step, slot)
+#define TW_PHASE(k)
 #endif
 
     const int tid = threadIdx.x;
@@ -141,14 +142,128 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     uint16_t *const sA = smem;
     uint16_t *const sB = smem + 2 * ASTAGE;
 
-    for (;;) {
-        if (tid == 0)
-            s_item = atomicAdd(&p.ticket[0], 1);
-        __syncthreads();
-        const int item = s_item;
-        if (item >= p.n_items)
-            break;
+    // ---- work items ----------------------------------------------------------------
+    // A ticket names an item: tickets below n_pipe_items are GEMM items with at least one
+    // step, then come GEMM items of units that keep no K row (their kept columns receive
+    // alpha*0 + beta*C), then the zero-fill items.  The workgroup always holds the ticket
+    // of its current and its next item and has the atomic for the one after in flight, so
+    // a ticket's round trip is hidden behind a whole item.
+    struct Item {
+        int ticket;
+        int m0;
+        UnitDev u; // valid for ticket < n_gemm_items
+    };
+    auto make_item = [&](int ticket) {
+        Item it;
+        it.ticket = ticket;
+        it.m0 = 0;
+        if (ticket < p.n_gemm_items) {
+            const int ui = ticket / p.n_mblk;
+            it.m0 = (ticket - ui * p.n_mblk) * BM;
+            it.u = p.units[ui];
+        }
+        return it;
+    };
+    // per-thread addressing of an item
+    struct Thr {
+        const int32_t *klist;
+        const uint16_t *b_src[BPASS];
+        int64_t b_pack;
+        int m_ld, m_eff;
+        bool m_ok;
+    };
+    auto setup = [&](const Item &it) {
+        Thr t;
+        t.klist = p.kept_k + it.u.kk_off; // padded past k_pad
+        t.m_ld = it.m0 + chunk * 8;
+        t.m_ok = t.m_ld < p.M;
+        t.m_eff = t.m_ok ? t.m_ld : 0; // a valid chunk to read when this one is beyond M
+        // This thread's 16-byte chunks of a step's packed weight.  The weight is packed per
+        // kBlockK rows as (step, nb, k16, lane); chunk c of a BK-row step of this kernel is
+        // (nb = c / (KS*64), k16 = (c / 64) % KS, lane = c % 64).  A block beyond the unit
+        // reads block 0 (its products land in columns that are never stored).
+#pragma unroll
+        for (int bp = 0; bp < BPASS; ++bp) {
+            const int c = tid + bp * NT;
+            const int nbl = c / (KS * 64);
+            const int k16 = (c >> 6) % KS;
+            t.b_src[bp] = Bp + it.u.b_off +
+                          (((int64_t)(it.u.nb0 + (nbl < it.u.nb_cnt ? nbl : 0)) * PKS + k16) * 64 +
+                           (c & 63)) * 8;
+        }
+        t.b_pack = (int64_t)it.u.nblk * (PKS * 64 * 8);
+        return t;
+    };
 
+    // Kept-K indices: every wave fetches the BK indices of a step with one coalesced load
+    // (lane l holds row l of the step) D iterations before the row loads that use them;
+    // loads return in order, so the word has landed by then without an extra wait.  The row
+    // loads pick their index out of that register with a cross-lane permute.
+    auto load_idx = [&](const Thr &t, int s, int &ix) {
+        ix = t.klist[s * BK + (lane & (BK - 1))];
+#ifdef TW_EXP_AWINDOW
+        ix &= 63;
+#endif
+    };
+    // No lane-dependent branches here: rows beyond K_t and chunks beyond M are loaded from a
+    // valid address and replaced by zeros when they are staged (not here, so that nothing
+    // waits on a load that was just issued).
+    auto issue = [&](const Thr &t, int s, int ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ++ps) {
+            const int row = __builtin_amdgcn_ds_bpermute((ps * RPP + rrow) * 4, ix);
+            ar[ps] = *reinterpret_cast<const u32x4 *>(A + (int64_t)row * p.lda + t.m_eff);
+        }
+        // element offset of step s: inside a packed step the k16 index advances, across
+        // packed steps the whole block does
+        const int64_t boff =
+            (int64_t)(s / (PKS / KS)) * t.b_pack + (int64_t)(s % (PKS / KS)) * (KS * 64 * 8);
+#pragma unroll
+        for (int bp = 0; bp < BPASS; ++bp)
+            if (BCH >= NT || tid < BCH)
+                br[bp] = *reinterpret_cast<const u32x4 *>(t.b_src[bp] + boff);
+    };
+
+    constexpr int R = D + 1; // register slots: the step being staged plus D steps in flight
+    u32x4 a_ring[R][PASSES];
+    u32x4 b_ring[R][BPASS];
+    int i_ring[R];
+    int n_idx[2 * D]; // index words of the next item's first 2 D steps
+
+    // The first item of a workgroup is its block index; later ones are claimed from the
+    // shared counter (which starts at 0 for every launch) one item ahead, with the atomic of
+    // the claim after that already in flight.
+    const int ticket_base = gridDim.x;
+    int t_pending = 0; // thread 0: claim in flight
+    if (tid == 0)
+        t_pending = atomicAdd(&p.ticket[0], 1);
+    Item cur = make_item(blockIdx.x);
+    Item nxt = cur;
+    bool have_next = false; // nxt is known for the current item
+    // Publishes the claim in flight as the next item and starts the claim after it.
+    auto claim_next = [&]() {
+        if (tid == 0) {
+            s_tk[0] = ticket_base + t_pending;
+            t_pending = atomicAdd(&p.ticket[0], 1);
+        }
+        __syncthreads();
+        // tickets are workgroup-uniform: keep them, and everything derived from them, scalar
+        nxt = make_item(__builtin_amdgcn_readfirstlane(s_tk[0]));
+        have_next = true;
+        __syncthreads();
+    };
+    bool preloaded = false; // cur's first D steps are already in flight, i_ring holds D..2D-1
+
+    bool first = true;
+    int n_done_items = 0;
+    while (cur.ticket < p.n_items) {
+        const int item = cur.ticket;
+        TW_PHASE(0)
+        // the very first claim of a workgroup is published after the first item's loads have
+        // been issued, so that its round trip overlaps with them
+        if (!first || item >= p.n_pipe_items)
+            claim_next();
+        first = false;
         if (item >= p.n_gemm_items) {
             // ---- zero-fill item: pruned columns of one tile receive beta*C ----
             const int z = item - p.n_gemm_items;
@@ -170,243 +285,241 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 }
                 store_chunk(dst, v, m, p.M);
             }
-            __syncthreads();
-            continue;
-        }
+        } else {
+            // ---- GEMM item ------------------------------------------------------
+            const UnitDev &u = cur.u;
+            const int m0 = cur.m0;
+            const int nsteps = u.k_pad / BK;
+            const Thr tc = setup(cur);
 
-        // ---- GEMM item ----------------------------------------------------------
-        const int ui = item / p.n_mblk;
-        const int m0 = (item - ui * p.n_mblk) * BM;
-        const UnitDev u = p.units[ui];
-        const int nsteps = u.k_pad / BK;
-        const int32_t *const klist = p.kept_k + u.kk_off; // padded past k_pad
-        const int m_ld = m0 + chunk * 8;
-        const bool m_ok = m_ld < p.M;
-        const int m_eff = m_ok ? m_ld : 0; // a valid chunk to read when this one is beyond M
-        // This thread's 16-byte chunks of the step's packed weight.  The weight is packed per
-        // kBlockK rows as ((step, nb, k16, lane)); chunk c of a BK-row step of this kernel is
-        // (nb = c / (KS*64), k16 = (c / 64) % KS, lane = c % 64).  A block beyond the unit
-        // reads block 0 (its products land in columns that are never stored).
-        const uint16_t *b_src[BPASS];
+            f32x16 acc[2][2];
 #pragma unroll
-        for (int bp = 0; bp < BPASS; ++bp) {
-            const int c = tid + bp * NT;
-            const int nbl = c / (KS * 64);
-            const int k16 = (c >> 6) % KS;
-            b_src[bp] = Bp + u.b_off +
-                        (((int64_t)(u.nb0 + (nbl < u.nb_cnt ? nbl : 0)) * PKS + k16) * 64 +
-                         (c & 63)) * 8;
-        }
-        // element strides between consecutive BK-row steps: inside a packed step the k16
-        // index advances, across packed steps the whole block does
-        const int64_t b_pack = (int64_t)u.nblk * (PKS * 64 * 8);
-        auto b_off_of = [&](int s) -> int64_t {
-            return (int64_t)(s / (PKS / KS)) * b_pack + (int64_t)(s % (PKS / KS)) * (KS * 64 * 8);
-        };
+            for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[mi][ni][r] = 0.0f;
 
-        f32x16 acc[2][2];
+            // Pipeline over steps of BK rows.  Iteration s issues the global loads of step
+            // s+D into a free register slot, writes the registers of step s (loaded D
+            // iterations ago) to LDS buffer s&1, and after one barrier multiplies step s out
+            // of LDS.  So D steps of gathered A rows and packed weight are in flight.
+            auto stage = [&](int s, const u32x4(&ar)[PASSES], const u32x4(&br)[BPASS]) {
+                uint16_t *const stA = sA + (s & 1) * ASTAGE;
+                uint16_t *const stB = sB + (s & 1) * BSTAGE;
+                if (s * BK + BK > u.k_kept || m0 + BM > p.M) {
+                    // edge step: rows beyond K_t and chunks beyond M become zeros
 #pragma unroll
-        for (int mi = 0; mi < 2; ++mi)
+                    for (int ps = 0; ps < PASSES; ++ps) {
+                        const uint32_t keep =
+                            (s * BK + ps * RPP + rrow < u.k_kept && tc.m_ok) ? 0xFFFFFFFFu : 0u;
+                        u32x4 v = ar[ps];
+                        v.x &= keep;
+                        v.y &= keep;
+                        v.z &= keep;
+                        v.w &= keep;
+                        *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) = v;
+                    }
+                } else {
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    acc[mi][ni][r] = 0.0f;
-
-        // Pipeline over steps of BK rows.  Iteration s issues the global loads of step s+D
-        // into a free register slot, writes the registers of step s (loaded D iterations
-        // ago) to LDS buffer s&1, and after one barrier multiplies step s out of LDS.  So D
-        // steps of gathered A rows and packed weight are in flight per workgroup.
-        // Kept-K indices: every wave fetches the BK indices of a step with one coalesced
-        // load (lane l holds row l of the step) D iterations before the row loads that use
-        // them; loads return in order, so the word has landed by then without an extra wait.
-        // The row loads pick their index out of that register with a cross-lane permute.
-        auto load_idx = [&](int s, int &ix) {
-            ix = klist[s * BK + (lane & (BK - 1))];
-#ifdef TW_EXP_AWINDOW
-            ix &= 63;
-#endif
-        };
-        // No lane-dependent branches here: rows beyond K_t and chunks beyond M are loaded
-        // from a valid address and replaced by zeros when they are staged (not here, so that
-        // nothing waits on a load that was just issued).
-        auto issue = [&](int s, int ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps) {
-                const int row = __builtin_amdgcn_ds_bpermute((ps * RPP + rrow) * 4, ix);
-                ar[ps] = *reinterpret_cast<const u32x4 *>(A + (int64_t)row * p.lda + m_eff);
-            }
-#pragma unroll
-            for (int bp = 0; bp < BPASS; ++bp)
-                if (BCH >= NT || tid < BCH)
-                    br[bp] = *reinterpret_cast<const u32x4 *>(b_src[bp] + b_off_of(s));
-        };
-        auto stage = [&](int s, const u32x4(&ar)[PASSES], const u32x4(&br)[BPASS]) {
-            uint16_t *const stA = sA + (s & 1) * ASTAGE;
-            uint16_t *const stB = sB + (s & 1) * BSTAGE;
-            if (s * BK + BK > u.k_kept || m0 + BM > p.M) {
-                // edge step: rows beyond K_t and chunks beyond M become zeros
-#pragma unroll
-                for (int ps = 0; ps < PASSES; ++ps) {
-                    const uint32_t keep =
-                        (s * BK + ps * RPP + rrow < u.k_kept && m_ok) ? 0xFFFFFFFFu : 0u;
-                    u32x4 v = ar[ps];
-                    v.x &= keep;
-                    v.y &= keep;
-                    v.z &= keep;
-                    v.w &= keep;
-                    *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) = v;
+                    for (int ps = 0; ps < PASSES; ++ps)
+                        *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) =
+                            ar[ps];
                 }
-            } else {
 #pragma unroll
-                for (int ps = 0; ps < PASSES; ++ps)
-                    *reinterpret_cast<u32x4 *>(stA + (ps * RPP + rrow) * PITCH + chunk * 8) =
-                        ar[ps];
-            }
+                for (int bp = 0; bp < BPASS; ++bp)
+                    if (BCH >= NT || tid < BCH)
+                        *reinterpret_cast<u32x4 *>(stB + (tid + bp * NT) * 8) = br[bp];
+            };
+            auto frags = [&](int s, int ks, u32x4(&af)[2], u32x4(&bf)[2]) {
+                const uint16_t *const stA = sA + (s & 1) * ASTAGE;
+                const uint16_t *const stB = sB + (s & 1) * BSTAGE;
 #pragma unroll
-            for (int bp = 0; bp < BPASS; ++bp)
-                if (BCH >= NT || tid < BCH)
-                    *reinterpret_cast<u32x4 *>(stB + (tid + bp * NT) * 8) = br[bp];
-        };
-        auto frags = [&](int s, int ks, u32x4(&af)[2], u32x4(&bf)[2]) {
-            const uint16_t *const stA = sA + (s & 1) * ASTAGE;
-            const uint16_t *const stB = sB + (s & 1) * BSTAGE;
+                for (int mi = 0; mi < 2; ++mi) {
+                    // ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(m) block; lane L addresses
+                    // row L/4, columns 4*(L%4)..+3 and receives column L of the 4 rows.
+                    const int L = lane & 15;
+                    const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
+                    const int col = wm * 64 + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
+                    const uint16_t *q = stA + row * PITCH + col;
+                    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
+                    s16x4 hi =
+                        __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * PITCH));
+                    u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                    af[mi].x = l2.x;
+                    af[mi].y = l2.y;
+                    af[mi].z = h2.x;
+                    af[mi].w = h2.y;
+                }
 #pragma unroll
-            for (int mi = 0; mi < 2; ++mi) {
-                // ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(m) block; lane L addresses
-                // row L/4, columns 4*(L%4)..+3 and receives column L of the 4 rows.
-                const int L = lane & 15;
-                const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
-                const int col = wm * 64 + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
-                const uint16_t *q = stA + row * PITCH + col;
-                s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
-                s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * PITCH));
-                u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
-                af[mi].x = l2.x;
-                af[mi].y = l2.y;
-                af[mi].z = h2.x;
-                af[mi].w = h2.y;
-            }
+                for (int ni = 0; ni < 2; ++ni)
+                    bf[ni] = *reinterpret_cast<const u32x4 *>(
+                        stB + ((((wn * 2 + ni) * KS + ks) * 64) + lane) * 8);
+            };
+            // one iteration; r == s % R is the register slot of step s
+            auto iteration = [&](int s, int r, bool more_loads) {
+                u32x4 af[2], bf[2];
+                if (more_loads) {
+                    load_idx(tc, s + 2 * D, i_ring[(r + 2 * D) % R]); // padded list: in bounds
+                    issue(tc, s + D, i_ring[(r + D) % R], a_ring[(r + D) % R], b_ring[(r + D) % R]);
+                }
+                TW_STAMP(s, 0)
+                stage(s, a_ring[r], b_ring[r]);
+                TW_STAMP(s, 1)
+                __syncthreads();
+                TW_STAMP(s, 2)
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
-                bf[ni] = *reinterpret_cast<const u32x4 *>(
-                    stB + ((((wn * 2 + ni) * KS + ks) * 64) + lane) * 8);
-        };
-        auto mma = [&](const u32x4(&af)[2], const u32x4(&bf)[2]) {
+                for (int ks = 0; ks < KS; ++ks) {
+                    frags(s, ks, af, bf);
 #ifdef TW_EXP_NOMFMA
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+                    for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi)
-                    acc[mi][ni][0] += __uint_as_float(af[mi].x ^ bf[ni].x);
+                        for (int mi = 0; mi < 2; ++mi)
+                            acc[mi][ni][0] += __uint_as_float(af[mi].x ^ bf[ni].x);
 #else
 #pragma unroll
-            for (int ni = 0; ni < 2; ++ni)
+                    for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
-                for (int mi = 0; mi < 2; ++mi)
-                    acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
+                        for (int mi = 0; mi < 2; ++mi)
+                            acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
 #endif
-        };
+                }
+                TW_STAMP(s, 3)
+            };
 
-        constexpr int R = D + 1; // register slots: step s being staged plus D steps in flight
-        u32x4 a_ring[R][PASSES];
-        u32x4 b_ring[R][BPASS];
-        int i_ring[R];
-        // one iteration; r == s % R is the register slot of step s
-        auto iteration = [&](int s, int r, bool more_loads) {
-            u32x4 af[2], bf[2];
-            if (more_loads) {
-                load_idx(s + 2 * D, i_ring[(r + 2 * D) % R]); // padded list: stays in bounds
-                issue(s + D, i_ring[(r + D) % R], a_ring[(r + D) % R], b_ring[(r + D) % R]);
-            }
-            TW_STAMP(s, 0)
-            stage(s, a_ring[r], b_ring[r]);
-            TW_STAMP(s, 1)
-            __syncthreads();
-            TW_STAMP(s, 2)
+            if (!preloaded) {
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                frags(s, ks, af, bf);
-                mma(af, bf);
-            }
-            TW_STAMP(s, 3)
-        };
-
+                for (int j = 0; j < D; ++j)
+                    load_idx(tc, j, i_ring[j % R]);
 #pragma unroll
-        for (int j = 0; j < D; ++j)
-            load_idx(j, i_ring[j % R]);
-#pragma unroll
-        for (int j = 0; j < D; ++j) {
-            if (j < nsteps) {
-                issue(j, i_ring[j % R], a_ring[j], b_ring[j]);
-                load_idx(j + D, i_ring[(j + D) % R]);
-            }
-        }
-        int s0 = 0;
-        // steady state: every iteration issues, stages and multiplies, no conditionals
-        for (; s0 + R + D <= nsteps; s0 += R) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                iteration(s0 + r, r, true);
-        }
-        // drain: fewer than R + D steps remain
-        for (; s0 < nsteps; s0 += R) {
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                const int s = s0 + r;
-                if (s < nsteps)
-                    iteration(s, r, s + D < nsteps);
-            }
-        }
-        __syncthreads();
-
-#ifdef TW_EXP_TIMING
-        if (item == 0 && tid < 256)
-            reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
-#endif
-        // ---- epilogue ------------------------------------------------------------
-        const int32_t *const nlist = p.kept_n + u.kn_off;
-#pragma unroll
-        for (int ni = 0; ni < 2; ++ni) {
-            const int j = wn * 64 + ni * 32 + (lane & 31); // compact column inside the unit
-            int64_t coff = 0;
-            if (p.beta != 0.0f && j < u.n_cnt)
-                coff = (int64_t)(u.col0 + nlist[j]) * p.ldc;
-#pragma unroll
-            for (int mi = 0; mi < 2; ++mi) {
-                const int mloc = wm * 64 + mi * 32 + (lane >> 5) * 4;
-#pragma unroll
-                for (int r4 = 0; r4 < 4; ++r4) {
-                    float v[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        v[e] = p.alpha * acc[mi][ni][r4 * 4 + e];
-                        if (p.beta != 0.0f) {
-                            const int m = m0 + mloc + r4 * 8 + e;
-                            if (j < u.n_cnt && m < p.M)
-                                v[e] += p.beta * E::from_bits(C[coff + m]);
-                        }
+                for (int j = 0; j < D; ++j) {
+                    if (j < nsteps) {
+                        issue(tc, j, i_ring[j % R], a_ring[j], b_ring[j]);
+                        load_idx(tc, j + D, i_ring[(j + D) % R]);
                     }
-                    u32x2 pk;
-                    pk.x = E::to_bits(v[0]) | (E::to_bits(v[1]) << 16);
-                    pk.y = E::to_bits(v[2]) | (E::to_bits(v[3]) << 16);
-                    *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
                 }
             }
+            TW_PHASE(1)
+            if (!have_next)
+                claim_next();
+            TW_PHASE(2)
+            int s0 = 0;
+            // steady state: every iteration issues, stages and multiplies, no conditionals
+            for (; s0 + R + D <= nsteps; s0 += R) {
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    iteration(s0 + r, r, true);
+            }
+            // The next item's index words are fetched before the drain, so that its first row
+            // loads can be issued right after this item's last step and fly over the epilogue.
+            const bool chain = nxt.ticket < p.n_pipe_items;
+            Thr tn;
+            if (chain) {
+                tn = setup(nxt);
+#pragma unroll
+                for (int j = 0; j < 2 * D; ++j)
+                    load_idx(tn, j, n_idx[j]);
+            }
+            // drain: fewer than R + D steps remain
+            for (; s0 < nsteps; s0 += R) {
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    const int s = s0 + r;
+                    if (s < nsteps)
+                        iteration(s, r, s + D < nsteps);
+                }
+            }
+            __syncthreads();
+            TW_PHASE(3)
+            if (chain) {
+                const int nn = nxt.u.k_pad / BK;
+#pragma unroll
+                for (int j = 0; j < D; ++j) {
+                    if (j < nn)
+                        issue(tn, j, n_idx[j], a_ring[j], b_ring[j]);
+                    i_ring[(j + D) % R] = n_idx[j + D];
+                }
+            }
+            preloaded = chain;
+            TW_PHASE(4)
+
+            // ---- epilogue --------------------------------------------------------
+            const int32_t *const nlist = p.kept_n + u.kn_off;
+            float scale = p.alpha;
+            if (p.beta != 0.0f) {
+                // rare path, kept out of the way of the common one: fold alpha and beta*C into
+                // the accumulators first (C is read on kept columns only)
+#pragma unroll
+                for (int ni = 0; ni < 2; ++ni) {
+                    const int j = wn * 64 + ni * 32 + (lane & 31);
+                    const int64_t coff =
+                        j < u.n_cnt ? (int64_t)(u.col0 + nlist[j]) * p.ldc : (int64_t)0;
+#pragma unroll
+                    for (int mi = 0; mi < 2; ++mi)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) {
+                            const int m = m0 + wm * 64 + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
+                            float old = 0.0f;
+                            if (j < u.n_cnt && m < p.M)
+                                old = E::from_bits(C[coff + m]);
+                            acc[mi][ni][r] = p.alpha * acc[mi][ni][r] + p.beta * old;
+                        }
+                }
+                scale = 1.0f;
+            }
+#pragma unroll
+            for (int ni = 0; ni < 2; ++ni) {
+                const int j = wn * 64 + ni * 32 + (lane & 31); // compact column inside the unit
+#pragma unroll
+                for (int mi = 0; mi < 2; ++mi) {
+                    const int mloc = wm * 64 + mi * 32 + (lane >> 5) * 4;
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        u32x2 pk;
+                        pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
+                               (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
+                        pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
+                               (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
+                        *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                    }
+                }
+            }
+            __syncthreads();
+            TW_PHASE(5)
+            for (int j = rrow; j < u.n_cnt; j += RPP) {
+                const int c = u.col0 + nlist[j];
+                // rows of the staging tile are 8-byte aligned only: two 8-byte reads
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(smem + j * CPITCH + chunk * 8);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(smem + j * CPITCH + chunk * 8 + 4);
+                u32x4 v;
+                v.x = lo.x;
+                v.y = lo.y;
+                v.z = hi.x;
+                v.w = hi.y;
+                store_chunk(C + (int64_t)c * p.ldc + tc.m_ld, v, tc.m_ld, p.M);
+            }
         }
+
+        TW_PHASE(6)
         __syncthreads();
-        for (int j = rrow; j < u.n_cnt; j += RPP) {
-            const int c = u.col0 + nlist[j];
-            const u32x4 v = *reinterpret_cast<const u32x4 *>(smem + j * CPITCH + chunk * 8);
-            store_chunk(C + (int64_t)c * p.ldc + m_ld, v, m_ld, p.M);
-        }
-        __syncthreads();
+        TW_PHASE(7)
+        cur = nxt;
+        have_next = false;
+        ++n_done_items;
     }
 
-    // the last workgroup to leave re-arms the ticket slot for the next launch
+#ifdef TW_EXP_TIMING
+    __syncthreads();
+    if (blockIdx.x == 0 && tid < 256)
+        reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
+#endif
+    // the last workgroup to leave re-arms the ticket slot for the next launch; waiting for
+    // the pending ticket first keeps every atomic of this workgroup ahead of that reset
     if (tid == 0) {
         __threadfence();
-        const int done = atomicAdd(&p.ticket[1], 1);
+        const int done = atomicAdd(&p.ticket[1], t_pending >= 0 ? 1 : 1);
         if (done == (int)gridDim.x - 1) {
             p.ticket[0] = 0;
             p.ticket[1] = 0;
@@ -645,6 +758,7 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
         a.M = M;
         a.n_mblk = (M + 127) / 128;
         a.n_gemm_items = plan->n_units * a.n_mblk;
+        a.n_pipe_items = plan->n_pipe_units * a.n_mblk;
         a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
         a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
         a.alpha = alpha;
@@ -695,6 +809,7 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     a.M = M;
     a.n_mblk = (M + BM - 1) / BM;
     a.n_gemm_items = plan->n_units * a.n_mblk;
+    a.n_pipe_items = plan->n_pipe_units * a.n_mblk;
     a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
     a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
     a.alpha = alpha;

@@ -57,6 +57,7 @@ struct GemmArgs {
     int32_t M;
     int32_t n_mblk;       // ceil(M / BM)
     int32_t n_gemm_items; // n_units * n_mblk
+    int32_t n_pipe_items; // items of units with at least one kept K row (they come first)
     int32_t n_items;      // + n_zero_tiles * n_mblk when zero-filling
     int32_t n_zero_tiles; // tiles with pruned columns (first entries of `tiles`)
     float alpha, beta;
@@ -74,7 +75,7 @@ struct tw_plan {
     std::vector<int32_t> k_pad, n_pad;
     std::vector<int64_t> b_off; // element offset of each tile's packed weight
     int64_t packed_elems = 0;
-    int n_units = 0, n_zero_tiles = 0, max_unit_n = 0;
+    int n_units = 0, n_pipe_units = 0, n_zero_tiles = 0, max_unit_n = 0;
     // device
     int32_t *d_kept_k = nullptr, *d_kept_n = nullptr, *d_rel_k = nullptr, *d_rel_n = nullptr;
     int32_t *d_pruned_n = nullptr;

@@ -24,6 +24,11 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 
+# HBM bytes per sparse launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
+# by what the same counter reads for a 256 MiB copy in the same run (reads x 2.0, writes x 1.0);
+# the runs and their commands are in profiles/tw_gemm_kmajor_kernel__vgg16_conv4_2.md.
+MEASURED_TRAFFIC_BYTES = {"vgg16_conv4_2": (124780 + 14032) * 1024}
+
 
 def make_workload(name):
     from tilesparsity_amd import workloads as W
@@ -181,7 +186,9 @@ def main():
         "mfma_utilisation_dense_run": res["mfma_util_dense_run"],
         "us_sparse": res["us_sparse"], "us_dense": res["us_dense"],
         "roofline": {"bound": "hbm", "achieved": res["hbm_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": res["hbm_gbs"] / HBM_PEAK_GBS, "traffic": None},
+                     "unit": "GB/s", "frac": res["hbm_gbs"] / HBM_PEAK_GBS,
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+                     "algorithmic_bytes": res["algorithmic_bytes"]},
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, A, B)

@@ -23,6 +23,7 @@
 #include "tw_internal.h"
 
 #include <atomic>
+#include <cstddef>
 #include <cstdlib>
 
 namespace tw {
@@ -528,6 +529,528 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     }
 }
 
+// Workgroup barrier for hand-overs through LDS only: waits for this wave's LDS operations, not
+// for its global loads, stores or atomics in flight (which __syncthreads() would do for stores
+// and atomics), so prefetched loads, the item's output stores and the ticket atomic keep flying.
+#define TW_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+
+// ---------------------------------------------------------------------------------
+// Wave-specialised 256 x 128 kernel (8 waves, one workgroup per CU).  Waves 0-3 only multiply:
+// wave w owns rows 64w..64w+63 of the row block and all 128 compact columns (2 x 4 MFMA
+// blocks, 128 accumulator registers).  Waves 4-7 only move data: they gather the kept rows of
+// A and the packed weight global -> registers -> LDS, R steps of 64 rows in flight.  Both
+// halves meet at one barrier per step: while the multiplying waves read stage s & 1, the
+// moving waves fill stage (s + 1) & 1, so LDS traffic, vector-memory traffic and MFMA work
+// overlap instead of following each other.  One multiplying and one moving wave share a SIMD.
+// Work items, tickets, the chained first loads of the next item and the epilogue are those of
+// tw_gemm_kmajor_kernel.
+template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(const GemmArgs p)
+{
+    constexpr int NT = 512, NP = 256, BM = 256, BN = 128, BK = 64;
+    constexpr int KS = BK / kMfmaK, PKS = kBlockK / kMfmaK;
+    constexpr int R = 2;                       // register slots = steps of loads in flight
+    constexpr int MI = 2, NI = 4;
+    constexpr int CPR = BM / 8;                // 16-byte chunks per staged A row / stored C column
+    constexpr int RPP = NP / CPR;              // A rows covered by one pass of the moving waves
+    constexpr int PASSES = BK / RPP;           // A loads per moving thread and step
+    constexpr int BPASS = BN * BK / 8 / NP;    // weight loads per moving thread and step
+    constexpr int PITCH = BM + TW_A_PAD;
+    constexpr int ASTAGE = BK * PITCH, BSTAGE = BN * BK;
+    constexpr int CPITCH = BM + 4;
+    constexpr int PIPE = 2 * (ASTAGE + BSTAGE);
+    constexpr int SMEM = PIPE > BN * CPITCH ? PIPE : BN * CPITCH;
+    static_assert(BK == kBlockK && KS == PKS, "one packed weight step per main-loop step");
+    using E = Elem<DT>;
+
+    __shared__ __align__(16) uint16_t smem[SMEM];
+    __shared__ int s_tk[2];
+    __shared__ int s_cols[BN]; // output columns of the current item's unit
+#ifdef TW_EXP_TIMING
+    __shared__ unsigned long long s_ws[256];
+    bool ws_first = true;
+#define TW_WS_STAMP(step, k, t)                                                          \
+    if (blockIdx.x == 0 && ws_first && threadIdx.x == (t) && (step) < 30)               \
+        s_ws[(step)*8 + (k)] = __builtin_readcyclecounter();
+#define TW_WS_PHASE(k, t)                                                                \
+    if (blockIdx.x == 0 && ws_first && threadIdx.x == (t))                               \
+        s_ws[240 + (k)] = __builtin_readcyclecounter();
+#else
+#define TW_WS_STAMP(step, k, t)
+#define TW_WS_PHASE(k, t)
+#endif
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
+    uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
+    const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
+    uint16_t *const sA = smem;
+    uint16_t *const sB = smem + 2 * ASTAGE;
+
+    struct Item {
+        int ticket;
+        int m0, m_end; // rows [m0, m_end) of A and C, at most BM of them
+        UnitDev u;     // valid for ticket < n_gemm_items
+    };
+    auto make_item = [&](int ticket) {
+        Item it;
+        it.ticket = ticket;
+        it.m0 = 0;
+        it.m_end = 0;
+        if (ticket < p.n_gemm_items) {
+            const auto *ka = (const __attribute__((address_space(4))) int32_t *)
+                __builtin_amdgcn_kernarg_segment_ptr();
+            const int ui = ticket / p.n_mblk;
+            it.m0 = (ticket - ui * p.n_mblk) * BM;
+            it.m_end = it.m0 + BM < p.M ? it.m0 + BM : p.M;
+            static_assert(sizeof(UnitDev) == 48, "UnitDev is read as 12 words");
+            int32_t w[12];
+            if (p.n_arg_units) {
+                // from the kernel-argument segment: scalar loads, no global round trip
+#pragma unroll
+                for (int i = 0; i < 12; ++i)
+                    w[i] = ka[offsetof(GemmArgs, arg_units) / 4 + ui * 12 + i];
+            } else {
+                __builtin_memcpy(w, &p.units[ui], sizeof(UnitDev));
+            }
+            // the descriptor is workgroup-uniform: keep it, and all derived from it, scalar
+#pragma unroll
+            for (int i = 0; i < 12; ++i)
+                w[i] = __builtin_amdgcn_readfirstlane(w[i]);
+            __builtin_memcpy(&it.u, w, sizeof(UnitDev));
+        }
+        return it;
+    };
+    // Both halves of the workgroup walk the same item sequence and execute the same sequence
+    // of barriers; thread 0 (a multiplying wave) owns the ticket counter.
+#ifdef TW_EXP_TIMING
+    if (blockIdx.x == 0 && tid == 0) {
+        s_ws[248] = __builtin_readcyclecounter();
+        s_ws[249] = __builtin_amdgcn_s_memrealtime();
+    }
+#if TW_EXP_TIMING == 2
+    if (tid == 0 && blockIdx.x < 256)
+        reinterpret_cast<unsigned *>(p.dbg)[blockIdx.x * 2] = (unsigned)__builtin_amdgcn_s_memrealtime();
+#endif
+#endif
+    const int ticket_base = gridDim.x;
+    int t_pending = 0;
+    if (tid == 0)
+        t_pending = atomicAdd(&p.ticket[0], 1);
+    auto claim = [&]() { // two barriers
+        if (tid == 0) {
+            s_tk[0] = ticket_base + t_pending;
+            t_pending = atomicAdd(&p.ticket[0], 1);
+        }
+        TW_LDS_BARRIER();
+        const Item it = make_item(__builtin_amdgcn_readfirstlane(s_tk[0]));
+        TW_LDS_BARRIER();
+        return it;
+    };
+    // zero-fill item: pruned columns of one tile receive beta*C (all threads, no barrier)
+    auto zero_fill = [&](int item) {
+        const int z = item - p.n_gemm_items;
+        const int zt = z / p.n_mblk;
+        const int m = (z - zt * p.n_mblk) * BM + (tid % CPR) * 8;
+        const TileDev t = p.tiles[zt];
+        for (int j = tid / CPR; j < t.n_pruned; j += NT / CPR) {
+            const int c = t.col0 + p.pruned_n[t.pn_off + j];
+            uint16_t *dst = C + (int64_t)c * p.ldc + m;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (p.beta != 0.0f && m < p.M) {
+                uint32_t w[4] = {0u, 0u, 0u, 0u};
+                for (int e = 0; e < 8 && m + e < p.M; ++e)
+                    w[e >> 1] |= E::to_bits(p.beta * E::from_bits(dst[e])) << ((e & 1) * 16);
+                v.x = w[0];
+                v.y = w[1];
+                v.z = w[2];
+                v.w = w[3];
+            }
+            store_chunk(dst, v, m, p.M);
+        }
+    };
+    // scatters the staged C tile (all threads): whole columns col0 + kept_n[j], 16-byte stores
+    // (the output columns col0 + kept_n[j] come from s_cols, filled by the moving waves)
+    auto store_tile = [&](const UnitDev &u, int m0, int m_end) {
+        const int m_st = m0 + (tid % CPR) * 8;
+        for (int j = tid / CPR; j < u.n_cnt; j += NT / CPR) {
+            const int c = s_cols[j];
+            // rows of the staging tile are 8-byte aligned only: two 8-byte reads
+            const u32x2 lo = *reinterpret_cast<const u32x2 *>(smem + j * CPITCH + (tid % CPR) * 8);
+            const u32x2 hi = *reinterpret_cast<const u32x2 *>(smem + j * CPITCH + (tid % CPR) * 8 + 4);
+            u32x4 v;
+            v.x = lo.x;
+            v.y = lo.y;
+            v.z = hi.x;
+            v.w = hi.y;
+#ifdef TW_EXP_NOSTORE
+            if (v.x == 0x12345678u)
+#endif
+            store_chunk(C + (int64_t)c * p.ldc + m_st, v, m_st, m_end);
+        }
+    };
+
+    if (wave >= 4) {
+        // ================= moving waves ===================================================
+        // Thread pt moves chunk pt % 32 (8 consecutive m) of the rows 8 * (pt / 32) .. + 7 of a
+        // step: a wave covers 16 consecutive kept rows, whose indices it fetches with one
+        // scalar load.  Addresses are a uniform base plus a 32-bit byte offset per lane.
+        const int pt = tid - NP;
+        const int chunk = pt % CPR, rgrp = pt / CPR;
+        const bool upper = (lane >> 5) != 0;           // second row group of this wave
+        const int mw = wave - 4;
+        const uint32_t lda_b = (uint32_t)p.lda * 2u;   // bytes; K * lda * 2 < 2^32 (host check)
+        typedef int i32x16 __attribute__((ext_vector_type(16)));
+        struct Idx {
+            int k[16];
+        };
+        struct Thr {
+            const int32_t *klist;   // + 16 * mw: this wave's rows of step 0
+            const char *a_base;     // A + m0 (bytes), uniform
+            const char *b_base[BPASS];
+            int64_t b_pack_b;
+            uint32_t v_chunk;       // byte offset of this lane's chunk inside a gathered row
+            bool m_ok;
+        };
+        auto setup = [&](const Item &it) {
+            Thr t;
+            t.klist = p.kept_k + it.u.kk_off + 16 * mw; // padded past k_pad
+            t.a_base = reinterpret_cast<const char *>(A + it.m0);
+            t.m_ok = it.m0 + chunk * 8 < it.m_end;
+            t.v_chunk = t.m_ok ? chunk * 16 : 0; // beyond the row block: re-read its first chunk
+            // weight chunk c = pt + bp * NP of a step is (nb = bp, k16 = pt / 64, lane = pt % 64);
+            // a block beyond the unit reads block 0 (its products are never stored)
+#pragma unroll
+            for (int bp = 0; bp < BPASS; ++bp)
+                t.b_base[bp] = reinterpret_cast<const char *>(
+                    Bp + it.u.b_off + (int64_t)(it.u.nb0 + (bp < it.u.nb_cnt ? bp : 0)) * (PKS * 64 * 8));
+            t.b_pack_b = (int64_t)it.u.nblk * (PKS * 64 * 8 * 2);
+            return t;
+        };
+        auto load_idx = [&](const Thr &t, int s, Idx &ix) {
+            const i32x16 v = *reinterpret_cast<const __attribute__((address_space(4))) i32x16 *>(
+                (uintptr_t)(t.klist + s * BK));
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                ix.k[i] = v[i];
+                asm volatile("" : "+s"(ix.k[i])); // keep the words scalar and the load whole
+            }
+        };
+        auto load_a = [&](const Thr &t, const Idx &ix, int ps) {
+            uint32_t o0 = (uint32_t)ix.k[ps] * lda_b, o1 = (uint32_t)ix.k[8 + ps] * lda_b;
+            asm volatile("" : "+s"(o0), "+s"(o1)); // multiply on the scalar unit, select afterwards
+            return *reinterpret_cast<const u32x4 *>(t.a_base + ((upper ? o1 : o0) + t.v_chunk));
+        };
+        auto load_b = [&](const Thr &t, int s, int bp) {
+#ifdef TW_EXP_NOB
+            return u32x4{(unsigned)s, 0u, 0u, 0u};
+#else
+            return *reinterpret_cast<const u32x4 *>(t.b_base[bp] + (int64_t)s * t.b_pack_b +
+                                                    (uint32_t)(pt * 16));
+#endif
+        };
+        auto issue = [&](const Thr &t, int s, const Idx &ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps)
+                ar[ps] = load_a(t, ix, ps);
+#pragma unroll
+            for (int bp = 0; bp < BPASS; ++bp)
+                br[bp] = load_b(t, s, bp);
+        };
+        u32x4 a_ring[R][PASSES];
+        u32x4 b_ring[R][BPASS];
+        Idx ix_next;            // row indices of the step issued next
+        bool preloaded = false; // cur's first R steps are in flight, ix_next is that of step R
+
+        TW_WS_PHASE(6, 256)
+        Item cur = make_item(blockIdx.x);
+        Item nxt = cur;
+        bool have_next = false, first = true;
+#ifdef TW_EXP_TIMING
+        if (cur.u.k_pad >= 0)
+            TW_WS_PHASE(7, 256)
+#endif
+        while (cur.ticket < p.n_items) {
+            const int item = cur.ticket;
+            if (!first || item >= p.n_pipe_items) {
+                nxt = claim();
+                have_next = true;
+            }
+            first = false;
+            if (item >= p.n_gemm_items) {
+                zero_fill(item);
+            } else {
+                const UnitDev &u = cur.u;
+                const int m0 = cur.m0;
+                const int nsteps = u.k_pad / BK;
+                const Thr tc = setup(cur);
+                if (!preloaded) {
+                    Idx ix[R];
+#pragma unroll
+                    for (int j = 0; j < R; ++j)
+                        load_idx(tc, j, ix[j]); // the padded list keeps every index load in bounds
+                    load_idx(tc, R, ix_next);
+#ifdef TW_EXP_TIMING
+                    if (ix_next.k[0] >= 0 && blockIdx.x == 0 && ws_first && threadIdx.x == 256)
+                        s_ws[252] = __builtin_readcyclecounter();
+#endif
+#pragma unroll
+                    for (int j = 0; j < R; ++j)
+                        if (j < nsteps)
+                            issue(tc, j, ix[j], a_ring[j], b_ring[j]);
+                }
+                TW_WS_PHASE(0, 256)
+                if (!have_next) {
+                    nxt = claim();
+                    have_next = true;
+                }
+                TW_WS_PHASE(1, 256)
+                // time slot j: write step j (loaded R slots ago) into stage j & 1 and reuse its
+                // registers for the loads of step j + R.  Every register is written to LDS and
+                // refilled by its next load back to back, so that the LDS queue and the
+                // vector-memory queue are fed at the same time.
+                auto slot = [&](int j, int r, bool more) {
+                    TW_WS_STAMP(j, 2, 256)
+                    uint16_t *const stA = sA + (j & 1) * ASTAGE;
+                    uint16_t *const stB = sB + (j & 1) * BSTAGE;
+                    const bool edge = j * BK + BK > u.k_kept || m0 + BM > cur.m_end;
+                    const Idx ix = ix_next;
+                    if (more)
+                        load_idx(tc, j + R + 1, ix_next);
+#pragma unroll
+                    for (int ps = 0; ps < PASSES; ++ps) {
+                        u32x4 v = a_ring[r][ps];
+                        if (edge) {
+                            // rows beyond K_t and chunks beyond M become zeros
+                            const uint32_t keep =
+                                (j * BK + rgrp * 8 + ps < u.k_kept && tc.m_ok) ? 0xFFFFFFFFu : 0u;
+                            v.x &= keep;
+                            v.y &= keep;
+                            v.z &= keep;
+                            v.w &= keep;
+                        }
+                        *reinterpret_cast<u32x4 *>(stA + (rgrp * 8 + ps) * PITCH + chunk * 8) = v;
+                        if (more)
+                            a_ring[r][ps] = load_a(tc, ix, ps);
+                    }
+#pragma unroll
+                    for (int bp = 0; bp < BPASS; ++bp) {
+                        *reinterpret_cast<u32x4 *>(stB + (pt + bp * NP) * 8) = b_ring[r][bp];
+                        if (more)
+                            b_ring[r][bp] = load_b(tc, j + R, bp);
+                    }
+                    TW_WS_STAMP(j, 4, 256)
+                    TW_LDS_BARRIER();
+                    TW_WS_STAMP(j, 5, 256)
+                };
+                int j0 = 0;
+                for (; j0 + 2 * R <= nsteps; j0 += R) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        slot(j0 + r, r, true);
+                }
+                for (; j0 < nsteps; j0 += R) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        if (j0 + r < nsteps)
+                            slot(j0 + r, r, j0 + r + R < nsteps);
+                }
+                // last time slot: the multiplying waves work on the last step; the first loads of
+                // the next item start now and fly over the epilogue
+                int out_col = 0;
+                if (pt < BN)
+                    out_col = u.col0 + p.kept_n[u.kn_off + (pt < u.n_cnt ? pt : 0)];
+                const bool chain = nxt.ticket < p.n_pipe_items;
+                if (chain) {
+                    const Thr tn = setup(nxt);
+                    const int nn = nxt.u.k_pad / BK;
+                    Idx ix[R];
+#pragma unroll
+                    for (int j = 0; j < R; ++j)
+                        load_idx(tn, j, ix[j]);
+                    load_idx(tn, R, ix_next);
+#pragma unroll
+                    for (int j = 0; j < R; ++j)
+                        if (j < nn)
+                            issue(tn, j, ix[j], a_ring[j], b_ring[j]);
+                }
+                preloaded = chain;
+                if (pt < BN)
+                    s_cols[pt] = out_col;
+                TW_WS_PHASE(2, 256)
+                TW_LDS_BARRIER(); // end of the last time slot
+                TW_WS_PHASE(3, 256)
+                TW_LDS_BARRIER(); // the C tile is staged
+                TW_WS_PHASE(4, 256)
+                store_tile(u, m0, cur.m_end);
+                TW_WS_PHASE(5, 256)
+            }
+            TW_LDS_BARRIER(); // LDS may be reused now
+            cur = nxt;
+            have_next = false;
+#ifdef TW_EXP_TIMING
+            ws_first = false;
+#endif
+        }
+    } else {
+        // ================= multiplying waves ==============================================
+        Item cur = make_item(blockIdx.x);
+        Item nxt = cur;
+        bool have_next = false, first = true;
+        while (cur.ticket < p.n_items) {
+            const int item = cur.ticket;
+            if (!first || item >= p.n_pipe_items) {
+                nxt = claim();
+                have_next = true;
+            }
+            first = false;
+            if (item >= p.n_gemm_items) {
+                zero_fill(item);
+            } else {
+                const UnitDev &u = cur.u;
+                const int m0 = cur.m0;
+                const int nsteps = u.k_pad / BK;
+                f32x16 acc[MI][NI];
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r)
+                            acc[mi][ni][r] = 0.0f;
+                if (!have_next) {
+                    nxt = claim();
+                    have_next = true;
+                }
+                const bool w_active = m0 + wave * 64 < cur.m_end;
+                auto frags = [&](int s, int ks, u32x4(&af)[MI], u32x4(&bf)[NI]) {
+                    const uint16_t *const stA = sA + (s & 1) * ASTAGE;
+                    const uint16_t *const stB = sB + (s & 1) * BSTAGE;
+#pragma unroll
+                    for (int mi = 0; mi < MI; ++mi) {
+                        // ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(m) block; lane L addresses
+                        // row L/4, columns 4*(L%4)..+3 and receives column L of the 4 rows.
+                        const int L = lane & 15;
+                        const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
+                        const int col = wave * 64 + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
+                        const uint16_t *q = stA + row * PITCH + col;
+                        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
+                        s16x4 hi =
+                            __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * PITCH));
+                        u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                        af[mi].x = l2.x;
+                        af[mi].y = l2.y;
+                        af[mi].z = h2.x;
+                        af[mi].w = h2.y;
+                    }
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+                        bf[ni] = *reinterpret_cast<const u32x4 *>(stB + ((ni * KS + ks) * 64 + lane) * 8);
+                };
+                TW_LDS_BARRIER(); // time slot 0: step 0 is being staged
+                for (int s = 0; s < nsteps; ++s) {
+                    TW_WS_STAMP(s, 0, 0)
+#ifdef TW_EXP_NOMFMA
+                    if (w_active && s == 0) {
+#else
+                    if (w_active) {
+#endif
+                        u32x4 af[2][MI], bf[2][NI];
+                        frags(s, 0, af[0], bf[0]);
+#pragma unroll
+                        for (int ks = 0; ks < KS; ++ks) {
+                            if (ks + 1 < KS)
+                                frags(s, ks + 1, af[(ks + 1) & 1], bf[(ks + 1) & 1]);
+#pragma unroll
+                            for (int ni = 0; ni < NI; ++ni)
+#pragma unroll
+                                for (int mi = 0; mi < MI; ++mi)
+                                    acc[mi][ni] = E::mfma(af[ks & 1][mi], bf[ks & 1][ni], acc[mi][ni]);
+                        }
+                    }
+                    TW_WS_STAMP(s, 1, 0)
+                    TW_LDS_BARRIER();
+                }
+
+                // epilogue: alpha/beta in fp32, round, hand the tile over through LDS
+                const int32_t *const nlist = p.kept_n + u.kn_off;
+                float scale = p.alpha;
+                if (p.beta != 0.0f) {
+                    // rare path: fold alpha and beta*C into the accumulators first (C is read on
+                    // kept columns only)
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int j = ni * 32 + (lane & 31);
+                        const int64_t coff =
+                            j < u.n_cnt ? (int64_t)(u.col0 + nlist[j]) * p.ldc : (int64_t)0;
+#pragma unroll
+                        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+                            for (int r = 0; r < 16; ++r) {
+                                const int m = m0 + wave * 64 + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
+                                float old = 0.0f;
+                                if (j < u.n_cnt && m < cur.m_end)
+                                    old = E::from_bits(C[coff + m]);
+                                acc[mi][ni][r] = p.alpha * acc[mi][ni][r] + p.beta * old;
+                            }
+                    }
+                    scale = 1.0f;
+                }
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int j = ni * 32 + (lane & 31); // compact column inside the unit
+#pragma unroll
+                    for (int mi = 0; mi < MI; ++mi) {
+                        const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
+#pragma unroll
+                        for (int r4 = 0; r4 < 4; ++r4) {
+                            u32x2 pk;
+                            pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
+                                   (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
+                            pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
+                                   (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
+                            *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                        }
+                    }
+                }
+                TW_LDS_BARRIER(); // the C tile is staged
+                store_tile(u, m0, cur.m_end);
+            }
+            TW_LDS_BARRIER(); // LDS may be reused now
+            cur = nxt;
+            have_next = false;
+#ifdef TW_EXP_TIMING
+            ws_first = false;
+#endif
+        }
+#ifdef TW_EXP_TIMING
+        if (blockIdx.x == 0 && tid == 0) {
+            s_ws[250] = __builtin_readcyclecounter();
+            s_ws[251] = __builtin_amdgcn_s_memrealtime();
+        }
+        __builtin_amdgcn_s_waitcnt(0);
+#if TW_EXP_TIMING == 2
+        if (tid == 0 && blockIdx.x < 256)
+            reinterpret_cast<unsigned *>(p.dbg)[blockIdx.x * 2 + 1] = (unsigned)__builtin_amdgcn_s_memrealtime();
+#else
+        if (blockIdx.x == 0 && tid < 256)
+            reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ws[tid];
+#endif
+#endif
+        // the last workgroup to leave re-arms the ticket slot for the next launch
+        if (tid == 0) {
+            __threadfence();
+            const int done = atomicAdd(&p.ticket[1], t_pending >= 0 ? 1 : 1);
+            if (done == (int)gridDim.x - 1) {
+                p.ticket[0] = 0;
+                p.ticket[1] = 0;
+                __threadfence();
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // Layout-generic kernel: any combination of K-major / row-major A and C through element
 // strides.  One workgroup (4 waves, 128 x 128 tile, 32-row steps) per work item in queue
@@ -685,12 +1208,14 @@ static int env_int(const char *name, int dflt)
     return v && *v ? atoi(v) : dflt;
 }
 
-// Tile shapes: 0: 256 x 128 (8 waves, one workgroup per CU), 1: 128 x 128 (4 waves, two
-// per CU), 2: 512 x 64, 3: 256 x 64 (the two shapes for tiles of at most 64 kept columns).
+// Tile shapes: 0: 256 x 128 (8 waves of 64 x 64, one workgroup per CU), 1: 128 x 128 (4 waves,
+// two per CU), 2: 512 x 64, 3: 256 x 64 (the two shapes for tiles of at most 64 kept columns),
+// 4: 256 x 128 wave-specialised (the default for wider tiles; shape 0 remains for operands the
+// 32-bit offsets of shape 4 cannot address).
 struct Shape {
     int bm, wgs_per_cu;
 };
-static const Shape kShapes[4] = {{256, 1}, {128, 2}, {512, 1}, {256, 2}};
+static const Shape kShapes[5] = {{256, 1}, {128, 2}, {512, 1}, {256, 2}, {256, 1}};
 
 template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int grid, hipStream_t s)
 {
@@ -704,8 +1229,11 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
     case 2:
         hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 8, 1, 32, 2, 1>), dim3(grid), dim3(512), 0, s, a);
         break;
-    default:
+    case 3:
         hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 1, 32, 2, 2>), dim3(grid), dim3(256), 0, s, a);
+        break;
+    default: // 4: wave-specialised 256 x 128
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT>), dim3(grid), dim3(512), 0, s, a);
         break;
     }
 }
@@ -765,6 +1293,7 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
         a.beta = beta;
         a.ticket = nullptr;
         a.dbg = nullptr;
+        a.n_arg_units = 0;
         if (a.n_items == 0)
             return TW_OK;
         const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
@@ -784,15 +1313,17 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     // Shape choice: the large tile halves the weight traffic per row of A, but needs enough
     // work items to fill the chip; otherwise the small tile with two workgroups per CU.
     const bool narrow = plan->max_unit_n <= 64;
-    int shape = narrow ? 2 : 0;
+    // the wave-specialised kernel addresses A with 32-bit byte offsets
+    const bool ws_ok = (uint64_t)plan->K * (uint64_t)lda * 2u < (1ull << 32);
+    int shape = narrow ? 2 : (ws_ok ? 4 : 0);
     {
         const int forced = env_int("TWGEMM_SHAPE", -1);
         const int64_t big_items =
             (int64_t)plan->n_units * ((M + kShapes[shape].bm - 1) / kShapes[shape].bm);
-        if (forced >= 0 && forced < 4 && (forced >= 2) == narrow)
+        if (forced >= 0 && forced < 5 && (forced == 2 || forced == 3) == narrow && (forced != 4 || ws_ok))
             shape = forced;
         else if (big_items * 5 < 3 * (int64_t)plan->cu_count)
-            shape += 1; // too few large items to occupy the chip
+            shape = narrow ? 3 : 1; // too few large items to occupy the chip
     }
     const int BM = kShapes[shape].bm;
     GemmArgs a;
@@ -810,6 +1341,7 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     a.n_mblk = (M + BM - 1) / BM;
     a.n_gemm_items = plan->n_units * a.n_mblk;
     a.n_pipe_items = plan->n_pipe_units * a.n_mblk;
+    const int per_cu = env_int("TWGEMM_WGS_PER_CU", kShapes[shape].wgs_per_cu);
     a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
     a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
     a.alpha = alpha;
@@ -820,8 +1352,10 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
         __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kTicketSlots;
     a.ticket = plan->d_tickets + 2 * slot;
     a.dbg = plan->d_tickets + 2 * kTicketSlots;
+    a.n_arg_units = plan->n_units <= kMaxArgUnits ? plan->n_units : 0;
+    for (int i = 0; i < a.n_arg_units; ++i)
+        a.arg_units[i] = plan->h_units[i];
 
-    const int per_cu = env_int("TWGEMM_WGS_PER_CU", kShapes[shape].wgs_per_cu);
     const int grid = (int)std::min<int64_t>(a.n_items, (int64_t)plan->cu_count * per_cu);
     hipStream_t s = (hipStream_t)stream;
     if (plan->dtype == TW_F16)

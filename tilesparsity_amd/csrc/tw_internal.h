@@ -19,6 +19,7 @@ constexpr int kMfmaK = 16;    // k extent of one v_mfma_f32_32x32x16
 constexpr int kBlockK = 64;   // k rows per packed weight step; K_t is padded to this
 constexpr int kMaxUnitN = 128; // compact columns handled by one work item
 constexpr int kTicketSlots = 256;
+constexpr int kMaxArgUnits = 32;
 
 // One schedulable piece of a tile: at most kMaxUnitN compact columns.
 // 48 bytes; read with scalar loads.
@@ -63,6 +64,11 @@ struct GemmArgs {
     float alpha, beta;
     int32_t *ticket;      // [0] next item, [1] finished workgroups
     void *dbg;            // 2 KiB scratch after the ticket slots (instrumented builds only)
+    // Copy of `units` inside the kernel arguments for plans of at most kMaxArgUnits units
+    // (n_arg_units == 0 otherwise): a workgroup then reads its first unit through the scalar
+    // cache instead of waiting for a global load before it can fetch anything else.
+    int32_t n_arg_units;
+    UnitDev arg_units[kMaxArgUnits];
 };
 
 } // namespace tw
@@ -76,6 +82,7 @@ struct tw_plan {
     std::vector<int64_t> b_off; // element offset of each tile's packed weight
     int64_t packed_elems = 0;
     int n_units = 0, n_pipe_units = 0, n_zero_tiles = 0, max_unit_n = 0;
+    std::vector<tw::UnitDev> h_units; // host copy of d_units (queue order)
     // device
     int32_t *d_kept_k = nullptr, *d_kept_n = nullptr, *d_rel_k = nullptr, *d_rel_n = nullptr;
     int32_t *d_pruned_n = nullptr;

@@ -380,6 +380,7 @@ int finalize_plan_geometry(tw_plan *p)
                      [](const UnitDev &a, const UnitDev &b) { return a.k_kept > b.k_kept; });
     p->packed_elems = off;
     p->n_units = (int)units.size();
+    p->h_units = units;
     p->n_pipe_units = 0;
     for (const UnitDev &u : units)
         p->n_pipe_units += u.k_pad > 0;

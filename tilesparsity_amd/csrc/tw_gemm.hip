@@ -567,7 +567,11 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     __shared__ int s_cols[BN]; // output columns of the current item's unit
 #ifdef TW_EXP_TIMING
     __shared__ unsigned long long s_ws[256];
-    bool ws_first = true;
+#ifndef TW_EXP_ITEM
+#define TW_EXP_ITEM 0
+#endif
+    int ws_item = 0;
+#define ws_first (ws_item == TW_EXP_ITEM)
 #define TW_WS_STAMP(step, k, t)                                                          \
     if (blockIdx.x == 0 && ws_first && threadIdx.x == (t) && (step) < 30)               \
         s_ws[(step)*8 + (k)] = __builtin_readcyclecounter();
@@ -634,18 +638,40 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         reinterpret_cast<unsigned *>(p.dbg)[blockIdx.x * 2] = (unsigned)__builtin_amdgcn_s_memrealtime();
 #endif
 #endif
-    const int ticket_base = gridDim.x;
-    int t_pending = 0;
+    // The first two items of a workgroup are fixed (block index, block index + grid size), so
+    // that no atomic's round trip sits between the start of the kernel and the first loads;
+    // the shared counter hands out the items after those.
+    const int ticket_base = 2 * gridDim.x;
+    int t_pending = 0;                     // thread 0: result of the claim in flight
+    int t_next = gridDim.x + blockIdx.x;   // thread 0: the next ticket once known, or -1
     if (tid == 0)
         t_pending = atomicAdd(&p.ticket[0], 1);
-    auto claim = [&]() { // two barriers
-        if (tid == 0) {
-            s_tk[0] = ticket_base + t_pending;
+    // Picks up the claim in flight and starts the one after it.  Called before an item's output
+    // stores are issued: memory operations complete in order, so waiting for an atomic issued
+    // after them (or overwriting its register) would wait for the stores as well.
+    auto pick_up = [&]() {
+        if (tid == 0 && t_next < 0) {
+            t_next = ticket_base + t_pending;
+            asm volatile("" : "+v"(t_next)); // here, not where it is published
             t_pending = atomicAdd(&p.ticket[0], 1);
         }
+    };
+    auto claim = [&]() { // two barriers
+        if (tid == 0) {
+            pick_up();
+            s_tk[0] = t_next;
+            t_next = -1;
+        }
+        TW_WS_STAMP(0, 6, 256)
         TW_LDS_BARRIER();
+        TW_WS_STAMP(0, 7, 256)
         const Item it = make_item(__builtin_amdgcn_readfirstlane(s_tk[0]));
+#ifdef TW_EXP_TIMING
+        if (it.u.k_pad >= 0)
+            TW_WS_STAMP(1, 6, 256)
+#endif
         TW_LDS_BARRIER();
+        TW_WS_STAMP(1, 7, 256)
         return it;
     };
     // zero-fill item: pruned columns of one tile receive beta*C (all threads, no barrier)
@@ -773,10 +799,16 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #endif
         while (cur.ticket < p.n_items) {
             const int item = cur.ticket;
+#if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
+            TW_WS_PHASE(6, 256)
+#endif
             if (!first || item >= p.n_pipe_items) {
                 nxt = claim();
                 have_next = true;
             }
+#if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
+            TW_WS_PHASE(7, 256)
+#endif
             first = false;
             if (item >= p.n_gemm_items) {
                 zero_fill(item);
@@ -791,10 +823,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     for (int j = 0; j < R; ++j)
                         load_idx(tc, j, ix[j]); // the padded list keeps every index load in bounds
                     load_idx(tc, R, ix_next);
-#ifdef TW_EXP_TIMING
-                    if (ix_next.k[0] >= 0 && blockIdx.x == 0 && ws_first && threadIdx.x == 256)
-                        s_ws[252] = __builtin_readcyclecounter();
-#endif
 #pragma unroll
                     for (int j = 0; j < R; ++j)
                         if (j < nsteps)
@@ -890,7 +918,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             cur = nxt;
             have_next = false;
 #ifdef TW_EXP_TIMING
-            ws_first = false;
+            ++ws_item;
 #endif
         }
     } else {
@@ -1014,6 +1042,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                         }
                     }
                 }
+                pick_up();
                 TW_LDS_BARRIER(); // the C tile is staged
                 store_tile(u, m0, cur.m_end);
             }
@@ -1021,7 +1050,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             cur = nxt;
             have_next = false;
 #ifdef TW_EXP_TIMING
-            ws_first = false;
+            ++ws_item;
 #endif
         }
 #ifdef TW_EXP_TIMING

@@ -1,4 +1,8 @@
-// The tile-wise-sparse GEMM of libtwgemm: one persistent grouped kernel for gfx950.
+// The tile-wise-sparse GEMM of libtwgemm: persistent grouped kernels for gfx950.  Two K-major
+// kernels share the decomposition and the data path below: tw_gemm_ws_kernel (wave-specialised,
+// the default for wide tiles) and tw_gemm_kmajor_kernel (every wave loads, stages and
+// multiplies; used for narrow tiles and small launches); tw_gemm_generic_kernel takes the other
+// layouts.
 //
 // Work decomposition.  A work item is (unit, m-block): a unit is up to 128
 // compact columns of one weight tile, an m-block is BM consecutive rows of A.

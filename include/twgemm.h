@@ -138,6 +138,13 @@ int tw_plan_create_dense(int K, int N, int G, int dtype, const float *B, tw_plan
 int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask,
                       const float *B, tw_plan **out);
 
+/* The same for an explicit tile table (tiles cover [0,N) in order, without gaps), e.g. the
+ * tiles that end after every G kept columns of tiled_wise_2d
+ * (Pruning/VGG/prune_algo.py:76-88; tw_tiles_every_g_kept_columns below). */
+int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                            const int32_t *tile_width, const uint8_t *mask, const float *B,
+                            tw_plan **out);
+
 /* Build a plan from the operands of the reference's Stream_Gemm_NN
  * (basic_nn.cu:378-393): B_stream is the compacted weight in DEVICE memory in
  * the layout of gen_masked_stream_weight (:757-769; tile t column-major with
@@ -209,6 +216,65 @@ int tw_delete_row(const void *matrix, void *matrix_2, int rows, int columns,
                   const int32_t *mask, void *stream);
 int tw_insert_row(void *matrix, const void *matrix_2, int rows, int columns,
                   const int32_t *mask, void *stream);
+
+/* ---- TW mask producers ---------------------------------------------------------------
+ * The reference derives its masks from importance scores with NumPy: per layer a 2-D score
+ * matrix [K,N] (|w|; conv kernels HWIO reshaped to (H*W*I) x O, Pruning/VGG/prune_algo.py:16-24),
+ * one threshold over the whole network.  These entry points run that on the GPU and return the
+ * same masks bit for bit (every float operation repeats NumPy's, in its order).
+ *   scores[l]   device, fp32 row-major [K[l], N[l]]   (sign is irrelevant, only squares are used)
+ *   masks[l]    device out, one byte per element, 1 = kept
+ * np.percentile computes in the type of its `q`: pass TW_Q_F32 when the reference's caller gives
+ * the sparsity as a Python number (float32 arithmetic on float32 norms), TW_Q_F64 when it is a
+ * NumPy float64.  All layers are processed on `stream`; the calls return after the masks are
+ * complete. */
+#define TW_Q_F32 0
+#define TW_Q_F64 1
+
+/* tiled_wise_1d (Pruning/VGG/prune_algo.py:114-148; BERT pruning type 7,
+ * Pruning/BERT/utils/MyHook.py:226-259): tiles of `granularity` original columns (last one
+ * ragged); norm of every tile row / tile width; the `sparsity`-th percentile of all of them is
+ * the threshold; a tile row is kept iff its norm is strictly above it.  *threshold (optional)
+ * receives the threshold. */
+int tw_prune_tiled_wise_1d(int n_layers, const int32_t *K, const int32_t *N,
+                           const float *const *scores, double sparsity, int q_type,
+                           int granularity, uint8_t *const *masks, double *threshold,
+                           void *stream);
+
+/* tiled_wise_2d (Pruning/VGG/prune_algo.py:55-112; BERT type 8, MyHook.py:261-313): columns
+ * first (column norm / K against the percentile of all column norms), then tiles that end
+ * after every `granularity` kept columns, then tile rows as above on the column-pruned scores
+ * (norm / original tile width); mask = rows x columns.  With transform != 0 the percentile
+ * used for both steps is 100 - sqrt(10000 - 100*sparsity) (prune_algo.py:61, a float64 whatever
+ * q_type says); with 0 it is `sparsity` itself (BERT type 8).  col_masks (optional, device,
+ * N[l] bytes each) receive the column masks, from which tw_tiles_every_g_kept_columns gives the
+ * tile table; thresholds (optional) receives {columns, rows}. */
+int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
+                           const float *const *scores, double sparsity, int q_type, int transform,
+                           int granularity, uint8_t *const *masks, uint8_t *const *col_masks,
+                           double *thresholds, void *stream);
+
+/* The building blocks of the two producers, on device buffers:
+ *   tw_prune_tile_row_norms   norms[t*K + k] = ||scores[k][tile t]|| / width_t in NumPy's float32
+ *                             summation order; col_keep (optional, N bytes) zeroes pruned
+ *                             columns (prune_algo.py:92, 130)
+ *   tw_prune_col_norms        norms[c] = ||scores[:, c]|| / K (prune_algo.py:64)
+ *   tw_percentile_linear      np.percentile(values, q) with linear interpolation, in float32
+ *                             (TW_Q_F32; the result is that float32 widened) or float64 */
+int tw_prune_tile_row_norms(int K, int N, const float *scores, int n_tiles,
+                            const int32_t *tile_col0, const int32_t *tile_width,
+                            const uint8_t *col_keep, float *norms, void *stream);
+int tw_prune_col_norms(int K, int N, const float *scores, float *norms, void *stream);
+int tw_percentile_linear(const float *values, int64_t n, double q, int q_type, double *result,
+                         void *stream);
+
+/* Tile tables (host): every G original columns (prune_algo.py:119-128), and ending after every
+ * G-th kept column, the last tile taking the rest (prune_algo.py:76-88).  tile_col0 and
+ * tile_width need room for N entries. */
+int tw_tiles_every_g_columns(int N, int G, int32_t *tile_col0, int32_t *tile_width,
+                             int32_t *n_tiles);
+int tw_tiles_every_g_kept_columns(int N, int G, const uint8_t *col_mask, int32_t *tile_col0,
+                                  int32_t *tile_width, int32_t *n_tiles);
 
 #ifdef __cplusplus
 }

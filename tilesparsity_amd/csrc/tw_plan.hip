@@ -144,17 +144,19 @@ __global__ void unpack_stream_kernel(const PackTile *tiles, const uint16_t *Bp, 
 // ---------------------------------------------------------------------------------
 // mask -> flags -> lists  (integer pre-pass)
 
-// rowflag[t*K + k] = any byte of mask[k][t*G .. t*G+w) is non-zero
-__global__ void row_flags_kernel(const uint8_t *mask, int K, int N, int G, int n_tiles,
-                                 uint8_t *rowflag)
+// The tile table on the device: tcol0[t] is the first column of tile t, tcol0[n_tiles] == N.
+
+// rowflag[t*K + k] = any byte of mask[k][tcol0[t] .. tcol0[t+1]) is non-zero
+__global__ void row_flags_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0,
+                                 int n_tiles, uint8_t *rowflag)
 {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (int64_t)K * n_tiles)
         return;
     const int t = (int)(idx % n_tiles);
     const int k = (int)(idx / n_tiles);
-    const int c0 = t * G;
-    const int w = min(G, N - c0);
+    const int c0 = tcol0[t];
+    const int w = tcol0[t + 1] - c0;
     const uint8_t *row = mask + (int64_t)k * N + c0;
     uint32_t any = 0;
     for (int j = 0; j < w; ++j)
@@ -178,8 +180,8 @@ __global__ void col_flags_kernel(const uint8_t *mask, int K, int N, uint32_t *co
 }
 
 // counts the elements where mask != rowflag & colflag (a TW mask has none)
-__global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, int G,
-                                   const uint8_t *rowflag, const uint32_t *colflag,
+__global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0,
+                                   int n_tiles, const uint8_t *rowflag, const uint32_t *colflag,
                                    unsigned long long *mismatch)
 {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -187,7 +189,15 @@ __global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, int G,
         return;
     const int c = (int)(idx % N);
     const int k = (int)(idx / N);
-    const int t = c / G;
+    int lo = 0, hi = n_tiles; // the tile with tcol0[t] <= c < tcol0[t+1]
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (tcol0[mid] <= c)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    const int t = lo;
     const bool m = mask[idx] != 0;
     const bool e = rowflag[(int64_t)t * K + k] && colflag[c];
     if (m != e)
@@ -195,8 +205,8 @@ __global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, int G,
 }
 
 // counts[t] = kept rows of tile t, counts[n_tiles + t] = kept columns of tile t
-__global__ void count_flags_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K, int N,
-                                   int G, int n_tiles, int32_t *counts)
+__global__ void count_flags_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K,
+                                   const int32_t *tcol0, int n_tiles, int32_t *counts)
 {
     __shared__ int s_sum[2];
     const int t = blockIdx.x;
@@ -208,7 +218,7 @@ __global__ void count_flags_kernel(const uint8_t *rowflag, const uint32_t *colfl
     int rk = 0, ck = 0;
     for (int k = threadIdx.x; k < K; k += blockDim.x)
         rk += rowflag[(int64_t)t * K + k];
-    const int c0 = t * G, w = min(G, N - c0);
+    const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
     for (int j = threadIdx.x; j < w; j += blockDim.x)
         ck += colflag[c0 + j] ? 1 : 0;
     atomicAdd(&s_sum[0], rk);
@@ -257,15 +267,15 @@ __device__ void block_compact(const uint8_t *flag8, const uint32_t *flag32, int 
 
 // grid (n_tiles, 2): y == 0 rows, y == 1 columns
 __global__ void __launch_bounds__(256)
-    compact_lists_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K, int N, int G,
-                         const int32_t *k_ptr, const int32_t *n_ptr, int32_t *kept_k,
-                         int32_t *rel_k, int32_t *kept_n, int32_t *rel_n)
+    compact_lists_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K,
+                         const int32_t *tcol0, const int32_t *k_ptr, const int32_t *n_ptr,
+                         int32_t *kept_k, int32_t *rel_k, int32_t *kept_n, int32_t *rel_n)
 {
     const int t = blockIdx.x;
     if (blockIdx.y == 0) {
         block_compact(rowflag + (int64_t)t * K, nullptr, K, kept_k + k_ptr[t], rel_k + k_ptr[t]);
     } else {
-        const int c0 = t * G, w = min(G, N - c0);
+        const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
         block_compact(nullptr, colflag + c0, w, kept_n + n_ptr[t], rel_n + n_ptr[t]);
     }
 }
@@ -600,21 +610,55 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
+    if (K <= 0 || N <= 0 || G <= 0)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d G=%d must all be positive", K, N, G);
+    const int nt = (N + G - 1) / G;
+    std::vector<int32_t> col0(nt), width(nt);
+    for (int t = 0; t < nt; ++t) {
+        col0[t] = t * G;
+        width[t] = std::min(G, N - t * G);
+    }
+    return tw_plan_from_mask_tiles(K, N, dtype, nt, col0.data(), width.data(), mask, B, out);
+}
+
+int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                            const int32_t *tile_width, const uint8_t *mask, const float *B,
+                            tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
     int st = check_dtype(dtype);
     if (st)
         return st;
-    if (K <= 0 || N <= 0 || G <= 0)
-        return fail(TW_ERR_SHAPE, "K=%d N=%d G=%d must all be positive", K, N, G);
-    if (!mask || !B)
-        return fail(TW_ERR_NULL, "mask or B is NULL");
-    const int nt = (N + G - 1) / G;
+    if (K <= 0 || N <= 0 || n_tiles <= 0)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d n_tiles=%d must all be positive", K, N, n_tiles);
+    if (!mask || !B || !tile_col0 || !tile_width)
+        return fail(TW_ERR_NULL, "mask, B or the tile table is NULL");
+    const int nt = n_tiles;
+    std::vector<int32_t> tcol0(nt + 1);
+    {
+        int c = 0;
+        for (int t = 0; t < nt; ++t) {
+            if (tile_col0[t] != c || tile_width[t] <= 0)
+                return fail(TW_ERR_TILE_TABLE,
+                            "tile %d: col0=%d width=%d, tiles must cover [0,N) in order without gaps",
+                            t, tile_col0[t], tile_width[t]);
+            tcol0[t] = c;
+            c += tile_width[t];
+        }
+        if (c != N)
+            return fail(TW_ERR_TILE_TABLE, "tiles cover %d columns, N=%d", c, N);
+        tcol0[nt] = N;
+    }
 
     uint8_t *d_mask = nullptr, *d_rowflag = nullptr;
     uint32_t *d_colflag = nullptr;
     unsigned long long *d_mismatch = nullptr;
-    int32_t *d_counts = nullptr, *d_kptr = nullptr, *d_nptr = nullptr;
+    int32_t *d_counts = nullptr, *d_kptr = nullptr, *d_nptr = nullptr, *d_tcol0 = nullptr;
     tw_plan *p = nullptr;
     auto cleanup = [&]() {
+        hipFree(d_tcol0);
         hipFree(d_mask);
         hipFree(d_rowflag);
         hipFree(d_colflag);
@@ -639,6 +683,8 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     TW_TRY(hipMalloc((void **)&d_colflag, sizeof(uint32_t) * N));
     TW_TRY(hipMalloc((void **)&d_mismatch, sizeof(unsigned long long)));
     TW_TRY(hipMalloc((void **)&d_counts, sizeof(int32_t) * 2 * nt));
+    TW_TRY(hipMalloc((void **)&d_tcol0, sizeof(int32_t) * (nt + 1)));
+    TW_TRY(hipMemcpy(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
     TW_TRY(hipMemcpy(d_mask, mask, mask_bytes, hipMemcpyHostToDevice));
     TW_TRY(hipMemset(d_colflag, 0, sizeof(uint32_t) * N));
     TW_TRY(hipMemset(d_mismatch, 0, sizeof(unsigned long long)));
@@ -646,14 +692,14 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     {
         const int64_t n_rt = (int64_t)K * nt;
         hipLaunchKernelGGL(row_flags_kernel, dim3((unsigned)((n_rt + 255) / 256)), dim3(256), 0,
-                           nullptr, d_mask, K, N, G, nt, d_rowflag);
+                           nullptr, d_mask, K, N, d_tcol0, nt, d_rowflag);
         hipLaunchKernelGGL(col_flags_kernel, dim3((N + 255) / 256, (K + 63) / 64), dim3(256), 0,
                            nullptr, d_mask, K, N, d_colflag);
         const int64_t n_el = (int64_t)K * N;
         hipLaunchKernelGGL(validate_tw_kernel, dim3((unsigned)((n_el + 255) / 256)), dim3(256), 0,
-                           nullptr, d_mask, K, N, G, d_rowflag, d_colflag, d_mismatch);
+                           nullptr, d_mask, K, N, d_tcol0, nt, d_rowflag, d_colflag, d_mismatch);
         hipLaunchKernelGGL(count_flags_kernel, dim3(nt), dim3(256), 0, nullptr, d_rowflag,
-                           d_colflag, K, N, G, nt, d_counts);
+                           d_colflag, K, d_tcol0, nt, d_counts);
         TW_TRY(hipGetLastError());
     }
     unsigned long long mismatch = 0;
@@ -663,8 +709,8 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     if (mismatch != 0) {
         cleanup();
         return fail(TW_ERR_NOT_TW,
-                    "%llu mask elements differ from (row kept) & (column kept) for G=%d", mismatch,
-                    G);
+                    "%llu mask elements differ from (row kept) & (column kept) of their tile",
+                    mismatch);
     }
 
     p = new (std::nothrow) tw_plan;
@@ -681,8 +727,8 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     p->kept_k_ptr.assign(nt + 1, 0);
     p->kept_n_ptr.assign(nt + 1, 0);
     for (int t = 0; t < nt; ++t) {
-        p->tile_col0[t] = t * G;
-        p->tile_width[t] = std::min(G, N - t * G);
+        p->tile_col0[t] = tile_col0[t];
+        p->tile_width[t] = tile_width[t];
         p->kept_k_ptr[t + 1] = p->kept_k_ptr[t] + counts[t];
         p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + counts[nt + t];
     }
@@ -696,7 +742,7 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     TW_TRY(hipMalloc((void **)&p->d_kept_n, sizeof(int32_t) * sn));
     TW_TRY(hipMalloc((void **)&p->d_rel_n, sizeof(int32_t) * sn));
     hipLaunchKernelGGL(compact_lists_kernel, dim3(nt, 2), dim3(256), 0, nullptr, d_rowflag,
-                       d_colflag, K, N, G, d_kptr, d_nptr, p->d_kept_k, p->d_rel_k, p->d_kept_n,
+                       d_colflag, K, d_tcol0, d_kptr, d_nptr, p->d_kept_k, p->d_rel_k, p->d_kept_n,
                        p->d_rel_n);
     TW_TRY(hipGetLastError());
     p->kept_k_idx.resize(p->kept_k_ptr[nt]);

@@ -37,6 +37,9 @@ EXPORTED_SYMBOLS = (
     "tw_plan_create", "tw_plan_create_dense", "tw_plan_from_mask",
     "tw_plan_from_stream_operands", "tw_plan_info", "tw_plan_export", "tw_plan_destroy",
     "tw_gemm", "tw_stream_gemm_nn", "tw_cast_f32", "tw_delete_row", "tw_insert_row",
+    "tw_plan_from_mask_tiles", "tw_prune_tiled_wise_1d", "tw_prune_tiled_wise_2d",
+    "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
+    "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear",
 )
 
 
@@ -112,6 +115,18 @@ def lib():
         "tw_cast_f32": (c_int, [vp, vp, c_i64, c_int, vp]),
         "tw_delete_row": (c_int, [vp, vp, c_int, c_int, vp, vp]),
         "tw_insert_row": (c_int, [vp, vp, c_int, c_int, vp, vp]),
+        "tw_plan_from_mask_tiles": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
+        "tw_prune_tiled_wise_1d": (c_int, [c_int, i32p, i32p, pp, ctypes.c_double, c_int, c_int,
+                                           pp, ctypes.POINTER(ctypes.c_double), vp]),
+        "tw_prune_tiled_wise_2d": (c_int, [c_int, i32p, i32p, pp, ctypes.c_double, c_int, c_int,
+                                           c_int, pp, pp, ctypes.POINTER(ctypes.c_double), vp]),
+        "tw_tiles_every_g_columns": (c_int, [c_int, c_int, i32p, i32p, ctypes.POINTER(c_int)]),
+        "tw_prune_tile_row_norms": (c_int, [c_int, c_int, vp, c_int, i32p, i32p, vp, vp, vp]),
+        "tw_prune_col_norms": (c_int, [c_int, c_int, vp, vp, vp]),
+        "tw_percentile_linear": (c_int, [vp, c_i64, ctypes.c_double, c_int,
+                                         ctypes.POINTER(ctypes.c_double), vp]),
+        "tw_tiles_every_g_kept_columns": (c_int, [c_int, c_int, u8p, i32p, i32p,
+                                                  ctypes.POINTER(c_int)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -247,6 +262,23 @@ class Plan:
         h = ctypes.c_void_p()
         _check(lib().tw_plan_from_mask(K, N, G, dtype_code(dtype), _ptr(mask, ctypes.c_uint8),
                                        _ptr(B, ctypes.c_float), ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def from_mask_tiles(cls, mask, tile_table, dtype, B):
+        """From a dense 0/1 mask [K,N] and an explicit tile table [(col0, width), ...]."""
+        mask = np.ascontiguousarray(mask, dtype=np.uint8)
+        K, N = mask.shape
+        B = np.ascontiguousarray(B, dtype=np.float32)
+        if B.size != K * N:
+            raise TwError(ERR_SHAPE, "B has %d elements, expected K*N=%d" % (B.size, K * N))
+        col0 = _i32([t[0] for t in tile_table])
+        width = _i32([t[1] for t in tile_table])
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_from_mask_tiles(K, N, dtype_code(dtype), len(tile_table),
+                                             _ptr(col0, ctypes.c_int32), _ptr(width, ctypes.c_int32),
+                                             _ptr(mask, ctypes.c_uint8), _ptr(B, ctypes.c_float),
+                                             ctypes.byref(h)))
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod

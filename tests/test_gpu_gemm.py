@@ -65,6 +65,8 @@ CASES = [
     (64, 512, 130, 128, 0.1, 0.5, 0),     # last tile 2 columns wide
     (257, 64, 96, 32, 0.5, 0.75, 2),      # G = 32
     (192, 200, 512, 256, 0.3, 0.9, 0),    # tiles wider than one work unit
+    (300, 96, 5120, 128, 0.5, 1.0, 7),    # more units than fit the kernel-argument table
+    (2048, 64, 4224, 128, 0.6, 0.9, 0),   # several items per workgroup, one 64-row step each
 ]
 
 

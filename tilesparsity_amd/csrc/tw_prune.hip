@@ -108,15 +108,30 @@ __global__ void tile_row_norms_kernel(const float *score, int K, int N, const in
     norms[(int64_t)t * K + k] = sqrtf(s) / (float)w; // both correctly rounded (compiler default)
 }
 
-// cnorm[c] = ||score[:, c]|| / K, the rows accumulated in order
+// cnorm[c] = ||score[:, c]|| / K, the rows accumulated in order.  The chain of additions is
+// sequential by definition; the loads are not, so they are issued 32 rows at a time.
 __global__ void col_norms_kernel(const float *score, int K, int N, float *cnorm)
 {
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= N)
         return;
+    constexpr int U = 32;
+    const float *p = score + c;
     float acc = 0.0f;
-    for (int k = 0; k < K; ++k) {
-        const float v = score[(int64_t)k * N + c];
+    int k = 0;
+    for (; k + U <= K; k += U) {
+        float v[U];
+#pragma unroll
+        for (int j = 0; j < U; ++j)
+            v[j] = p[(int64_t)(k + j) * N];
+#pragma unroll
+        for (int j = 0; j < U; ++j) {
+            const float sq = v[j] * v[j];
+            acc = acc + sq;
+        }
+    }
+    for (; k < K; ++k) {
+        const float v = p[(int64_t)k * N];
         const float sq = v * v;
         acc = acc + sq;
     }
@@ -172,10 +187,29 @@ __global__ void __launch_bounds__(256)
         else
             mn = min(mn, key);
     }
-    if (cnt)
-        atomicAdd(count_le, cnt);
-    if (mn != 0xFFFFFFFFu)
-        atomicMin(min_gt, mn);
+    // one pair of atomics per workgroup
+    __shared__ unsigned long long s_cnt;
+    __shared__ unsigned int s_min;
+    if (threadIdx.x == 0) {
+        s_cnt = 0;
+        s_min = 0xFFFFFFFFu;
+    }
+    __syncthreads();
+    for (int off = 32; off > 0; off >>= 1) {
+        cnt += __shfl_down(cnt, off);
+        mn = min(mn, (unsigned int)__shfl_down(mn, off));
+    }
+    if ((threadIdx.x & 63) == 0) {
+        atomicAdd(&s_cnt, cnt);
+        atomicMin(&s_min, mn);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        if (s_cnt)
+            atomicAdd(count_le, s_cnt);
+        if (s_min != 0xFFFFFFFFu)
+            atomicMin(min_gt, s_min);
+    }
 }
 
 // keep[c] = cnorm[c] > threshold

@@ -135,6 +135,76 @@ def cpu_baseline(wl, A, B, budget_s=20.0):
                        % (rows, M, len(times), t))
 
 
+# VGG16's 13 conv layers as im2col score matrices (H*W*I) x O, plus a 4096 x 4096 dense layer
+PRODUCER_LAYERS = [(27, 64), (576, 64), (576, 128), (1152, 128), (1152, 256), (2304, 256),
+                   (2304, 256), (2304, 512), (4608, 512), (4608, 512), (4608, 512), (4608, 512),
+                   (4608, 512), (4096, 4096)]
+
+
+def bench_producers(steps, warmup, torch):
+    """The TW mask producers (tiled_wise_1d / tiled_wise_2d at 75 % sparsity, G=128) on a
+    VGG16-sized list of score matrices resident in HBM; the NumPy oracle is the CPU baseline."""
+    import ctypes
+    from tilesparsity_amd import twgemm as tw
+    from tilesparsity_amd import twprune
+    from oracle import tw_prune_oracle as po
+    rng = np.random.default_rng(20200615)
+    scores = [np.abs(rng.standard_normal(s)).astype(np.float32) for s in PRODUCER_LAYERS]
+    elems = sum(k * n for k, n in PRODUCER_LAYERS)
+    d = twprune._DeviceLayers(scores)
+    L = tw.lib()
+    pp = ctypes.POINTER(ctypes.c_void_p)
+    i32 = ctypes.c_int32
+
+    def run1d():
+        thr = ctypes.c_double()
+        tw._check(L.tw_prune_tiled_wise_1d(len(d.shapes), tw._ptr(d.K, i32), tw._ptr(d.N, i32),
+                                           ctypes.cast(d.p_scores, pp), 75.0, 0, 128,
+                                           ctypes.cast(d.p_masks, pp), ctypes.byref(thr), d.stream))
+
+    def run2d():
+        thr = (ctypes.c_double * 2)()
+        tw._check(L.tw_prune_tiled_wise_2d(len(d.shapes), tw._ptr(d.K, i32), tw._ptr(d.N, i32),
+                                           ctypes.cast(d.p_scores, pp), 75.0, 0, 1, 128,
+                                           ctypes.cast(d.p_masks, pp), ctypes.cast(d.p_cols, pp),
+                                           thr, d.stream))
+
+    out = {}
+    for name, fn, passes in (("tiled_wise_1d", run1d, 1), ("tiled_wise_2d", run2d, 2)):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()                      # every call returns with its masks complete
+        t = (time.perf_counter() - t0) / steps
+        by = elems * (4 * passes + 1)  # scores read once per stage, one mask byte written
+        out[name] = dict(ms=t * 1e3, algorithmic_bytes=by, gbs=by / t / 1e9)
+    t0 = time.perf_counter()
+    po.tiled_wise_1d(scores, 75.0, 128)
+    t1 = time.perf_counter()
+    po.tiled_wise_2d(scores, 75.0, 128)
+    t2 = time.perf_counter()
+    one = out["tiled_wise_1d"]
+    return {
+        "metric": "TW mask producer throughput (tiled_wise_1d, 14 VGG16-sized layers, 75 %, G=128)",
+        "value": one["gbs"], "unit": "GB/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": one["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "mask producers, %d layers, %.1f M score elements" % (
+            len(PRODUCER_LAYERS), elems / 1e6)},
+        "tiled_wise_2d": out["tiled_wise_2d"],
+        "roofline": {"bound": "hbm", "achieved": one["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": one["gbs"] / HBM_PEAK_GBS, "traffic": None,
+                     "algorithmic_bytes": one["algorithmic_bytes"]},
+        "cpu_baseline": {"value": elems * 5 / (t1 - t0) / 1e9, "unit": "GB/s", "cores": 1,
+                         "kind": "port",
+                         "sample": "NumPy oracle on the same layers: tiled_wise_1d %.1f ms, "
+                                   "tiled_wise_2d %.1f ms (one run each)" % ((t1 - t0) * 1e3,
+                                                                             (t2 - t1) * 1e3)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -143,6 +213,8 @@ def main():
     ap.add_argument("--workload", default="vgg16_conv4_2")
     ap.add_argument("--all", action="store_true", help="also run the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--producers", action="store_true",
+                    help="benchmark the TW mask producers instead of the GEMM (one JSON line)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (4 launches over rotating buffers), "
                          "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
@@ -158,6 +230,9 @@ def main():
         return 1
     from tilesparsity_amd import twgemm as tw
     tw.lib()  # fails loudly if the HIP library has not been built
+    if args.producers:
+        print(json.dumps(bench_producers(min(args.steps, 20), min(args.warmup, 3), torch)), flush=True)
+        return 0
 
     if args.copy_calibration:
         n = (256 << 20) // 4

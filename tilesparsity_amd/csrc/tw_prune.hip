@@ -21,6 +21,7 @@
 
 #include <cmath>
 #include <cstring>
+#include <mutex>
 
 #pragma clang fp contract(off)
 
@@ -32,8 +33,11 @@ __device__ __forceinline__ float sq_term(const float *x, const uint8_t *keep, in
     return v * v;
 }
 
-// NumPy's pairwise sum for n <= 128 terms
-__device__ float pairwise_block(const float *x, const uint8_t *keep, int n)
+// NumPy's pairwise sum for n <= 128 terms, by a group of 8 adjacent lanes: lane j keeps NumPy's
+// running sum r[j] (terms j, j+8, j+16, ...), the three shuffle steps are NumPy's
+// ((r0+r1)+(r2+r3)) + ((r4+r5)+(r6+r7)), lane 0 then adds the n % 8 trailing terms.  The result
+// is valid in lane 0 of the group.
+__device__ float pairwise_block(const float *x, const uint8_t *keep, int n, int l8)
 {
     if (n < 8) {
         float r = 0.0f;
@@ -41,27 +45,23 @@ __device__ float pairwise_block(const float *x, const uint8_t *keep, int n)
             r = r + sq_term(x, keep, i);
         return r;
     }
-    float r[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j)
-        r[j] = sq_term(x, keep, j);
+    float r = sq_term(x, keep, l8);
     int i = 8;
-    for (; i < n - (n % 8); i += 8) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            r[j] = r[j] + sq_term(x, keep, i + j);
-    }
-    float res = ((r[0] + r[1]) + (r[2] + r[3])) + ((r[4] + r[5]) + (r[6] + r[7]));
+    for (; i < n - (n % 8); i += 8)
+        r = r + sq_term(x, keep, i + l8);
+    r = r + __shfl_down(r, 1, 8);
+    r = r + __shfl_down(r, 2, 8);
+    r = r + __shfl_down(r, 4, 8);
     for (; i < n; ++i)
-        res = res + sq_term(x, keep, i);
-    return res;
+        r = r + sq_term(x, keep, i);
+    return r;
 }
 
 // ... and for any n: halves (the first a multiple of 8) are summed separately and added
-__device__ float pairwise_sq_sum(const float *x, const uint8_t *keep, int n)
+__device__ float pairwise_sq_sum(const float *x, const uint8_t *keep, int n, int l8)
 {
     if (n <= 128)
-        return pairwise_block(x, keep, n);
+        return pairwise_block(x, keep, n, l8);
     struct Frame {
         int off, n, stage;
         float left;
@@ -73,7 +73,7 @@ __device__ float pairwise_sq_sum(const float *x, const uint8_t *keep, int n)
     while (sp > 0) {
         Frame &f = st[sp - 1];
         if (f.n <= 128) {
-            ret = pairwise_block(x + f.off, keep ? keep + f.off : nullptr, f.n);
+            ret = pairwise_block(x + f.off, keep ? keep + f.off : nullptr, f.n, l8);
             --sp;
             continue;
         }
@@ -94,29 +94,79 @@ __device__ float pairwise_sq_sum(const float *x, const uint8_t *keep, int n)
     return ret;
 }
 
-// norms[t*K + k] = ||score[k][tcol0[t] .. tcol0[t+1])|| / width, pruned columns counting as 0
-__global__ void tile_row_norms_kernel(const float *score, int K, int N, const int32_t *tcol0,
-                                      int n_tiles, const uint8_t *colkeep, float *norms)
+// One entry per layer of a producer call; all layers run in one launch per stage.
+struct PruneLayer {
+    const float *score;
+    uint8_t *mask;
+    const uint8_t *colkeep; // nullptr: every column counts
+    const int32_t *tcol0;   // n_tiles + 1 entries
+    float *norms;           // [n_tiles][K]
+    int32_t K, N, n_tiles, pad_;
+    int64_t rt_begin;       // first (row, tile) pair of this layer in the launch-wide numbering
+    int64_t el_begin;       // first 16-column chunk likewise (ceil(N/16) chunks per row)
+};
+
+__device__ __forceinline__ int find_layer(const PruneLayer *layers, int n_layers, int64_t idx,
+                                          bool by_elements)
 {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)K * n_tiles)
-        return;
-    const int t = (int)(idx % n_tiles);
-    const int k = (int)(idx / n_tiles);
-    const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
-    const float s = pairwise_sq_sum(score + (int64_t)k * N + c0, colkeep ? colkeep + c0 : nullptr, w);
-    norms[(int64_t)t * K + k] = sqrtf(s) / (float)w; // both correctly rounded (compiler default)
+    int lo = 0, hi = n_layers;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if ((by_elements ? layers[mid].el_begin : layers[mid].rt_begin) <= idx)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
 }
 
-// cnorm[c] = ||score[:, c]|| / K, the rows accumulated in order.  The chain of additions is
-// sequential by definition; the loads are not, so they are issued 32 rows at a time.
-__global__ void col_norms_kernel(const float *score, int K, int N, float *cnorm)
+// norms[t*K + k] = ||score[k][tcol0[t] .. tcol0[t+1])|| / width, pruned columns counting as 0;
+// 8 lanes per (row, tile), neighbouring groups take neighbouring tiles of a row
+__global__ void __launch_bounds__(256)
+    tile_row_norms_kernel(const PruneLayer *layers, int n_layers, int64_t n_pairs)
 {
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= N)
+    const int64_t gid = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) >> 3;
+    const int l8 = threadIdx.x & 7;
+    if (gid >= n_pairs)
+        return; // whole groups leave together
+    const PruneLayer L = layers[find_layer(layers, n_layers, gid, false)];
+    const int64_t idx = gid - L.rt_begin;
+    const int t = (int)(idx % L.n_tiles);
+    const int k = (int)(idx / L.n_tiles);
+    const int c0 = L.tcol0[t], w = L.tcol0[t + 1] - c0;
+    const float s = pairwise_sq_sum(L.score + (int64_t)k * L.N + c0,
+                                    L.colkeep ? L.colkeep + c0 : nullptr, w, l8);
+    if (l8 == 0)
+        L.norms[(int64_t)t * L.K + k] = sqrtf(s) / (float)w; // both correctly rounded
+}
+
+// One entry per layer for the column stage.
+struct ColLayer {
+    const float *score;
+    int32_t K, N;
+    int64_t col_begin; // first column of this layer in the pooled numbering
+};
+
+// cnorm[pooled c] = ||score[:, c]|| / K, the rows accumulated in order.  The chain of additions
+// is sequential by definition; the loads are not, so they are issued 32 rows at a time, and all
+// layers share one launch.
+__global__ void col_norms_kernel(const ColLayer *layers, int n_layers, int64_t n_cols, float *cnorm)
+{
+    const int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (g >= n_cols)
         return;
+    int lo = 0, hi = n_layers;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (layers[mid].col_begin <= g)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    const ColLayer L = layers[lo];
+    const int K = L.K, N = L.N;
     constexpr int U = 32;
-    const float *p = score + c;
+    const float *p = L.score + (g - L.col_begin);
     float acc = 0.0f;
     int k = 0;
     for (; k + U <= K; k += U) {
@@ -135,7 +185,7 @@ __global__ void col_norms_kernel(const float *score, int K, int N, float *cnorm)
         const float sq = v * v;
         acc = acc + sq;
     }
-    cnorm[c] = sqrtf(acc) / (float)K;
+    cnorm[g] = sqrtf(acc) / (float)K;
 }
 
 // order-preserving map float -> uint32
@@ -144,23 +194,41 @@ __device__ __forceinline__ uint32_t sort_key(float v)
     const uint32_t b = __float_as_uint(v);
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
-static float key_value(uint32_t key)
+// Selection state in device memory, so that the passes follow each other on the stream without
+// a host round trip.
+struct SelectState {
+    unsigned long long hist[256];
+    unsigned long long rank;      // rank still to find among the values matching the prefix
+    unsigned long long count_le;  // values <= the k-th smallest
+    uint32_t prefix, mask;        // key bits fixed so far
+    uint32_t min_gt;              // smallest key above the k-th smallest's (0xFFFFFFFF: none)
+    int32_t lost;                 // set if a pass found no digit (cannot happen for rank < n)
+    float thr32;                  // the threshold, for the kernels that follow
+    double thr64;
+};
+
+__global__ void select_init_kernel(SelectState *st, unsigned long long rank)
 {
-    const uint32_t b = (key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key;
-    float v;
-    std::memcpy(&v, &b, 4);
-    return v;
+    st->hist[threadIdx.x] = 0;
+    if (threadIdx.x == 0) {
+        st->rank = rank;
+        st->count_le = 0;
+        st->prefix = 0;
+        st->mask = 0;
+        st->min_gt = 0xFFFFFFFFu;
+        st->lost = 0;
+    }
 }
 
-// hist[d] = number of values whose key matches `prefix` in the bits of `mask` and has digit d
+// hist[d] += number of values whose key matches the prefix in the masked bits and has digit d
 // at `shift`
 __global__ void __launch_bounds__(256)
-    select_hist_kernel(const float *v, int64_t n, uint32_t mask, uint32_t prefix, int shift,
-                       unsigned long long *hist)
+    select_hist_kernel(const float *v, int64_t n, int shift, SelectState *st)
 {
     __shared__ unsigned int s_h[256];
     s_h[threadIdx.x] = 0;
     __syncthreads();
+    const uint32_t mask = st->mask, prefix = st->prefix;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
          i += (int64_t)gridDim.x * blockDim.x) {
         const uint32_t key = sort_key(v[i]);
@@ -169,14 +237,38 @@ __global__ void __launch_bounds__(256)
     }
     __syncthreads();
     if (s_h[threadIdx.x])
-        atomicAdd(&hist[threadIdx.x], (unsigned long long)s_h[threadIdx.x]);
+        atomicAdd(&st->hist[threadIdx.x], (unsigned long long)s_h[threadIdx.x]);
 }
 
-// out[0] = number of values <= a, out[1] = smallest key above a's (0xFFFFFFFF if none)
-__global__ void __launch_bounds__(256)
-    rank_stats_kernel(const float *v, int64_t n, uint32_t key_a, unsigned long long *count_le,
-                      unsigned int *min_gt)
+// one workgroup: picks the digit that holds the rank, fixes it in the prefix, clears the histogram
+__global__ void __launch_bounds__(256) select_digit_kernel(int shift, SelectState *st)
 {
+    __shared__ unsigned long long s_c[256];
+    s_c[threadIdx.x] = st->hist[threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long rank = st->rank;
+        int d = 0;
+        for (; d < 256; ++d) {
+            if (rank < s_c[d])
+                break;
+            rank -= s_c[d];
+        }
+        if (d == 256) {
+            st->lost = 1;
+            d = 255;
+        }
+        st->rank = rank;
+        st->prefix |= (uint32_t)d << shift;
+        st->mask |= 255u << shift;
+    }
+    st->hist[threadIdx.x] = 0;
+}
+
+// count_le = number of values <= the selected one, min_gt = smallest key above it
+__global__ void __launch_bounds__(256) rank_stats_kernel(const float *v, int64_t n, SelectState *st)
+{
+    const uint32_t key_a = st->prefix;
     unsigned long long cnt = 0;
     unsigned int mn = 0xFFFFFFFFu;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -206,44 +298,103 @@ __global__ void __launch_bounds__(256)
     __syncthreads();
     if (threadIdx.x == 0) {
         if (s_cnt)
-            atomicAdd(count_le, s_cnt);
+            atomicAdd(&st->count_le, s_cnt);
         if (s_min != 0xFFFFFFFFu)
-            atomicMin(min_gt, s_min);
+            atomicMin(&st->min_gt, s_min);
+    }
+}
+
+__device__ __forceinline__ float key_to_float(uint32_t key)
+{
+    return __uint_as_float((key & 0x80000000u) ? (key & 0x7FFFFFFFu) : ~key);
+}
+
+// NumPy's two-sided linear interpolation between the k-th smallest value a and its upper
+// neighbour b (a again if it is repeated, or if the index is the last one): float32 throughout
+// for a float32 gamma, float64 with a float32 difference b - a otherwise.
+__global__ void select_lerp_kernel(SelectState *st, unsigned long long k, int top, int f64,
+                                   float gamma32, double gamma64)
+{
+    const float a = key_to_float(st->prefix);
+    float b = a;
+    if (!top && st->count_le <= k + 1 && st->min_gt != 0xFFFFFFFFu)
+        b = key_to_float(st->min_gt);
+    const float diff = b - a;
+    if (f64) {
+        const double prod = gamma64 >= 0.5 ? (double)diff * (1.0 - gamma64) : (double)diff * gamma64;
+        const double r = gamma64 >= 0.5 ? (double)b - prod : (double)a + prod;
+        st->thr64 = r;
+        st->thr32 = (float)r;
+    } else {
+        const float prod = gamma32 >= 0.5f ? diff * (1.0f - gamma32) : diff * gamma32;
+        const float r = gamma32 >= 0.5f ? b - prod : a + prod;
+        st->thr32 = r;
+        st->thr64 = (double)r;
     }
 }
 
 // keep[c] = cnorm[c] > threshold
-__global__ void col_keep_kernel(const float *cnorm, int N, float thr32, double thr64, int f64,
+__global__ void col_keep_kernel(const float *cnorm, int N, const SelectState *st, int f64,
                                 uint8_t *keep)
 {
+    const float thr32 = st->thr32;
+    const double thr64 = st->thr64;
     const int c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c < N)
         keep[c] = (f64 ? (double)cnorm[c] > thr64 : cnorm[c] > thr32) ? 1 : 0;
 }
 
-// mask[k][c] = (norm of row k in c's tile > threshold) and column c kept
-__global__ void fill_mask_kernel(const float *norms, int K, int N, const int32_t *tcol0,
-                                 int n_tiles, const uint8_t *colkeep, float thr32, double thr64,
-                                 int f64, uint8_t *mask)
+// mask[k][c] = (norm of row k in c's tile > threshold) and column c kept.  One thread per 16
+// consecutive columns of a row: one 16-byte store where the chunk is whole and aligned.
+__global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t n_chunks,
+                                 const SelectState *st, int f64)
 {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)K * N)
+    const float thr32 = st->thr32;
+    const double thr64 = st->thr64;
+    const int64_t gidx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gidx >= n_chunks)
         return;
-    const int c = (int)(idx % N);
-    const int k = (int)(idx / N);
-    int lo = 0, hi = n_tiles;
-    while (hi - lo > 1) {
-        const int mid = (lo + hi) >> 1;
-        if (tcol0[mid] <= c)
-            lo = mid;
+    const PruneLayer L = layers[find_layer(layers, n_layers, gidx, true)];
+    const int64_t idx = gidx - L.el_begin;
+    const int cpr = (L.N + 15) >> 4; // chunks per row
+    const int k = (int)(idx / cpr);
+    const int c0 = (int)(idx - (int64_t)k * cpr) << 4;
+    int t = 0, hi = L.n_tiles;
+    while (hi - t > 1) {
+        const int mid = (t + hi) >> 1;
+        if (L.tcol0[mid] <= c0)
+            t = mid;
         else
             hi = mid;
     }
-    const float nv = norms[(int64_t)lo * K + k];
-    bool keep = f64 ? (double)nv > thr64 : nv > thr32;
-    if (colkeep)
-        keep = keep && colkeep[c];
-    mask[idx] = keep ? 1 : 0;
+    int t_end = L.tcol0[t + 1];
+    float nv = L.norms[(int64_t)t * L.K + k];
+    bool row_keep = f64 ? (double)nv > thr64 : nv > thr32;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    const int n = min(16, L.N - c0);
+    for (int e = 0; e < n; ++e) {
+        const int c = c0 + e;
+        if (c >= t_end) {
+            ++t;
+            t_end = L.tcol0[t + 1];
+            nv = L.norms[(int64_t)t * L.K + k];
+            row_keep = f64 ? (double)nv > thr64 : nv > thr32;
+        }
+        const bool keep = row_keep && (!L.colkeep || L.colkeep[c]);
+        w[e >> 2] |= (keep ? 1u : 0u) << ((e & 3) * 8);
+    }
+    uint8_t *dst = L.mask + (int64_t)k * L.N + c0;
+    if (n == 16 && (((uintptr_t)dst) & 15) == 0) {
+        uint4 v;
+        v.x = w[0];
+        v.y = w[1];
+        v.z = w[2];
+        v.w = w[3];
+        *reinterpret_cast<uint4 *>(dst) = v;
+    } else {
+        for (int e = 0; e < n; ++e)
+            dst[e] = (uint8_t)(w[e >> 2] >> ((e & 3) * 8));
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -251,69 +402,64 @@ __global__ void fill_mask_kernel(const float *norms, int K, int N, const int32_t
 
 namespace {
 
-struct DevBuf {
-    void *p = nullptr;
-    ~DevBuf() { hipFree(p); }
-    template <class T> T *as() { return static_cast<T *>(p); }
+// Temporaries of one producer call come from a process-wide device buffer that only grows, so
+// that a steady stream of calls does not pay for hipMalloc / hipFree.  The arena holds the
+// buffer's lock for the duration of the call (producer calls are serialised).
+std::mutex g_ws_mutex;
+void *g_ws = nullptr;
+size_t g_ws_size = 0;
+
+class Arena {
+public:
+    Arena() : lock_(g_ws_mutex) {}
+    ~Arena()
+    {
+        for (void *p : extras_)
+            hipFree(p);
+        if (need_ > g_ws_size) { // grow for the next call
+            hipFree(g_ws);
+            g_ws = nullptr;
+            g_ws_size = 0;
+            const size_t want = need_ + need_ / 2;
+            if (hipMalloc(&g_ws, want) == hipSuccess)
+                g_ws_size = want;
+        }
+    }
+    void *alloc(size_t bytes)
+    {
+        bytes = (bytes + 255) / 256 * 256;
+        need_ += bytes;
+        if (off_ + bytes <= g_ws_size) {
+            void *p = static_cast<char *>(g_ws) + off_;
+            off_ += bytes;
+            return p;
+        }
+        void *p = nullptr;
+        if (hipMalloc(&p, bytes) != hipSuccess)
+            return nullptr;
+        extras_.push_back(p);
+        return p;
+    }
+    template <class T> T *alloc_n(size_t n) { return static_cast<T *>(alloc(sizeof(T) * std::max<size_t>(n, 1))); }
+
+private:
+    std::lock_guard<std::mutex> lock_;
+    size_t off_ = 0, need_ = 0;
+    std::vector<void *> extras_;
 };
 
 // The k-th (0-based) smallest of v[0..n) and its upper neighbour in sorted order.
-int order_statistics(const float *d_v, int64_t n, int64_t k, hipStream_t s, float *a, float *b)
-{
-    DevBuf scratch;
-    if (hipMalloc(&scratch.p, 256 * sizeof(unsigned long long) + 16) != hipSuccess)
-        return fail(TW_ERR_ALLOC, "hipMalloc of the selection scratch failed");
-    unsigned long long *d_hist = scratch.as<unsigned long long>();
-    const int grid = (int)std::min<int64_t>(1024, (n + 255) / 256);
-    uint32_t mask = 0, prefix = 0;
-    int64_t rank = k;
-    unsigned long long hist[256];
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        TW_HIP(hipMemsetAsync(d_hist, 0, 256 * sizeof(unsigned long long), s));
-        hipLaunchKernelGGL(select_hist_kernel, dim3(grid), dim3(256), 0, s, d_v, n, mask, prefix,
-                           shift, d_hist);
-        TW_HIP(hipGetLastError());
-        TW_HIP(hipMemcpyAsync(hist, d_hist, sizeof(hist), hipMemcpyDeviceToHost, s));
-        TW_HIP(hipStreamSynchronize(s));
-        int d = 0;
-        for (; d < 256; ++d) {
-            if (rank < (int64_t)hist[d])
-                break;
-            rank -= (int64_t)hist[d];
-        }
-        if (d == 256)
-            return fail(TW_ERR_DEVICE, "radix select lost rank %lld", (long long)k);
-        prefix |= (uint32_t)d << shift;
-        mask |= 255u << shift;
-    }
-    *a = key_value(prefix);
-    // upper neighbour: a again if more than k+1 values are <= a, else the smallest value above
-    unsigned long long *d_cnt = d_hist;
-    unsigned int *d_min = reinterpret_cast<unsigned int *>(d_hist + 1);
-    unsigned long long cnt = 0;
-    unsigned int mn = 0xFFFFFFFFu;
-    TW_HIP(hipMemsetAsync(d_cnt, 0, sizeof(unsigned long long), s));
-    TW_HIP(hipMemcpyAsync(d_min, &mn, sizeof(mn), hipMemcpyHostToDevice, s));
-    hipLaunchKernelGGL(rank_stats_kernel, dim3(grid), dim3(256), 0, s, d_v, n, prefix, d_cnt, d_min);
-    TW_HIP(hipGetLastError());
-    TW_HIP(hipMemcpyAsync(&cnt, d_cnt, sizeof(cnt), hipMemcpyDeviceToHost, s));
-    TW_HIP(hipMemcpyAsync(&mn, d_min, sizeof(mn), hipMemcpyDeviceToHost, s));
-    TW_HIP(hipStreamSynchronize(s));
-    *b = ((int64_t)cnt > k + 1 || mn == 0xFFFFFFFFu) ? *a : key_value(mn);
-    return TW_OK;
-}
-
 struct Threshold {
-    float f32;
-    double f64;
+    SelectState *state; // device; thr32 / thr64 are valid once the stream has run
     int is_f64;
 };
 
-// np.percentile(v, q) with linear interpolation for a float32 vector on the device.  With
-// q_is_f64 == 0 (q was a Python number) the quantile q/100, the virtual index (n-1)*quantile
-// and the interpolation are float32; with 1 (q was a NumPy float64) they are float64, only
-// the difference of the two neighbours stays float32.
-int percentile_linear(const float *d_v, int64_t n, double q, int q_is_f64, hipStream_t s,
+// np.percentile(v, q) with linear interpolation for a float32 vector on the device, queued on the
+// stream: four histogram passes of a radix select for the k-th smallest value, its upper
+// neighbour, then the interpolation.  With q_is_f64 == 0 (q was a Python number) the quantile
+// q/100, the virtual index (n-1)*quantile and the interpolation are float32; with 1 (q was a
+// NumPy float64) they are float64, only the difference of the two neighbours stays float32.
+int percentile_linear(Arena &ar, const float *d_v, int64_t n, double q, int q_is_f64, hipStream_t s,
                       Threshold *out)
 {
     if (n <= 0)
@@ -337,32 +483,34 @@ int percentile_linear(const float *d_v, int64_t n, double q, int q_is_f64, hipSt
         lo = top ? n - 1 : (int64_t)std::floor(virt);
         gamma32 = virt - std::floor(virt);
     }
-    float a, b;
-    int st = order_statistics(d_v, n, std::min(lo, n - 1), s, &a, &b);
-    if (st)
-        return st;
-    if (top)
-        b = a;
-    const float diff = b - a;
-    out->is_f64 = q_is_f64;
-    if (q_is_f64) {
-        const double r = gamma64 >= 0.5 ? (double)b - (double)diff * (1.0 - gamma64)
-                                        : (double)a + (double)diff * gamma64;
-        out->f64 = r;
-        out->f32 = (float)r;
-    } else {
-        volatile float prod; // keep the product a rounded float32 (no fma on the host either)
-        float r;
-        if (gamma32 >= 0.5f) {
-            prod = diff * (1.0f - gamma32);
-            r = b - prod;
-        } else {
-            prod = diff * gamma32;
-            r = a + prod;
-        }
-        out->f32 = r;
-        out->f64 = (double)r;
+    const unsigned long long k = (unsigned long long)std::min(lo, n - 1);
+    SelectState *st = ar.alloc_n<SelectState>(1);
+    if (!st)
+        return fail(TW_ERR_ALLOC, "hipMalloc of the selection state failed");
+    const int grid = (int)std::min<int64_t>(1024, (n + 255) / 256);
+    hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(256), 0, s, st, k);
+    for (int shift = 24; shift >= 0; shift -= 8) {
+        hipLaunchKernelGGL(select_hist_kernel, dim3(grid), dim3(256), 0, s, d_v, n, shift, st);
+        hipLaunchKernelGGL(select_digit_kernel, dim3(1), dim3(256), 0, s, shift, st);
     }
+    hipLaunchKernelGGL(rank_stats_kernel, dim3(grid), dim3(256), 0, s, d_v, n, st);
+    hipLaunchKernelGGL(select_lerp_kernel, dim3(1), dim3(1), 0, s, st, k, top ? 1 : 0, q_is_f64,
+                       gamma32, gamma64);
+    TW_HIP(hipGetLastError());
+    out->state = st;
+    out->is_f64 = q_is_f64;
+    return TW_OK;
+}
+
+// waits for the stream and returns the threshold as a double
+int read_threshold(const Threshold &t, hipStream_t s, double *value)
+{
+    SelectState h;
+    TW_HIP(hipMemcpyAsync(&h, t.state, sizeof(h), hipMemcpyDeviceToHost, s));
+    TW_HIP(hipStreamSynchronize(s));
+    if (h.lost)
+        return fail(TW_ERR_DEVICE, "radix select lost its rank");
+    *value = h.thr64;
     return TW_OK;
 }
 
@@ -390,9 +538,10 @@ struct LayerTiles {
 };
 
 // norms of all layers into one pooled vector, one threshold, masks
-int rows_stage(int n_layers, const int32_t *K, const int32_t *N, const float *const *scores,
-               std::vector<LayerTiles> &lt, const std::vector<uint8_t *> &d_colkeep, double q,
-               int q_is_f64, uint8_t *const *masks, Threshold *thr, hipStream_t s)
+int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
+               const float *const *scores, std::vector<LayerTiles> &lt,
+               const std::vector<uint8_t *> &d_colkeep, double q, int q_is_f64,
+               uint8_t *const *masks, Threshold *thr, hipStream_t s)
 {
     int64_t total = 0, tab = 0;
     for (int l = 0; l < n_layers; ++l) {
@@ -400,43 +549,45 @@ int rows_stage(int n_layers, const int32_t *K, const int32_t *N, const float *co
         total += (int64_t)K[l] * ((int64_t)lt[l].tcol0.size() - 1);
         tab += (int64_t)lt[l].tcol0.size();
     }
-    DevBuf norms, tables;
-    if (hipMalloc(&norms.p, sizeof(float) * total) != hipSuccess ||
-        hipMalloc(&tables.p, sizeof(int32_t) * tab) != hipSuccess)
+    float *d_norms = ar.alloc_n<float>(total);
+    int32_t *d_tables = ar.alloc_n<int32_t>(tab);
+    PruneLayer *d_table = ar.alloc_n<PruneLayer>(n_layers);
+    if (!d_norms || !d_tables || !d_table)
         return fail(TW_ERR_ALLOC, "hipMalloc of %lld norms failed", (long long)total);
     std::vector<int32_t> flat;
-    std::vector<int64_t> tab_off(n_layers);
+    std::vector<PruneLayer> pl(n_layers);
+    int64_t n_pairs = 0, n_elems = 0;
     for (int l = 0; l < n_layers; ++l) {
-        tab_off[l] = (int64_t)flat.size();
+        PruneLayer &e = pl[l];
+        e.score = scores[l];
+        e.mask = masks ? masks[l] : nullptr;
+        e.colkeep = d_colkeep.empty() ? nullptr : d_colkeep[l];
+        e.tcol0 = d_tables + flat.size();
+        e.norms = d_norms + lt[l].norm_off;
+        e.K = K[l];
+        e.N = N[l];
+        e.n_tiles = (int32_t)lt[l].tcol0.size() - 1;
+        e.pad_ = 0;
+        e.rt_begin = n_pairs;
+        e.el_begin = n_elems;
+        n_pairs += (int64_t)e.K * e.n_tiles;
+        n_elems += (int64_t)e.K * ((e.N + 15) / 16);
         flat.insert(flat.end(), lt[l].tcol0.begin(), lt[l].tcol0.end());
     }
-    TW_HIP(hipMemcpyAsync(tables.p, flat.data(), sizeof(int32_t) * flat.size(),
+    TW_HIP(hipMemcpyAsync(d_tables, flat.data(), sizeof(int32_t) * flat.size(),
                           hipMemcpyHostToDevice, s));
-    TW_HIP(hipStreamSynchronize(s)); // `flat` is pageable host memory
-    for (int l = 0; l < n_layers; ++l) {
-        const int nt = (int)lt[l].tcol0.size() - 1;
-        const int64_t n_rt = (int64_t)K[l] * nt;
-        hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_rt + 255) / 256)), dim3(256),
-                           0, s, scores[l], K[l], N[l], tables.as<int32_t>() + tab_off[l], nt,
-                           d_colkeep.empty() ? nullptr : d_colkeep[l],
-                           norms.as<float>() + lt[l].norm_off);
-    }
+    TW_HIP(hipMemcpyAsync(d_table, pl.data(), sizeof(PruneLayer) * n_layers, hipMemcpyHostToDevice, s));
+    TW_HIP(hipStreamSynchronize(s)); // `flat` and `pl` are pageable host memory
+    hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_pairs * 8 + 255) / 256)), dim3(256),
+                       0, s, d_table, n_layers, n_pairs);
     TW_HIP(hipGetLastError());
-    int st = percentile_linear(norms.as<float>(), total, q, q_is_f64, s, thr);
+    int st = percentile_linear(ar, d_norms, total, q, q_is_f64, s, thr);
     if (st)
         return st;
-    for (int l = 0; l < n_layers; ++l) {
-        const int nt = (int)lt[l].tcol0.size() - 1;
-        const int64_t n_el = (int64_t)K[l] * N[l];
-        hipLaunchKernelGGL(fill_mask_kernel, dim3((unsigned)((n_el + 255) / 256)), dim3(256), 0, s,
-                           norms.as<float>() + lt[l].norm_off, K[l], N[l],
-                           tables.as<int32_t>() + tab_off[l], nt,
-                           d_colkeep.empty() ? nullptr : d_colkeep[l], thr->f32, thr->f64,
-                           thr->is_f64, masks[l]);
-    }
+    hipLaunchKernelGGL(fill_mask_kernel, dim3((unsigned)((n_elems + 255) / 256)), dim3(256), 0, s,
+                       d_table, n_layers, n_elems, thr->state, thr->is_f64);
     TW_HIP(hipGetLastError());
-    TW_HIP(hipStreamSynchronize(s)); // the temporaries are freed on return
-    return TW_OK;
+    return TW_OK; // the caller reads the threshold back, which waits for the stream
 }
 
 } // namespace
@@ -505,14 +656,29 @@ int tw_prune_tile_row_norms(int K, int N, const float *scores, int n_tiles,
         return fail(TW_ERR_TILE_TABLE, "tiles cover %d columns, N=%d", c, N);
     tcol0[n_tiles] = N;
     hipStream_t s = (hipStream_t)stream;
-    DevBuf tab;
-    if (hipMalloc(&tab.p, sizeof(int32_t) * (n_tiles + 1)) != hipSuccess)
+    Arena ar;
+    int32_t *d_tab = ar.alloc_n<int32_t>(n_tiles + 1);
+    PruneLayer *d_table = ar.alloc_n<PruneLayer>(1);
+    if (!d_tab || !d_table)
         return fail(TW_ERR_ALLOC, "hipMalloc of the tile table failed");
-    TW_HIP(hipMemcpyAsync(tab.p, tcol0.data(), sizeof(int32_t) * (n_tiles + 1), hipMemcpyHostToDevice, s));
+    PruneLayer e;
+    e.score = scores;
+    e.mask = nullptr;
+    e.colkeep = col_keep;
+    e.tcol0 = d_tab;
+    e.norms = norms;
+    e.K = K;
+    e.N = N;
+    e.n_tiles = n_tiles;
+    e.pad_ = 0;
+    e.rt_begin = 0;
+    e.el_begin = 0;
+    TW_HIP(hipMemcpyAsync(d_tab, tcol0.data(), sizeof(int32_t) * (n_tiles + 1), hipMemcpyHostToDevice, s));
+    TW_HIP(hipMemcpyAsync(d_table, &e, sizeof(e), hipMemcpyHostToDevice, s));
     TW_HIP(hipStreamSynchronize(s));
-    const int64_t n_rt = (int64_t)K * n_tiles;
-    hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_rt + 255) / 256)), dim3(256), 0, s,
-                       scores, K, N, tab.as<int32_t>(), n_tiles, col_keep, norms);
+    const int64_t n_pairs = (int64_t)K * n_tiles;
+    hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_pairs * 8 + 255) / 256)), dim3(256), 0, s,
+                       d_table, 1, n_pairs);
     TW_HIP(hipGetLastError());
     TW_HIP(hipStreamSynchronize(s));
     return TW_OK;
@@ -524,9 +690,17 @@ int tw_prune_col_norms(int K, int N, const float *scores, float *norms, void *st
         return fail(TW_ERR_SHAPE, "K=%d N=%d must be positive", K, N);
     if (!scores || !norms)
         return fail(TW_ERR_NULL, "a pointer is NULL");
-    hipLaunchKernelGGL(col_norms_kernel, dim3((N + 63) / 64), dim3(64), 0, (hipStream_t)stream, scores,
-                       K, N, norms);
+    hipStream_t s = (hipStream_t)stream;
+    Arena ar;
+    ColLayer *d_cl = ar.alloc_n<ColLayer>(1);
+    if (!d_cl)
+        return fail(TW_ERR_ALLOC, "hipMalloc of the layer table failed");
+    const ColLayer cl{scores, K, N, 0};
+    TW_HIP(hipMemcpyAsync(d_cl, &cl, sizeof(cl), hipMemcpyHostToDevice, s));
+    TW_HIP(hipStreamSynchronize(s));
+    hipLaunchKernelGGL(col_norms_kernel, dim3((N + 63) / 64), dim3(64), 0, s, d_cl, 1, (int64_t)N, norms);
     TW_HIP(hipGetLastError());
+    TW_HIP(hipStreamSynchronize(s));
     return TW_OK;
 }
 
@@ -538,9 +712,10 @@ int tw_percentile_linear(const float *values, int64_t n, double q, int q_type, d
     if (q_type != TW_Q_F32 && q_type != TW_Q_F64)
         return fail(TW_ERR_LAYOUT, "q_type=%d: unknown", q_type);
     Threshold t;
-    int st = percentile_linear(values, n, q, q_type, (hipStream_t)stream, &t);
+    Arena ar;
+    int st = percentile_linear(ar, values, n, q, q_type, (hipStream_t)stream, &t);
     if (!st)
-        *result = t.f64;
+        st = read_threshold(t, (hipStream_t)stream, result);
     return st;
 }
 
@@ -560,10 +735,14 @@ int tw_prune_tiled_wise_1d(int n_layers, const int32_t *K, const int32_t *N,
         lt[l].tcol0.push_back(N[l]);
     }
     Threshold thr;
-    st = rows_stage(n_layers, K, N, scores, lt, {}, sparsity, q_type, masks, &thr,
+    Arena ar;
+    st = rows_stage(ar, n_layers, K, N, scores, lt, {}, sparsity, q_type, masks, &thr,
                     (hipStream_t)stream);
+    double value = 0.0;
+    if (!st)
+        st = read_threshold(thr, (hipStream_t)stream, &value); // also: the masks are complete
     if (!st && threshold)
-        *threshold = thr.f64;
+        *threshold = value;
     return st;
 }
 
@@ -593,24 +772,29 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
         coff[l] = total_n;
         total_n += N[l];
     }
-    DevBuf cnorm, ckeep;
-    if (hipMalloc(&cnorm.p, sizeof(float) * total_n) != hipSuccess ||
-        hipMalloc(&ckeep.p, (size_t)total_n) != hipSuccess)
+    Arena ar;
+    float *d_cnorm = ar.alloc_n<float>(total_n);
+    uint8_t *d_ckeep = ar.alloc_n<uint8_t>(total_n);
+    ColLayer *d_cl = ar.alloc_n<ColLayer>(n_layers);
+    if (!d_cnorm || !d_ckeep || !d_cl)
         return fail(TW_ERR_ALLOC, "hipMalloc of %lld column norms failed", (long long)total_n);
+    std::vector<ColLayer> cl(n_layers);
     for (int l = 0; l < n_layers; ++l)
-        hipLaunchKernelGGL(col_norms_kernel, dim3((N[l] + 63) / 64), dim3(64), 0, s, scores[l], K[l],
-                           N[l], cnorm.as<float>() + coff[l]);
+        cl[l] = ColLayer{scores[l], K[l], N[l], coff[l]};
+    TW_HIP(hipMemcpyAsync(d_cl, cl.data(), sizeof(ColLayer) * n_layers, hipMemcpyHostToDevice, s));
+    TW_HIP(hipStreamSynchronize(s)); // `cl` is pageable host memory
+    hipLaunchKernelGGL(col_norms_kernel, dim3((unsigned)((total_n + 63) / 64)), dim3(64), 0, s, d_cl,
+                       n_layers, total_n, d_cnorm);
     TW_HIP(hipGetLastError());
     Threshold thr_c;
-    st = percentile_linear(cnorm.as<float>(), total_n, q, q_type, s, &thr_c);
+    st = percentile_linear(ar, d_cnorm, total_n, q, q_type, s, &thr_c);
     if (st)
         return st;
     hipLaunchKernelGGL(col_keep_kernel, dim3((unsigned)((total_n + 255) / 256)), dim3(256), 0, s,
-                       cnorm.as<float>(), (int)total_n, thr_c.f32, thr_c.f64, thr_c.is_f64,
-                       ckeep.as<uint8_t>());
+                       d_cnorm, (int)total_n, thr_c.state, thr_c.is_f64, d_ckeep);
     TW_HIP(hipGetLastError());
     std::vector<uint8_t> h_keep(total_n);
-    TW_HIP(hipMemcpyAsync(h_keep.data(), ckeep.p, (size_t)total_n, hipMemcpyDeviceToHost, s));
+    TW_HIP(hipMemcpyAsync(h_keep.data(), d_ckeep, (size_t)total_n, hipMemcpyDeviceToHost, s));
     TW_HIP(hipStreamSynchronize(s));
     // tiles end after every `granularity` kept columns
     std::vector<LayerTiles> lt(n_layers);
@@ -626,15 +810,20 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
             return st;
         lt[l].tcol0.assign(col0.begin(), col0.begin() + nt);
         lt[l].tcol0.push_back(N[l]);
-        d_colkeep[l] = ckeep.as<uint8_t>() + coff[l];
+        d_colkeep[l] = d_ckeep + coff[l];
         if (col_masks && col_masks[l])
             TW_HIP(hipMemcpyAsync(col_masks[l], d_colkeep[l], (size_t)N[l], hipMemcpyDeviceToDevice, s));
     }
     Threshold thr_r;
-    st = rows_stage(n_layers, K, N, scores, lt, d_colkeep, q, q_type, masks, &thr_r, s);
+    st = rows_stage(ar, n_layers, K, N, scores, lt, d_colkeep, q, q_type, masks, &thr_r, s);
+    double vc = 0.0, vr = 0.0;
+    if (!st)
+        st = read_threshold(thr_c, s, &vc);
+    if (!st)
+        st = read_threshold(thr_r, s, &vr);
     if (!st && thresholds) {
-        thresholds[0] = thr_c.f64;
-        thresholds[1] = thr_r.f64;
+        thresholds[0] = vc;
+        thresholds[1] = vr;
     }
     return st;
 }

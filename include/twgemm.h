@@ -193,6 +193,25 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda,
             void *C, int c_layout, int64_t ldc, int M, float alpha, float beta,
             int pruned_cols, void *stream);
 
+/* The same with a fused epilogue: C = act(alpha * A (B (.) mask) + beta * C + bias) on the written
+ * columns, i.e. the reference's masked dense layer in one pass (mask_dense,
+ * Pruning/BERT/utils/modeling.py:992-1007: matmul(input, kernel * mask) + bias, then the
+ * activation).  bias is a device fp32 vector of N entries indexed by the original column (or
+ * NULL); the arithmetic is fp32 with one rounding to the 16-bit output.  With TW_PRUNED_ZERO a
+ * pruned column receives act(beta * C + bias), as it does in the reference, where a fully masked
+ * column still gets its bias.  ep == NULL is tw_gemm. */
+#define TW_ACT_NONE 0
+#define TW_ACT_RELU 1
+#define TW_ACT_GELU 2 /* 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))), modeling.py:264-277 */
+#define TW_ACT_TANH 3
+typedef struct tw_epilogue {
+    const float *bias;
+    int activation;
+} tw_epilogue;
+int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
+               int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
+               const tw_epilogue *ep, void *stream);
+
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument
  * meaning: A column-major M x K (lda = M), B the compacted stream weight, C
  * column-major M x N (ldc = M), all DEVICE memory of `dtype`; mask_n/mask_k host

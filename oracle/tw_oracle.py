@@ -225,13 +225,27 @@ def quantize(x, dtype):
 
 
 # --------------------------------------------------------------------------- GEMM
-def mask_dense(x, kernel, mask, bias=None):
-    """Pruning/BERT/utils/modeling.py:992-1007: x @ (kernel * mask) + bias in fp32.
-    This is the reference's CPU/TF operator (BLAS-backed here, as TF's matmul is)."""
+def gelu(x):
+    """Pruning/BERT/utils/modeling.py:264-277: the tanh form of GELU."""
+    x = np.asarray(x)
+    cdf = 0.5 * (1.0 + np.tanh(np.sqrt(2 / np.pi) * (x + 0.044715 * np.power(x, 3))))
+    return x * cdf
+
+
+ACTIVATIONS = {
+    None: lambda v: v, "linear": lambda v: v, "none": lambda v: v,
+    "relu": lambda v: np.maximum(v, 0), "gelu": gelu, "tanh": np.tanh,
+}
+
+
+def mask_dense(x, kernel, mask, bias=None, activation=None):
+    """Pruning/BERT/utils/modeling.py:992-1007: activation(x @ (kernel * mask) + bias) in
+    fp32; activation by name as in get_activation (modeling.py:280-305).  This is the
+    reference's CPU/TF operator (BLAS-backed here, as TF's matmul is)."""
     y = np.asarray(x, dtype=np.float32) @ (np.asarray(kernel, dtype=np.float32) * mask)
     if bias is not None:
         y = y + bias
-    return y
+    return ACTIVATIONS[activation](y)
 
 
 def tw_gemm_reference(A, B, tiles, alpha=1.0, beta=0.0, C=None, acc=np.float64):

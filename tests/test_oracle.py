@@ -342,3 +342,29 @@ def test_ref_compat_problem(oracle):
     A2, B2, tiles2, _ = oracle.ref_compat_problem(16, 768, 64, 384, 32)
     assert np.array_equal(A, A2) and np.array_equal(B, B2)
     assert all(np.array_equal(a["kept_k"], b["kept_k"]) for a, b in zip(tiles, tiles2))
+
+
+def test_gelu_and_mask_dense_epilogue():
+    """gelu: known values of the tanh form (0 -> 0, large x -> x, large -x -> 0, odd part x/2);
+    mask_dense with bias and activation against a loop."""
+    from oracle import tw_oracle as o
+    import math
+    assert o.gelu(0.0) == 0.0
+    assert abs(o.gelu(10.0) - 10.0) < 1e-6 and abs(o.gelu(-10.0)) < 1e-6
+    for x in (0.3, 1.0, 2.5):
+        assert abs((o.gelu(x) - o.gelu(-x)) - x) < 1e-12        # gelu(x) - gelu(-x) = x
+        want = 0.5 * x * (1 + math.tanh(math.sqrt(2 / math.pi) * (x + 0.044715 * x ** 3)))
+        assert abs(o.gelu(x) - want) < 1e-12
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((5, 7)).astype(np.float32)
+    w = rng.standard_normal((7, 6)).astype(np.float32)
+    m = (rng.random((7, 6)) < 0.5).astype(np.float32)
+    b = rng.standard_normal(6).astype(np.float32)
+    y = o.mask_dense(x, w, m, b, "relu")
+    for i in range(5):
+        for j in range(6):
+            v = sum(float(x[i, k]) * float(w[k, j]) * float(m[k, j]) for k in range(7)) + float(b[j])
+            assert abs(y[i, j] - max(v, 0.0)) < 1e-4
+    # a fully pruned column still gets its bias
+    m[:, 2] = 0
+    assert np.allclose(o.mask_dense(x, w, m, b)[:, 2], b[2])

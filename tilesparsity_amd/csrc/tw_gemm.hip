@@ -27,6 +27,7 @@
 #include "tw_internal.h"
 
 #include <atomic>
+#include <type_traits>
 #include <cstddef>
 #include <cstdlib>
 
@@ -88,6 +89,31 @@ __device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M
         for (int e = 0; e < M - m; ++e)
             dst[e] = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
     }
+}
+
+// Activation of the fused epilogue (tw_gemm_ex): the activations the reference's dense layers
+// can be given (get_activation, Pruning/BERT/utils/modeling.py:280-305); GELU in its tanh form
+// (modeling.py:264-277).
+__device__ __forceinline__ float tw_activate(float v, int act)
+{
+    if (act == TW_ACT_RELU)
+        return v > 0.0f ? v : 0.0f;
+    // tanh(u) = 1 - 2 / (exp(2u) + 1) with the hardware exponential and reciprocal (1 ulp each):
+    // exact limits at +-inf, ~1e-6 relative error in between, far below the 16-bit rounding
+    if (act == TW_ACT_GELU) {
+        const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
+        return v - v * __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f); // 0.5 v (1 + tanh u)
+    }
+    if (act == TW_ACT_TANH)
+        return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * v) + 1.0f);
+    return v;
+}
+// alpha*acc + beta*C is already in `v`: adds the bias of column c and applies the activation
+__device__ __forceinline__ float tw_finish(float v, const float *bias, int c, int act)
+{
+    if (bias)
+        v += bias[c];
+    return tw_activate(v, act);
 }
 
 // WM x WN waves of 64 x 64 outputs each: workgroup tile BM = 64*WM rows by BN = 64*WN
@@ -279,10 +305,12 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 const int c = t.col0 + p.pruned_n[t.pn_off + j];
                 uint16_t *dst = C + (int64_t)c * p.ldc + m;
                 u32x4 v = {0u, 0u, 0u, 0u};
-                if (p.beta != 0.0f && m < p.M) {
+                if ((p.beta != 0.0f || p.bias || p.act) && m < p.M) {
                     uint32_t w[4] = {0u, 0u, 0u, 0u};
-                    for (int e = 0; e < 8 && m + e < p.M; ++e)
-                        w[e >> 1] |= E::to_bits(p.beta * E::from_bits(dst[e])) << ((e & 1) * 16);
+                    for (int e = 0; e < 8 && m + e < p.M; ++e) {
+                        const float old = p.beta != 0.0f ? p.beta * E::from_bits(dst[e]) : 0.0f;
+                        w[e >> 1] |= E::to_bits(tw_finish(old, p.bias, c, p.act)) << ((e & 1) * 16);
+                    }
                     v.x = w[0];
                     v.y = w[1];
                     v.z = w[2];
@@ -453,23 +481,25 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
             // ---- epilogue --------------------------------------------------------
             const int32_t *const nlist = p.kept_n + u.kn_off;
             float scale = p.alpha;
-            if (p.beta != 0.0f) {
-                // rare path, kept out of the way of the common one: fold alpha and beta*C into
-                // the accumulators first (C is read on kept columns only)
+            if (p.beta != 0.0f || p.bias || p.act) {
+                // rare path, kept out of the way of the common one: fold alpha, beta*C, the bias
+                // and the activation into the accumulators first (C is read on kept columns only)
 #pragma unroll
                 for (int ni = 0; ni < 2; ++ni) {
                     const int j = wn * 64 + ni * 32 + (lane & 31);
-                    const int64_t coff =
-                        j < u.n_cnt ? (int64_t)(u.col0 + nlist[j]) * p.ldc : (int64_t)0;
+                    const int col = j < u.n_cnt ? u.col0 + nlist[j] : 0;
+                    const int64_t coff = (int64_t)col * p.ldc;
+                    const float bj = p.bias ? p.bias[col] : 0.0f;
 #pragma unroll
                     for (int mi = 0; mi < 2; ++mi)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) {
                             const int m = m0 + wm * 64 + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
                             float old = 0.0f;
-                            if (j < u.n_cnt && m < p.M)
+                            if (p.beta != 0.0f && j < u.n_cnt && m < p.M)
                                 old = E::from_bits(C[coff + m]);
-                            acc[mi][ni][r] = p.alpha * acc[mi][ni][r] + p.beta * old;
+                            acc[mi][ni][r] =
+                                tw_activate(p.alpha * acc[mi][ni][r] + p.beta * old + bj, p.act);
                         }
                 }
                 scale = 1.0f;
@@ -568,7 +598,8 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 
     __shared__ __align__(16) uint16_t smem[SMEM];
     __shared__ int s_tk[2];
-    __shared__ int s_cols[BN]; // output columns of the current item's unit
+    __shared__ int s_cols[BN];   // output columns of the current item's unit
+    __shared__ float s_bias[BN]; // ... and their bias values (fused epilogue)
 #ifdef TW_EXP_TIMING
     __shared__ unsigned long long s_ws[256];
 #ifndef TW_EXP_ITEM
@@ -688,10 +719,12 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             const int c = t.col0 + p.pruned_n[t.pn_off + j];
             uint16_t *dst = C + (int64_t)c * p.ldc + m;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if (p.beta != 0.0f && m < p.M) {
+            if ((p.beta != 0.0f || p.bias || p.act) && m < p.M) {
                 uint32_t w[4] = {0u, 0u, 0u, 0u};
-                for (int e = 0; e < 8 && m + e < p.M; ++e)
-                    w[e >> 1] |= E::to_bits(p.beta * E::from_bits(dst[e])) << ((e & 1) * 16);
+                for (int e = 0; e < 8 && m + e < p.M; ++e) {
+                    const float old = p.beta != 0.0f ? p.beta * E::from_bits(dst[e]) : 0.0f;
+                    w[e >> 1] |= E::to_bits(tw_finish(old, p.bias, c, p.act)) << ((e & 1) * 16);
+                }
                 v.x = w[0];
                 v.y = w[1];
                 v.z = w[2];
@@ -821,6 +854,12 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 const int m0 = cur.m0;
                 const int nsteps = u.k_pad / BK;
                 const Thr tc = setup(cur);
+                // output columns of the unit and their bias: fetched now, handed to the other waves
+                // through LDS with the last step
+                int out_col = 0;
+                float out_bias = 0.0f;
+                if (pt < BN)
+                    out_col = u.col0 + p.kept_n[u.kn_off + (pt < u.n_cnt ? pt : 0)];
                 if (!preloaded) {
                     Idx ix[R];
 #pragma unroll
@@ -882,6 +921,9 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     for (int r = 0; r < R; ++r)
                         slot(j0 + r, r, true);
                 }
+                // (the column numbers have arrived by now: the bias load flies over the last slots)
+                if (p.bias && pt < BN)
+                    out_bias = p.bias[out_col];
                 for (; j0 < nsteps; j0 += R) {
 #pragma unroll
                     for (int r = 0; r < R; ++r)
@@ -890,9 +932,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 }
                 // last time slot: the multiplying waves work on the last step; the first loads of
                 // the next item start now and fly over the epilogue
-                int out_col = 0;
-                if (pt < BN)
-                    out_col = u.col0 + p.kept_n[u.kn_off + (pt < u.n_cnt ? pt : 0)];
                 const bool chain = nxt.ticket < p.n_pipe_items;
                 if (chain) {
                     const Thr tn = setup(nxt);
@@ -908,8 +947,10 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                             issue(tn, j, ix[j], a_ring[j], b_ring[j]);
                 }
                 preloaded = chain;
-                if (pt < BN)
+                if (pt < BN) {
                     s_cols[pt] = out_col;
+                    s_bias[pt] = out_bias;
+                }
                 TW_WS_PHASE(2, 256)
                 TW_LDS_BARRIER(); // end of the last time slot
                 TW_WS_PHASE(3, 256)
@@ -1008,41 +1049,85 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 // epilogue: alpha/beta in fp32, round, hand the tile over through LDS
                 const int32_t *const nlist = p.kept_n + u.kn_off;
                 float scale = p.alpha;
+                const bool fused = (p.bias || p.act) && p.beta == 0.0f;
                 if (p.beta != 0.0f) {
-                    // rare path: fold alpha and beta*C into the accumulators first (C is read on
-                    // kept columns only)
+                    // rare path: fold alpha, beta*C, the bias and the activation into the
+                    // accumulators first (C is read on kept columns only)
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int j = ni * 32 + (lane & 31);
-                        const int64_t coff =
-                            j < u.n_cnt ? (int64_t)(u.col0 + nlist[j]) * p.ldc : (int64_t)0;
+                        const int col = j < u.n_cnt ? u.col0 + nlist[j] : 0;
+                        const int64_t coff = (int64_t)col * p.ldc;
 #pragma unroll
                         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
                                 const int m = m0 + wave * 64 + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
                                 float old = 0.0f;
-                                if (j < u.n_cnt && m < cur.m_end)
+                                if (p.beta != 0.0f && j < u.n_cnt && m < cur.m_end)
                                     old = E::from_bits(C[coff + m]);
-                                acc[mi][ni][r] = p.alpha * acc[mi][ni][r] + p.beta * old;
+                                acc[mi][ni][r] =
+                                    tw_finish(p.alpha * acc[mi][ni][r] + p.beta * old, p.bias, col, p.act);
                             }
                     }
                     scale = 1.0f;
                 }
+                if (fused) {
+                    // bias (handed over through LDS by the moving waves) and activation in fp32,
+                    // one rounding; the activation is a compile-time constant of each copy
+                    auto stage_fused = [&](auto act_tag) {
+                        constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-                for (int ni = 0; ni < NI; ++ni) {
-                    const int j = ni * 32 + (lane & 31); // compact column inside the unit
+                        for (int ni = 0; ni < NI; ++ni) {
+                            const int j = ni * 32 + (lane & 31);
+                            const float bj = p.bias ? s_bias[j] : 0.0f;
 #pragma unroll
-                    for (int mi = 0; mi < MI; ++mi) {
-                        const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
+                            for (int mi = 0; mi < MI; ++mi) {
+                                const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
 #pragma unroll
-                        for (int r4 = 0; r4 < 4; ++r4) {
-                            u32x2 pk;
-                            pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
-                                   (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
-                            pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
-                                   (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
-                            *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                                for (int r4 = 0; r4 < 4; ++r4) {
+                                    float v[4];
+#pragma unroll
+                                    for (int e = 0; e < 4; ++e)
+                                        v[e] = tw_activate(scale * acc[mi][ni][r4 * 4 + e] + bj, ACT);
+                                    u32x2 pk;
+                                    pk.x = E::to_bits(v[0]) | (E::to_bits(v[1]) << 16);
+                                    pk.y = E::to_bits(v[2]) | (E::to_bits(v[3]) << 16);
+                                    *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                                }
+                            }
+                        }
+                    };
+                    switch (p.act) {
+                    case TW_ACT_RELU:
+                        stage_fused(std::integral_constant<int, TW_ACT_RELU>());
+                        break;
+                    case TW_ACT_GELU:
+                        stage_fused(std::integral_constant<int, TW_ACT_GELU>());
+                        break;
+                    case TW_ACT_TANH:
+                        stage_fused(std::integral_constant<int, TW_ACT_TANH>());
+                        break;
+                    default:
+                        stage_fused(std::integral_constant<int, TW_ACT_NONE>());
+                        break;
+                    }
+                } else {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni) {
+                        const int j = ni * 32 + (lane & 31); // compact column inside the unit
+#pragma unroll
+                        for (int mi = 0; mi < MI; ++mi) {
+                            const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
+#pragma unroll
+                            for (int r4 = 0; r4 < 4; ++r4) {
+                                u32x2 pk;
+                                pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
+                                       (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
+                                pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
+                                       (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
+                                *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                            }
                         }
                     }
                 }
@@ -1116,8 +1201,10 @@ __global__ void __launch_bounds__(256, 2) tw_gemm_generic_kernel(const GemmArgs 
         for (int e = tid; e < t.n_pruned * BM; e += 256) {
             const int j = e % t.n_pruned, m = m0 + e / t.n_pruned;
             if (m < p.M) {
-                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)(t.col0 + p.pruned_n[t.pn_off + j]) * sc_n;
-                *dst = p.beta != 0.0f ? (uint16_t)E::to_bits(p.beta * E::from_bits(*dst)) : (uint16_t)0;
+                const int c = t.col0 + p.pruned_n[t.pn_off + j];
+                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)c * sc_n;
+                const float old = p.beta != 0.0f ? p.beta * E::from_bits(*dst) : 0.0f;
+                *dst = (uint16_t)E::to_bits(tw_finish(old, p.bias, c, p.act));
             }
         }
         return;
@@ -1194,11 +1281,12 @@ __global__ void __launch_bounds__(256, 2) tw_gemm_generic_kernel(const GemmArgs 
             const int jl = e & 63, ml = e >> 6;
             const int j = half * 64 + jl, m = m0 + ml;
             if (j < u.n_cnt && m < p.M) {
-                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)(u.col0 + nlist[j]) * sc_n;
+                const int c = u.col0 + nlist[j];
+                uint16_t *dst = C + (int64_t)m * sc_m + (int64_t)c * sc_n;
                 float v = p.alpha * sF[jl * (BM + 1) + ml];
                 if (p.beta != 0.0f)
                     v += p.beta * E::from_bits(*dst);
-                *dst = (uint16_t)E::to_bits(v);
+                *dst = (uint16_t)E::to_bits(tw_finish(v, p.bias, c, p.act));
             }
         }
         __syncthreads();
@@ -1280,8 +1368,18 @@ extern "C" {
 int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
             int64_t ldc, int M, float alpha, float beta, int pruned_cols, void *stream)
 {
+    return tw_gemm_ex(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, nullptr,
+                      stream);
+}
+
+int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
+               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
+               void *stream)
+{
     if (!plan)
         return fail(TW_ERR_NULL, "plan is NULL");
+    if (ep && (ep->activation < TW_ACT_NONE || ep->activation > TW_ACT_TANH))
+        return fail(TW_ERR_LAYOUT, "activation=%d: unknown", ep->activation);
     if (M < 0)
         return fail(TW_ERR_SHAPE, "M=%d is negative", M);
     if ((a_layout != TW_LAYOUT_KMAJOR && a_layout != TW_LAYOUT_ROWMAJOR) ||
@@ -1327,6 +1425,8 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
         a.ticket = nullptr;
         a.dbg = nullptr;
         a.n_arg_units = 0;
+        a.bias = ep ? ep->bias : nullptr;
+        a.act = ep ? ep->activation : TW_ACT_NONE;
         if (a.n_items == 0)
             return TW_OK;
         const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
@@ -1379,6 +1479,8 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
     a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
     a.alpha = alpha;
     a.beta = beta;
+    a.bias = ep ? ep->bias : nullptr;
+    a.act = ep ? ep->activation : TW_ACT_NONE;
     if (a.n_items == 0)
         return TW_OK;
     const unsigned slot =

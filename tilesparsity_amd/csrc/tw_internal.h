@@ -62,6 +62,8 @@ struct GemmArgs {
     int32_t n_items;      // + n_zero_tiles * n_mblk when zero-filling
     int32_t n_zero_tiles; // tiles with pruned columns (first entries of `tiles`)
     float alpha, beta;
+    const float *bias;    // fp32 [N] added to every written column before the activation, or null
+    int32_t act;          // TW_ACT_*
     int32_t *ticket;      // [0] next item, [1] finished workgroups
     void *dbg;            // 2 KiB scratch after the ticket slots (instrumented builds only)
     // Copy of `units` inside the kernel arguments for plans of at most kMaxArgUnits units

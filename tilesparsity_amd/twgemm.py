@@ -23,6 +23,12 @@ LIB_PATH = os.environ.get("TWGEMM_LIB") or os.path.join(_PKG, "libtwgemm.so")
 F16, BF16 = 0, 1
 KMAJOR, ROWMAJOR = 0, 1
 PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
+ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
+
+
+class Epilogue(ctypes.Structure):
+    """tw_epilogue of include/twgemm.h."""
+    _fields_ = [("bias", ctypes.c_void_p), ("activation", ctypes.c_int)]
 
 OK = 0
 ERR_NULL, ERR_SHAPE, ERR_TILE_TABLE, ERR_INDEX_LIST, ERR_DTYPE = -1, -2, -3, -4, -5
@@ -39,7 +45,7 @@ EXPORTED_SYMBOLS = (
     "tw_gemm", "tw_stream_gemm_nn", "tw_cast_f32", "tw_delete_row", "tw_insert_row",
     "tw_plan_from_mask_tiles", "tw_prune_tiled_wise_1d", "tw_prune_tiled_wise_2d",
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
-    "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear",
+    "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
 )
 
 
@@ -110,6 +116,8 @@ def lib():
         "tw_plan_export": (c_int, [vp, i32p, i32p, i32p, i32p, i32p, i32p, i32p, i32p, u16p]),
         "tw_plan_destroy": (c_int, [vp]),
         "tw_gemm": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int, vp]),
+        "tw_gemm_ex": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int,
+                               ctypes.POINTER(Epilogue), vp]),
         "tw_stream_gemm_nn": (c_int, [c_int, c_int, c_int, c_int, c_f, vp, vp, c_f, vp, c_int,
                                       i32p, i32p, pp, pp, i64p, i64p, vp]),
         "tw_cast_f32": (c_int, [vp, vp, c_i64, c_int, vp]),
@@ -330,15 +338,23 @@ class Plan:
 
     # -- the GEMM
     def gemm(self, A_ptr, C_ptr, M, lda=None, ldc=None, alpha=1.0, beta=0.0,
-             a_layout=KMAJOR, c_layout=KMAJOR, pruned_cols=PRUNED_UNTOUCHED, stream=0):
-        """C = alpha * A (B (.) mask) + beta * C on device pointers; asynchronous."""
+             a_layout=KMAJOR, c_layout=KMAJOR, pruned_cols=PRUNED_UNTOUCHED, stream=0,
+             bias_ptr=None, activation=ACT_NONE):
+        """C = act(alpha * A (B (.) mask) + beta * C + bias) on device pointers; asynchronous.
+        bias_ptr: device fp32 [N] or None; activation: ACT_NONE / ACT_RELU / ACT_GELU / ACT_TANH."""
         if lda is None:
             lda = M if a_layout == KMAJOR else self.K
         if ldc is None:
             ldc = M if c_layout == KMAJOR else self.N
-        _check(lib().tw_gemm(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
-                             ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
-                             pruned_cols, ctypes.c_void_p(int(stream or 0))))
+        if bias_ptr is None and activation == ACT_NONE:
+            _check(lib().tw_gemm(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
+                                 ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
+                                 pruned_cols, ctypes.c_void_p(int(stream or 0))))
+            return
+        ep = Epilogue(ctypes.c_void_p(int(bias_ptr or 0)), int(activation))
+        _check(lib().tw_gemm_ex(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
+                                ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
+                                pruned_cols, ctypes.byref(ep), ctypes.c_void_p(int(stream or 0))))
 
     def destroy(self):
         if self._h is not None and self._h.value:

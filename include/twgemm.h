@@ -273,6 +273,13 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
                            int granularity, uint8_t *const *masks, uint8_t *const *col_masks,
                            double *thresholds, void *stream);
 
+/* granularity_pruning (Pruning/BERT/utils/MyHook.py:202-214): one layer, tiles of `granularity`
+ * columns (N must be a multiple), one threshold per tile: the `sparsity`-th percentile of that
+ * tile's K row norms (not divided by the width); a tile row is kept iff its norm is strictly
+ * above its tile's threshold. */
+int tw_prune_granularity(int K, int N, const float *scores, double sparsity, int q_type,
+                         int granularity, uint8_t *mask, void *stream);
+
 /* The building blocks of the two producers, on device buffers:
  *   tw_prune_tile_row_norms   norms[t*K + k] = ||scores[k][tile t]|| / width_t in NumPy's float32
  *                             summation order; col_keep (optional, N bytes) zeroes pruned

@@ -31,7 +31,8 @@ Parity with the reference's own files is pinned by tests/golden/prune_vectors.np
 by tests/golden/make_prune_vectors.py from Pruning/VGG/prune_algo.py under the NumPy of this
 image (2.2.6).  The reference's published environment used an older NumPy whose percentile
 interpolates in float64 for every input; the two can differ only when a norm ties with the
-threshold to the last bit.
+threshold to the last bit.  granularity_pruning has no vectors from the reference (MyHook.py
+imports TensorFlow, which this image lacks): parity unpinned beyond its property tests.
 """
 import numpy as np
 

@@ -168,10 +168,24 @@ def test_masks_feed_plans(tw, twprune, po, oracle):
         assert oracle.rel_error(C, ref) <= 1e-2
 
 
+def test_granularity_pruning_matches_oracle(twprune, po):
+    rng = np.random.default_rng(24)
+    for K, N, g in ((64, 128, 16), (768, 768, 64), (300, 512, 128), (5, 8, 2)):
+        s = np.abs(rng.standard_normal((K, N))).astype(np.float32)
+        for sp in (50, 75.0, 90, np.float64(33.3), 0, 100):
+            print("granularity", K, N, g, repr(sp), flush=True)
+            assert np.array_equal(twprune.granularity_pruning(s, sp, g), po.granularity_pruning(s, sp, g))
+    # ties inside a tile
+    s = (np.round(np.abs(rng.standard_normal((96, 64))) * 2) / 2).astype(np.float32)
+    assert np.array_equal(twprune.granularity_pruning(s, 60, 8), po.granularity_pruning(s, 60, 8))
+
+
 def test_error_paths(tw, twprune):
     with pytest.raises(tw.TwError):
         twprune.tiled_wise_1d([np.ones((4, 4), np.float32)], 150, 2)
     with pytest.raises(tw.TwError):
         twprune.tiled_wise_1d([np.ones((4, 4), np.float32)], 50, 0)
+    with pytest.raises(tw.TwError):
+        twprune.granularity_pruning(np.ones((4, 6), np.float32), 50, 4)
     with pytest.raises(tw.TwError):
         tw.Plan.from_mask_tiles(np.ones((4, 8), np.uint8), [(0, 4), (5, 3)], "f16", np.ones((4, 8), np.float32))

@@ -94,6 +94,9 @@ __device__ float pairwise_sq_sum(const float *x, const uint8_t *keep, int n, int
     return ret;
 }
 
+constexpr int kNormNotDivided = 1;   // norms are not divided by the tile width
+constexpr int kPerTileThreshold = 2; // tile t compares with selection state t, not with state 0
+
 // One entry per layer of a producer call; all layers run in one launch per stage.
 struct PruneLayer {
     const float *score;
@@ -101,7 +104,8 @@ struct PruneLayer {
     const uint8_t *colkeep; // nullptr: every column counts
     const int32_t *tcol0;   // n_tiles + 1 entries
     float *norms;           // [n_tiles][K]
-    int32_t K, N, n_tiles, pad_;
+    int32_t K, N, n_tiles;
+    int32_t flags;          // kNormNotDivided, kPerTileThreshold
     int64_t rt_begin;       // first (row, tile) pair of this layer in the launch-wide numbering
     int64_t el_begin;       // first 16-column chunk likewise (ceil(N/16) chunks per row)
 };
@@ -137,7 +141,8 @@ __global__ void __launch_bounds__(256)
     const float s = pairwise_sq_sum(L.score + (int64_t)k * L.N + c0,
                                     L.colkeep ? L.colkeep + c0 : nullptr, w, l8);
     if (l8 == 0)
-        L.norms[(int64_t)t * L.K + k] = sqrtf(s) / (float)w; // both correctly rounded
+        L.norms[(int64_t)t * L.K + k] =
+            (L.flags & kNormNotDivided) ? sqrtf(s) : sqrtf(s) / (float)w; // both correctly rounded
 }
 
 // One entry per layer for the column stage.
@@ -207,8 +212,12 @@ struct SelectState {
     double thr64;
 };
 
+// The selection kernels work on segments of equal length laid end to end (one segment for the
+// network-wide thresholds, one per tile for per-tile thresholds): segment g = blockIdx.y (or
+// blockIdx.x for the one-workgroup kernels) uses state st[g] and values v[g*n .. g*n+n).
 __global__ void select_init_kernel(SelectState *st, unsigned long long rank)
 {
+    st += blockIdx.x;
     st->hist[threadIdx.x] = 0;
     if (threadIdx.x == 0) {
         st->rank = rank;
@@ -225,6 +234,8 @@ __global__ void select_init_kernel(SelectState *st, unsigned long long rank)
 __global__ void __launch_bounds__(256)
     select_hist_kernel(const float *v, int64_t n, int shift, SelectState *st)
 {
+    st += blockIdx.y;
+    v += (int64_t)blockIdx.y * n;
     __shared__ unsigned int s_h[256];
     s_h[threadIdx.x] = 0;
     __syncthreads();
@@ -243,6 +254,7 @@ __global__ void __launch_bounds__(256)
 // one workgroup: picks the digit that holds the rank, fixes it in the prefix, clears the histogram
 __global__ void __launch_bounds__(256) select_digit_kernel(int shift, SelectState *st)
 {
+    st += blockIdx.x;
     __shared__ unsigned long long s_c[256];
     s_c[threadIdx.x] = st->hist[threadIdx.x];
     __syncthreads();
@@ -268,6 +280,8 @@ __global__ void __launch_bounds__(256) select_digit_kernel(int shift, SelectStat
 // count_le = number of values <= the selected one, min_gt = smallest key above it
 __global__ void __launch_bounds__(256) rank_stats_kernel(const float *v, int64_t n, SelectState *st)
 {
+    st += blockIdx.y;
+    v += (int64_t)blockIdx.y * n;
     const uint32_t key_a = st->prefix;
     unsigned long long cnt = 0;
     unsigned int mn = 0xFFFFFFFFu;
@@ -315,6 +329,7 @@ __device__ __forceinline__ float key_to_float(uint32_t key)
 __global__ void select_lerp_kernel(SelectState *st, unsigned long long k, int top, int f64,
                                    float gamma32, double gamma64)
 {
+    st += blockIdx.x;
     const float a = key_to_float(st->prefix);
     float b = a;
     if (!top && st->count_le <= k + 1 && st->min_gt != 0xFFFFFFFFu)
@@ -349,12 +364,13 @@ __global__ void col_keep_kernel(const float *cnorm, int N, const SelectState *st
 __global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t n_chunks,
                                  const SelectState *st, int f64)
 {
-    const float thr32 = st->thr32;
-    const double thr64 = st->thr64;
     const int64_t gidx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gidx >= n_chunks)
         return;
     const PruneLayer L = layers[find_layer(layers, n_layers, gidx, true)];
+    const bool per_tile = (L.flags & kPerTileThreshold) != 0;
+    float thr32 = st->thr32;
+    double thr64 = st->thr64;
     const int64_t idx = gidx - L.el_begin;
     const int cpr = (L.N + 15) >> 4; // chunks per row
     const int k = (int)(idx / cpr);
@@ -369,6 +385,10 @@ __global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t
     }
     int t_end = L.tcol0[t + 1];
     float nv = L.norms[(int64_t)t * L.K + k];
+    if (per_tile) {
+        thr32 = st[t].thr32;
+        thr64 = st[t].thr64;
+    }
     bool row_keep = f64 ? (double)nv > thr64 : nv > thr32;
     uint32_t w[4] = {0u, 0u, 0u, 0u};
     const int n = min(16, L.N - c0);
@@ -378,6 +398,10 @@ __global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t
             ++t;
             t_end = L.tcol0[t + 1];
             nv = L.norms[(int64_t)t * L.K + k];
+            if (per_tile) {
+                thr32 = st[t].thr32;
+                thr64 = st[t].thr64;
+            }
             row_keep = f64 ? (double)nv > thr64 : nv > thr32;
         }
         const bool keep = row_keep && (!L.colkeep || L.colkeep[c]);
@@ -408,15 +432,23 @@ namespace {
 std::mutex g_ws_mutex;
 void *g_ws = nullptr;
 size_t g_ws_size = 0;
+int g_ws_device = -1; // the device the buffer lives on; calls on another device do not use it
 
 class Arena {
 public:
-    Arena() : lock_(g_ws_mutex) {}
+    Arena() : lock_(g_ws_mutex)
+    {
+        if (hipGetDevice(&device_) != hipSuccess)
+            device_ = -2;
+        if (g_ws_device < 0)
+            g_ws_device = device_;
+        usable_ = device_ == g_ws_device;
+    }
     ~Arena()
     {
         for (void *p : extras_)
             hipFree(p);
-        if (need_ > g_ws_size) { // grow for the next call
+        if (usable_ && need_ > g_ws_size) { // grow for the next call
             hipFree(g_ws);
             g_ws = nullptr;
             g_ws_size = 0;
@@ -429,7 +461,7 @@ public:
     {
         bytes = (bytes + 255) / 256 * 256;
         need_ += bytes;
-        if (off_ + bytes <= g_ws_size) {
+        if (usable_ && off_ + bytes <= g_ws_size) {
             void *p = static_cast<char *>(g_ws) + off_;
             off_ += bytes;
             return p;
@@ -444,6 +476,8 @@ public:
 
 private:
     std::lock_guard<std::mutex> lock_;
+    int device_ = -1;
+    bool usable_ = false;
     size_t off_ = 0, need_ = 0;
     std::vector<void *> extras_;
 };
@@ -460,7 +494,7 @@ struct Threshold {
 // q/100, the virtual index (n-1)*quantile and the interpolation are float32; with 1 (q was a
 // NumPy float64) they are float64, only the difference of the two neighbours stays float32.
 int percentile_linear(Arena &ar, const float *d_v, int64_t n, double q, int q_is_f64, hipStream_t s,
-                      Threshold *out)
+                      Threshold *out, int n_segments = 1)
 {
     if (n <= 0)
         return fail(TW_ERR_SHAPE, "percentile of an empty set");
@@ -484,17 +518,18 @@ int percentile_linear(Arena &ar, const float *d_v, int64_t n, double q, int q_is
         gamma32 = virt - std::floor(virt);
     }
     const unsigned long long k = (unsigned long long)std::min(lo, n - 1);
-    SelectState *st = ar.alloc_n<SelectState>(1);
+    SelectState *st = ar.alloc_n<SelectState>(n_segments);
     if (!st)
         return fail(TW_ERR_ALLOC, "hipMalloc of the selection state failed");
-    const int grid = (int)std::min<int64_t>(1024, (n + 255) / 256);
-    hipLaunchKernelGGL(select_init_kernel, dim3(1), dim3(256), 0, s, st, k);
+    const int grid = (int)std::min<int64_t>(n_segments > 1 ? 64 : 1024, (n + 255) / 256);
+    const dim3 g2(grid, n_segments), g1(n_segments);
+    hipLaunchKernelGGL(select_init_kernel, g1, dim3(256), 0, s, st, k);
     for (int shift = 24; shift >= 0; shift -= 8) {
-        hipLaunchKernelGGL(select_hist_kernel, dim3(grid), dim3(256), 0, s, d_v, n, shift, st);
-        hipLaunchKernelGGL(select_digit_kernel, dim3(1), dim3(256), 0, s, shift, st);
+        hipLaunchKernelGGL(select_hist_kernel, g2, dim3(256), 0, s, d_v, n, shift, st);
+        hipLaunchKernelGGL(select_digit_kernel, g1, dim3(256), 0, s, shift, st);
     }
-    hipLaunchKernelGGL(rank_stats_kernel, dim3(grid), dim3(256), 0, s, d_v, n, st);
-    hipLaunchKernelGGL(select_lerp_kernel, dim3(1), dim3(1), 0, s, st, k, top ? 1 : 0, q_is_f64,
+    hipLaunchKernelGGL(rank_stats_kernel, g2, dim3(256), 0, s, d_v, n, st);
+    hipLaunchKernelGGL(select_lerp_kernel, g1, dim3(1), 0, s, st, k, top ? 1 : 0, q_is_f64,
                        gamma32, gamma64);
     TW_HIP(hipGetLastError());
     out->state = st;
@@ -541,7 +576,7 @@ struct LayerTiles {
 int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
                const float *const *scores, std::vector<LayerTiles> &lt,
                const std::vector<uint8_t *> &d_colkeep, double q, int q_is_f64,
-               uint8_t *const *masks, Threshold *thr, hipStream_t s)
+               uint8_t *const *masks, Threshold *thr, hipStream_t s, int flags = 0)
 {
     int64_t total = 0, tab = 0;
     for (int l = 0; l < n_layers; ++l) {
@@ -567,7 +602,7 @@ int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
         e.K = K[l];
         e.N = N[l];
         e.n_tiles = (int32_t)lt[l].tcol0.size() - 1;
-        e.pad_ = 0;
+        e.flags = flags;
         e.rt_begin = n_pairs;
         e.el_begin = n_elems;
         n_pairs += (int64_t)e.K * e.n_tiles;
@@ -581,7 +616,9 @@ int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
     hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_pairs * 8 + 255) / 256)), dim3(256),
                        0, s, d_table, n_layers, n_pairs);
     TW_HIP(hipGetLastError());
-    int st = percentile_linear(ar, d_norms, total, q, q_is_f64, s, thr);
+    // per-tile thresholds (one layer): every tile's K norms are one segment
+    const int n_seg = (flags & kPerTileThreshold) ? (int)lt[0].tcol0.size() - 1 : 1;
+    int st = percentile_linear(ar, d_norms, total / n_seg, q, q_is_f64, s, thr, n_seg);
     if (st)
         return st;
     hipLaunchKernelGGL(fill_mask_kernel, dim3((unsigned)((n_elems + 255) / 256)), dim3(256), 0, s,
@@ -670,7 +707,7 @@ int tw_prune_tile_row_norms(int K, int N, const float *scores, int n_tiles,
     e.K = K;
     e.N = N;
     e.n_tiles = n_tiles;
-    e.pad_ = 0;
+    e.flags = 0;
     e.rt_begin = 0;
     e.el_begin = 0;
     TW_HIP(hipMemcpyAsync(d_tab, tcol0.data(), sizeof(int32_t) * (n_tiles + 1), hipMemcpyHostToDevice, s));
@@ -743,6 +780,31 @@ int tw_prune_tiled_wise_1d(int n_layers, const int32_t *K, const int32_t *N,
         st = read_threshold(thr, (hipStream_t)stream, &value); // also: the masks are complete
     if (!st && threshold)
         *threshold = value;
+    return st;
+}
+
+int tw_prune_granularity(int K, int N, const float *scores, double sparsity, int q_type,
+                         int granularity, uint8_t *mask, void *stream)
+{
+    const float *const sc[1] = {scores};
+    uint8_t *const mk[1] = {mask};
+    int st = check_layers(1, &K, &N, sc, mk, granularity);
+    if (st)
+        return st;
+    if (q_type != TW_Q_F32 && q_type != TW_Q_F64)
+        return fail(TW_ERR_LAYOUT, "q_type=%d: unknown", q_type);
+    if (N % granularity != 0)
+        return fail(TW_ERR_SHAPE, "N=%d is not a multiple of the granularity %d", N, granularity);
+    std::vector<LayerTiles> lt(1);
+    for (int c = 0; c <= N; c += granularity)
+        lt[0].tcol0.push_back(c);
+    Threshold thr;
+    Arena ar;
+    st = rows_stage(ar, 1, &K, &N, sc, lt, {}, sparsity, q_type, mk, &thr, (hipStream_t)stream,
+                    kNormNotDivided | kPerTileThreshold);
+    double value = 0.0;
+    if (!st)
+        st = read_threshold(thr, (hipStream_t)stream, &value); // waits for the mask
     return st;
 }
 

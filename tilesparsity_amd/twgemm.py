@@ -46,6 +46,7 @@ EXPORTED_SYMBOLS = (
     "tw_plan_from_mask_tiles", "tw_prune_tiled_wise_1d", "tw_prune_tiled_wise_2d",
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
+    "tw_prune_granularity",
 )
 
 
@@ -131,6 +132,7 @@ def lib():
         "tw_tiles_every_g_columns": (c_int, [c_int, c_int, i32p, i32p, ctypes.POINTER(c_int)]),
         "tw_prune_tile_row_norms": (c_int, [c_int, c_int, vp, c_int, i32p, i32p, vp, vp, vp]),
         "tw_prune_col_norms": (c_int, [c_int, c_int, vp, vp, vp]),
+        "tw_prune_granularity": (c_int, [c_int, c_int, vp, ctypes.c_double, c_int, c_int, vp, vp]),
         "tw_percentile_linear": (c_int, [vp, c_i64, ctypes.c_double, c_int,
                                          ctypes.POINTER(ctypes.c_double), vp]),
         "tw_tiles_every_g_kept_columns": (c_int, [c_int, c_int, u8p, i32p, i32p,

@@ -102,6 +102,20 @@ def tiled_wise_2d(accumulated_scores, sparsity, granularity=128, transform=True,
     return masks, tables
 
 
+def granularity_pruning(score, sparsity, granularity):
+    """One threshold per tile (Pruning/BERT/utils/MyHook.py:202-214); `score` is one 2-D layer
+    whose width is a multiple of the granularity.  Returns a bool [K, N] mask."""
+    import torch
+    L = tw.lib()
+    t = torch.from_numpy(np.ascontiguousarray(score, dtype=np.float32)).cuda()
+    K, N = t.shape
+    m = torch.empty((K, N), dtype=torch.uint8, device="cuda")
+    tw._check(L.tw_prune_granularity(K, N, t.data_ptr(), float(sparsity), _q_type(sparsity),
+                                     int(granularity), m.data_ptr(),
+                                     torch.cuda.current_stream().cuda_stream))
+    return m.cpu().numpy().astype(bool)
+
+
 def tiles_every_g_columns(n_cols, granularity):
     L = tw.lib()
     col0 = np.zeros(n_cols, np.int32)

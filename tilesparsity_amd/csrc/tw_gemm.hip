@@ -691,7 +691,17 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             t_pending = atomicAdd(&p.ticket[0], 1);
         }
     };
-    auto claim = [&]() { // two barriers
+    // An item with at least one step learns its successor without barriers of its own: thread 0
+    // publishes the ticket before the item's first pipeline barrier, everybody reads it after.
+    auto publish = [&]() {
+        if (tid == 0) {
+            pick_up();
+            s_tk[0] = t_next;
+            t_next = -1;
+        }
+    };
+    auto published = [&]() { return make_item(__builtin_amdgcn_readfirstlane(s_tk[0])); };
+    auto claim = [&]() { // two barriers of its own: items without steps
         if (tid == 0) {
             pick_up();
             s_tk[0] = t_next;
@@ -747,9 +757,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             v.y = lo.y;
             v.z = hi.x;
             v.w = hi.y;
-#ifdef TW_EXP_NOSTORE
-            if (v.x == 0x12345678u)
-#endif
             store_chunk(C + (int64_t)c * p.ldc + m_st, v, m_st, m_end);
         }
     };
@@ -806,12 +813,8 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             return *reinterpret_cast<const u32x4 *>(t.a_base + ((upper ? o1 : o0) + t.v_chunk));
         };
         auto load_b = [&](const Thr &t, int s, int bp) {
-#ifdef TW_EXP_NOB
-            return u32x4{(unsigned)s, 0u, 0u, 0u};
-#else
             return *reinterpret_cast<const u32x4 *>(t.b_base[bp] + (int64_t)s * t.b_pack_b +
                                                     (uint32_t)(pt * 16));
-#endif
         };
         auto issue = [&](const Thr &t, int s, const Idx &ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
 #pragma unroll
@@ -829,7 +832,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         TW_WS_PHASE(6, 256)
         Item cur = make_item(blockIdx.x);
         Item nxt = cur;
-        bool have_next = false, first = true;
+        bool have_next = false;
 #ifdef TW_EXP_TIMING
         if (cur.u.k_pad >= 0)
             TW_WS_PHASE(7, 256)
@@ -839,14 +842,13 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
             TW_WS_PHASE(6, 256)
 #endif
-            if (!first || item >= p.n_pipe_items) {
+            if (item >= p.n_pipe_items) { // no step, no pipeline barrier to ride on
                 nxt = claim();
                 have_next = true;
             }
 #if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
             TW_WS_PHASE(7, 256)
 #endif
-            first = false;
             if (item >= p.n_gemm_items) {
                 zero_fill(item);
             } else {
@@ -872,10 +874,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                             issue(tc, j, ix[j], a_ring[j], b_ring[j]);
                 }
                 TW_WS_PHASE(0, 256)
-                if (!have_next) {
-                    nxt = claim();
-                    have_next = true;
-                }
                 TW_WS_PHASE(1, 256)
                 // time slot j: write step j (loaded R slots ago) into stage j & 1 and reuse its
                 // registers for the loads of step j + R.  Every register is written to LDS and
@@ -914,6 +912,10 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     TW_WS_STAMP(j, 4, 256)
                     TW_LDS_BARRIER();
                     TW_WS_STAMP(j, 5, 256)
+                    if (j == 0 && !have_next) {
+                        nxt = published();
+                        have_next = true;
+                    }
                 };
                 int j0 = 0;
                 for (; j0 + 2 * R <= nsteps; j0 += R) {
@@ -970,14 +972,13 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         // ================= multiplying waves ==============================================
         Item cur = make_item(blockIdx.x);
         Item nxt = cur;
-        bool have_next = false, first = true;
+        bool have_next = false;
         while (cur.ticket < p.n_items) {
             const int item = cur.ticket;
-            if (!first || item >= p.n_pipe_items) {
+            if (item >= p.n_pipe_items) {
                 nxt = claim();
                 have_next = true;
             }
-            first = false;
             if (item >= p.n_gemm_items) {
                 zero_fill(item);
             } else {
@@ -992,10 +993,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #pragma unroll
                         for (int r = 0; r < 16; ++r)
                             acc[mi][ni][r] = 0.0f;
-                if (!have_next) {
-                    nxt = claim();
-                    have_next = true;
-                }
                 const bool w_active = m0 + wave * 64 < cur.m_end;
                 auto frags = [&](int s, int ks, u32x4(&af)[MI], u32x4(&bf)[NI]) {
                     const uint16_t *const stA = sA + (s & 1) * ASTAGE;
@@ -1021,14 +1018,16 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     for (int ni = 0; ni < NI; ++ni)
                         bf[ni] = *reinterpret_cast<const u32x4 *>(stB + ((ni * KS + ks) * 64 + lane) * 8);
                 };
+                if (!have_next)
+                    publish();
                 TW_LDS_BARRIER(); // time slot 0: step 0 is being staged
+                if (!have_next) {
+                    nxt = published();
+                    have_next = true;
+                }
                 for (int s = 0; s < nsteps; ++s) {
                     TW_WS_STAMP(s, 0, 0)
-#ifdef TW_EXP_NOMFMA
-                    if (w_active && s == 0) {
-#else
                     if (w_active) {
-#endif
                         u32x4 af[2][MI], bf[2][NI];
                         frags(s, 0, af[0], bf[0]);
 #pragma unroll

@@ -145,6 +145,26 @@ int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t 
                             const int32_t *tile_width, const uint8_t *mask, const float *B,
                             tw_plan **out);
 
+/* The same for a mask whose tiles need not be rows x columns: a tile keeps every row and every
+ * column that holds a kept element, and the elements the mask drops inside that cover are stored
+ * as zeros, so the product is exactly A (B (.) mask) for ANY mask.  This runs the reference's
+ * mixed masks (tiled_wise_1d_mix / tiled_wise_2d_mix, Pruning/VGG/prune_algo.py:151-193: a TW
+ * mask plus a small element-wise remainder) on the same kernel; each remainder element costs
+ * the tile one more row (and column) of matrix-core work. */
+int tw_plan_from_mask_cover(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                            const int32_t *tile_width, const uint8_t *mask, const float *B,
+                            tw_plan **out);
+
+/* Build a plan from one layer of the reference's exported pruned model (exportPrunedModel,
+ * Pruning/BERT/utils/MyHook.py:54-89): mask_i / mask_o are the relative offsets
+ * (convert_mask_to_offset, :66-74) of the n_kept_k kept rows and n_kept_n kept columns, kernel is
+ * the compacted weight kernel[mask_i][:, mask_o], fp32 row-major [n_kept_k, n_kept_n] (:80-81);
+ * all host memory.  K and N are the layer's unpruned sizes (N is the length of the exported
+ * bias; K is not stored in the file: any K above the last kept row gives the same product).
+ * The plan has one tile over all columns. */
+int tw_plan_from_export(int K, int N, int dtype, int n_kept_k, const int32_t *mask_i,
+                        int n_kept_n, const int32_t *mask_o, const float *kernel, tw_plan **out);
+
 /* Build a plan from the operands of the reference's Stream_Gemm_NN
  * (basic_nn.cu:378-393): B_stream is the compacted weight in DEVICE memory in
  * the layout of gen_masked_stream_weight (:757-769; tile t column-major with
@@ -280,6 +300,16 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
 int tw_prune_granularity(int K, int N, const float *scores, double sparsity, int q_type,
                          int granularity, uint8_t *mask, void *stream);
 
+/* tw_mix_fn (Pruning/VGG/prune_algo.py:151-179), the second stage of tiled_wise_1d_mix and
+ * tiled_wise_2d_mix (:182-193): every element scores sqrt(x*x) minus 1 where layer_masks (the
+ * TW masks of the first stage, run at sparsity + g1percent) already keeps it; the elements
+ * strictly above the (100 - g1percent)-th percentile of all scores join the mask:
+ * masks = layer_masks | extra.  masks[l] may be layer_masks[l].  q_type as above, by the type of
+ * g1percent. */
+int tw_prune_mix(int n_layers, const int32_t *K, const int32_t *N, const float *const *scores,
+                 const uint8_t *const *layer_masks, double g1percent, int q_type,
+                 uint8_t *const *masks, double *threshold, void *stream);
+
 /* The building blocks of the two producers, on device buffers:
  *   tw_prune_tile_row_norms   norms[t*K + k] = ||scores[k][tile t]|| / width_t in NumPy's float32
  *                             summation order; col_keep (optional, N bytes) zeroes pruned
@@ -301,6 +331,16 @@ int tw_tiles_every_g_columns(int N, int G, int32_t *tile_col0, int32_t *tile_wid
                              int32_t *n_tiles);
 int tw_tiles_every_g_kept_columns(int N, int G, const uint8_t *col_mask, int32_t *tile_col0,
                                   int32_t *tile_width, int32_t *n_tiles);
+
+/* A tile table for a mask whose tiling is not known (host; mask is K x N bytes, row-major), e.g.
+ * the name -> mask dictionaries the reference's pruning runs store (Pruning/VGG/pruning.py:580-581,
+ * 639-640; Pruning/NMT/nmt/train.py:741-742).  Left to right, a tile takes columns while their
+ * kept rows equal those of the tile's first non-empty column, up to G of them (G <= 0: no limit);
+ * empty columns join the tile they fall into.  Every tile of the result is rows x columns, so
+ * tw_plan_from_mask_tiles accepts it for ANY mask; a mask that is not tile-wise merely gets
+ * narrow tiles.  tile_col0 and tile_width need room for N entries. */
+int tw_tiles_from_mask(int K, int N, int G, const uint8_t *mask, int32_t *tile_col0,
+                       int32_t *tile_width, int32_t *n_tiles);
 
 #ifdef __cplusplus
 }

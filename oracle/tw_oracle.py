@@ -19,6 +19,7 @@ Pins (the reference holds no golden vectors for this path):
   tw_gemm_reference      numpy.matmul on B*mask  vs  the per-tile
                          gather -> GEMM -> scatter form (stream_gemm_nn)
   mask_dense             numpy.matmul
+  export_pruned_model    hand known answer; export -> scatter back == kernel * outer(mi, mo)
   checkout               hand cases
 """
 import ctypes
@@ -125,6 +126,30 @@ def offsets_to_kept(offsets):
     """Relative offsets -> ascending kept indices (i + mask[i], basic_nn.cu:154)."""
     offsets = np.asarray(offsets, dtype=np.int32)
     return offsets + np.arange(offsets.size, dtype=np.int32)
+
+
+def export_pruned_model(layers):
+    """The dictionary the reference's export hook pickles, Pruning/BERT/utils/MyHook.py:54-89,
+    restated with its own loop: per layer (scope, mi [K], mo [N], kernel [K,N], bias [N]) the
+    entries scope/mask-i:0, mask-o:0 (relative offsets), kernel:0 (kept rows, then kept
+    columns) and bias:0 (bias * mo), in that order."""
+    def convert_mask_to_offset(mask):          # :66-74
+        offset = []
+        for index in range(len(mask)):
+            if mask[index] == 1:
+                offset.append(index - len(offset))
+        return np.array(offset, dtype=np.int64)
+
+    ckpt = {}
+    for scope, mi, mo, kernel, bias in layers:
+        mi, mo = np.asarray(mi), np.asarray(mo)
+        k = np.asarray(kernel)[np.array(mi, dtype=bool)]          # :80
+        k = (k.T[np.array(mo, dtype=bool)]).T                     # :81
+        ckpt[scope + "/mask-i:0"] = convert_mask_to_offset(mi)
+        ckpt[scope + "/mask-o:0"] = convert_mask_to_offset(mo)
+        ckpt[scope + "/kernel:0"] = k
+        ckpt[scope + "/bias:0"] = np.asarray(bias) * mo           # :79
+    return ckpt
 
 
 def tile_partition(M, N, K, N_pruned, K_pruned, n_dim=128):

@@ -7,7 +7,9 @@ network's importance scores into tile-wise (TW) masks:
   Pruning/BERT/utils/MyHook.py:226-259, is the same computation for N % G == 0);
 * ``tiled_wise_2d``  - Pruning/VGG/prune_algo.py:55-112 (BERT type 8,
   MyHook.py:261-313, is the same without the sparsity transform of line 61);
-* ``granularity_pruning`` - MyHook.py:202-214 (one threshold per tile).
+* ``granularity_pruning`` - MyHook.py:202-214 (one threshold per tile);
+* ``tw_mix_fn``, ``tiled_wise_1d_mix``, ``tiled_wise_2d_mix`` - prune_algo.py:151-193 (a TW mask
+  plus the largest remaining single elements).
 
 Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
 module; the product path (tilesparsity_amd.twprune -> libtwgemm.so) never does.
@@ -198,6 +200,32 @@ def tiled_wise_2d(scores, sparsity, granularity=128, transform=True):
     return masks, (thr_c, thr_r), tables, col_masks
 
 
+def tw_mix_fn(scores, g1percent, layer_masks):
+    """Second stage of the mixed (TEW) producers, prune_algo.py:151-179: every element scores
+    ||x|| over a tile of one column (sqrt(x*x) / 1 in float32) minus the TW mask (so kept
+    elements drop by 1); the elements strictly above the (100 - g1percent)-th percentile of
+    all of them are added to the masks.  Returns (masks, threshold)."""
+    scores = [np.asarray(s, F32) for s in scores]
+    vals = []
+    for s, m in zip(scores, layer_masks):
+        nrm = np.sqrt((s * s).astype(F32)).astype(F32) / F32(1)          # :158
+        vals.append((nrm - np.asarray(m, bool).astype(F32)).astype(F32))  # :160
+    thr = np.percentile(np.concatenate([v.ravel() for v in vals]), 100 - g1percent)   # :166
+    return [np.asarray(m, bool) | (v > thr) for m, v in zip(layer_masks, vals)], thr
+
+
+def tiled_wise_1d_mix(scores, sparsity, granularity=128, g1percent=5):
+    """prune_algo.py:182-186."""
+    masks, _, _ = tiled_wise_1d(scores, sparsity + g1percent, granularity)
+    return tw_mix_fn(scores, g1percent, masks)[0]
+
+
+def tiled_wise_2d_mix(scores, sparsity, granularity=128, g1percent=1):
+    """prune_algo.py:189-193."""
+    masks, _, _, _ = tiled_wise_2d(scores, sparsity + g1percent, granularity)
+    return tw_mix_fn(scores, g1percent, masks)[0]
+
+
 def granularity_pruning(score, sparsity, granularity):
     """One threshold per tile over that tile's row norms (not divided by the width); N must
     be a multiple of the granularity.  MyHook.py:202-214."""
@@ -215,6 +243,34 @@ def img2col(score):
     (prune_algo.py:16-24)."""
     score = np.abs(np.asarray(score, F32))
     return score.reshape(-1, score.shape[-1]) if score.ndim == 4 else score
+
+
+def tiles_from_mask(mask, g=0):
+    """(col0, width) tiles for a mask whose tiling is unknown: left to right a tile takes
+    columns while their kept rows equal those of its first non-empty column, at most g of them
+    (0: no limit); empty columns join the tile they fall into.  Columns are compared exactly."""
+    mask = np.asarray(mask) != 0
+    n = mask.shape[1]
+    tiles, start, kept, cur = [], 0, 0, None
+    for c in range(n):
+        col = mask[:, c]
+        if not col.any():
+            continue
+        if kept > 0 and (not np.array_equal(col, cur) or (g > 0 and kept == g)):
+            tiles.append((start, c - start))
+            start, kept = c, 0
+        cur = col
+        kept += 1
+    tiles.append((start, n - start))
+    return tiles
+
+
+def cover_tiles_from_mask(mask, table):
+    """Tile dicts whose rows / columns are every row / column holding a kept element of the
+    tile (the covering plan of an arbitrary mask)."""
+    mask = np.asarray(mask) != 0
+    return [dict(col0=int(c0), width=int(w), kept_k=np.flatnonzero(mask[:, c0:c0 + w].any(axis=1)).tolist(),
+                 kept_n=np.flatnonzero(mask[:, c0:c0 + w].any(axis=0)).tolist()) for c0, w in table]
 
 
 def plan_tiles_from_mask(mask, table):

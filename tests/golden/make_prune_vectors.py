@@ -7,7 +7,8 @@ Run in the development container only (it needs /root/reference):
     python tests/golden/make_prune_vectors.py
 
 It imports the NumPy-only module Pruning/VGG/prune_algo.py of the reference and calls
-img2col_forward, tiled_wise_1d and tiled_wise_2d on synthetic scores.  The fixture holds data
+img2col_forward, tiled_wise_1d, tiled_wise_2d, tiled_wise_1d_mix and tiled_wise_2d_mix on
+synthetic scores.  The fixture holds data
 only: the seeds' score tensors (float32), the call parameters and the returned masks (packed
 bits).  The NumPy version that executed the reference is recorded, because np.percentile's
 arithmetic type depends on it.
@@ -55,6 +56,20 @@ def main():
                 for i, m in enumerate(masks):
                     m = np.asarray(m)
                     out["%s/%s/%s/m%d" % (name, fn, repr(sp), i)] = np.packbits(m.astype(bool), axis=None)
+        # the mixed producers (TW at sparsity + g1percent, then the element-wise remainder)
+        mix = []
+        for sp in sparsities:
+            for fn, g1 in (("tiled_wise_1d_mix", 5), ("tiled_wise_2d_mix", 1),
+                           ("tiled_wise_1d_mix", 2.5)):
+                if sp + g1 > 100:
+                    continue
+                masks = getattr(ref, fn)(scores, sp, g, g1)
+                for i, m in enumerate(masks):
+                    m = np.asarray(m)
+                    out["%s/%s/%s/%s/m%d" % (name, fn, repr(sp), repr(g1), i)] = \
+                        np.packbits(m.astype(bool), axis=None)
+                mix.append([fn, repr(sp), repr(g1)])
+        meta.setdefault("mix", {})[name] = mix
         meta["cases"].append(dict(name=name, shapes=[list(s) for s in shapes], granularity=g,
                                   sparsities=[repr(s) for s in sparsities], seed=seed, quantise=quant))
     out["meta"] = np.frombuffer(json.dumps(meta).encode(), dtype=np.uint8)

@@ -1,0 +1,128 @@
+"""GPU parity of the mixed (TW + element-wise remainder) producers, tw_prune_mix through the C
+ABI, against the golden vectors of the reference's prune_algo.py:151-193 and the CPU oracle;
+and of the covering plan that runs such masks on the TW kernel.
+
+Masks: bit-exact.  GEMM on a covering plan: max relative error <= 1e-2 (fp16) / 2e-2 (bf16)
+against the float64 product of the 16-bit operands with the mask applied."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests.test_gpu_gemm import run_gemm
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden", "prune_vectors.npz")
+
+
+@pytest.fixture(scope="module")
+def twprune(tw):
+    from tilesparsity_amd import twprune as m
+    return m
+
+
+@pytest.fixture(scope="module")
+def po():
+    from oracle import tw_prune_oracle
+    return tw_prune_oracle
+
+
+def parse(text):
+    return int(text) if text.lstrip("-").isdigit() else float(text)
+
+
+def test_golden_vectors_mix(twprune):
+    z = np.load(GOLD)
+    meta = json.loads(bytes(z["meta"]).decode())
+    for case in meta["cases"]:
+        name, g = case["name"], case["granularity"]
+        scores = twprune.img2col_forward([z["%s/w%d" % (name, i)] for i in range(len(case["shapes"]))])
+        for fn, sp, g1 in meta["mix"][name]:
+            print("case", name, fn, sp, g1, flush=True)
+            got = getattr(twprune, fn)(scores, parse(sp), g, parse(g1))
+            for i, m in enumerate(got):
+                want = np.unpackbits(z["%s/%s/%s/%s/m%d" % (name, fn, sp, g1, i)])[:m.size]
+                assert np.array_equal(m.ravel(), want.astype(bool)), (name, fn, sp, g1, i)
+
+
+SHAPES = [
+    [(64, 256), (128, 384)],
+    [(100, 130), (33, 500), (257, 64)],
+    [(3, 3, 16, 48), (48, 72)],
+    [(1, 1)],
+]
+
+
+@pytest.mark.parametrize("shapes", SHAPES)
+@pytest.mark.parametrize("g1", [5, 1, 2.5, 0, np.float64(3.0)])
+def test_mix_matches_oracle(twprune, po, shapes, g1):
+    rng = np.random.default_rng(abs(hash((str(shapes), float(g1)))) % 2 ** 31)
+    scores = twprune.img2col_forward([rng.standard_normal(s).astype(np.float32) for s in shapes])
+    for sp, g in ((75, 32), (50.0, 128), (90, 8)):
+        print("mix", shapes, repr(g1), sp, g, flush=True)
+        for fn in ("tiled_wise_1d_mix", "tiled_wise_2d_mix"):
+            want = getattr(po, fn)(scores, sp, g, g1)
+            got = getattr(twprune, fn)(scores, sp, g, g1)
+            for w, m in zip(want, got):
+                assert np.array_equal(w, m), (fn, sp, g)
+    # the second stage alone, on masks that are not tile-wise at all
+    masks = [rng.random(s.shape) < 0.3 for s in scores]
+    want, thr = po.tw_mix_fn(scores, g1, masks)
+    got = twprune.tw_mix_fn(scores, g1, masks)
+    assert np.float64(thr) == twprune.tw_mix_fn.last_threshold
+    for w, m in zip(want, got):
+        assert np.array_equal(w, m)
+
+
+def test_mix_ties_and_extremes(twprune, po):
+    rng = np.random.default_rng(41)
+    scores = [(np.round(rng.standard_normal((96, 128)) * 2) / 2).astype(np.float32) for _ in range(2)]
+    scores = twprune.img2col_forward(scores)
+    for sp, g1 in ((50, 5), (0, 100), (95, 5), (60, 33.3), (99, 1)):
+        want = po.tiled_wise_1d_mix(scores, sp, 16, g1)
+        got = twprune.tiled_wise_1d_mix(scores, sp, 16, g1)
+        for a, b in zip(want, got):
+            assert np.array_equal(a, b), (sp, g1)
+
+
+def test_mix_error_paths(tw, twprune):
+    with pytest.raises(tw.TwError):
+        twprune.tiled_wise_1d_mix([np.ones((4, 4), np.float32)], 50, 2, 120)   # percentile < 0
+    with pytest.raises(tw.TwError):
+        twprune.tiled_wise_1d_mix([np.ones((4, 4), np.float32)], 98, 2, 5)     # TW stage > 100
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_cover_plan_runs_mixed_masks(tw, twprune, po, oracle, dtype):
+    """A mixed mask is not tile-wise (the plain builder refuses it); the covering plan computes
+    A (B (.) mask) exactly as masked, and its lists are the union of each tile's elements."""
+    rng = np.random.default_rng(42)
+    K, N, G, M = 320, 384, 128, 200
+    W = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    # structured magnitudes, so that the remainder does not touch every row of every tile
+    W *= (rng.random((K, 1)) < 0.5) * 0.9 + 0.1
+    scores = twprune.img2col_forward([W])
+    mask = twprune.tiled_wise_1d_mix(scores, 70, G, 2)[0]
+    table = po.tiles_every_g_columns(N, G)
+    with pytest.raises(tw.TwError) as e:
+        tw.Plan.from_mask_tiles(mask, table, dtype, W)
+    assert e.value.status == tw.ERR_NOT_TW
+    with tw.Plan.from_mask_tiles(mask, table, dtype, W, cover=True) as plan:
+        ex, _ = plan.export(with_weight=False)
+        want = po.cover_tiles_from_mask(mask, table)
+        for t, wt in zip(ex, want):
+            assert t["kept_k"].tolist() == wt["kept_k"] and t["kept_n"].tolist() == wt["kept_n"]
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        C, _ = run_gemm(tw, oracle, plan, A, dtype, N, pruned=1)
+        ref = oracle.quantize(A, dtype).astype(np.float64) @ (oracle.quantize(W, dtype) * mask).astype(np.float64)
+        assert oracle.rel_error(C, ref) <= (1e-2 if dtype == "f16" else 2e-2)
+    # a tile-wise mask gives the same plan with and without `cover`
+    m1 = twprune.tiled_wise_1d(scores, 70, G)[0]
+    with tw.Plan.from_mask_tiles(m1, table, dtype, W) as p1, \
+            tw.Plan.from_mask_tiles(m1, table, dtype, W, cover=True) as p2:
+        (t1, b1), (t2, b2) = p1.export(), p2.export()
+        assert np.array_equal(b1, b2)
+        for a, b in zip(t1, t2):
+            assert np.array_equal(a["kept_k"], b["kept_k"]) and np.array_equal(a["kept_n"], b["kept_n"])

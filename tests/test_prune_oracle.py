@@ -43,6 +43,40 @@ def test_oracle_matches_reference_vectors(name, sp):
             assert np.array_equal(m, want), (name, fn, sp, i)
 
 
+def gold_mix_cases():
+    _, meta = load_gold()
+    for name, calls in meta["mix"].items():
+        for fn, sp, g1 in calls:
+            yield name, fn, sp, g1
+
+
+@pytest.mark.parametrize("name,fn,sp,g1", list(gold_mix_cases()))
+def test_mix_oracle_matches_reference_vectors(name, fn, sp, g1):
+    z, meta = load_gold()
+    case = next(c for c in meta["cases"] if c["name"] == name)
+    scores = [po.img2col(z["%s/w%d" % (name, i)]) for i in range(len(case["shapes"]))]
+    masks = getattr(po, fn)(scores, parse_sparsity(sp), case["granularity"], parse_sparsity(g1))
+    for i, m in enumerate(masks):
+        want = np.unpackbits(z["%s/%s/%s/%s/m%d" % (name, fn, sp, g1, i)])[:m.size].reshape(m.shape)
+        assert np.array_equal(m, want.astype(bool)), (name, fn, sp, g1, i)
+
+
+def test_mix_adds_exactly_the_largest_unkept_elements():
+    """Property check of tw_mix_fn against a sort: without ties, the added elements are the
+    top g1percent of the shifted scores, and nothing kept by the TW mask is lost."""
+    rng = np.random.default_rng(21)
+    scores = [np.abs(rng.standard_normal(s)).astype(np.float32) for s in [(40, 64), (30, 50)]]
+    tw_masks, _, _ = po.tiled_wise_1d(scores, 80, 16)
+    mixed, thr = po.tw_mix_fn(scores, 5, tw_masks)
+    shifted = np.concatenate([(s - m).ravel() for s, m in zip(scores, tw_masks)])
+    n_extra = int(np.sum(shifted > thr))
+    assert abs(n_extra - 0.05 * shifted.size) <= 1
+    top = np.sort(shifted)[-n_extra:]
+    assert top[0] > thr >= np.sort(shifted)[-n_extra - 1]
+    for m0, m1 in zip(tw_masks, mixed):
+        assert np.all(m1[m0])
+
+
 def test_fixture_was_written_by_this_numpy_family():
     _, meta = load_gold()
     # np.percentile keeps float32 arithmetic for float32 data since NumPy 2; the fixture and the

@@ -4,6 +4,7 @@
 #include "tw_internal.h"
 
 #include <cstring>
+#include <vector>
 
 namespace tw {
 
@@ -181,6 +182,47 @@ int tw_tile_partition(int M, int N, int K, int N_pruned, int K_pruned, int n_dim
         oc += (int64_t)M * N_ori[i];
     }
     *block_num = bn;
+    return TW_OK;
+}
+
+int tw_tiles_from_mask(int K, int N, int G, const uint8_t *mask, int32_t *tile_col0,
+                       int32_t *tile_width, int32_t *n_tiles)
+{
+    if (K <= 0 || N <= 0)
+        return tw::fail(TW_ERR_SHAPE, "K=%d N=%d must be positive", K, N);
+    if (!mask || !tile_col0 || !tile_width || !n_tiles)
+        return tw::fail(TW_ERR_NULL, "a pointer is NULL");
+    // One pass over the rows: a position-dependent 64-bit fingerprint of every column's kept
+    // rows (two columns with different rows collide with probability 2^-64; the plan builders
+    // check every element of every tile afterwards, so a collision surfaces as TW_ERR_NOT_TW).
+    std::vector<uint64_t> sig((size_t)N, 0);
+    std::vector<uint8_t> any((size_t)N, 0);
+    for (int k = 0; k < K; ++k) {
+        const uint8_t *row = mask + (size_t)k * N;
+        for (int c = 0; c < N; ++c) {
+            const uint64_t bit = row[c] != 0;
+            sig[c] = sig[c] * 0x9E3779B97F4A7C15ull + bit * 0xD6E8FEB86659FD93ull;
+            any[c] |= (uint8_t)bit;
+        }
+    }
+    int t = 0, start = 0, kept = 0;
+    uint64_t cur = 0;
+    for (int c = 0; c < N; ++c) {
+        if (!any[c])
+            continue; // an empty column rides along with the tile it falls into
+        if (kept > 0 && (sig[c] != cur || (G > 0 && kept == G))) {
+            tile_col0[t] = start;
+            tile_width[t] = c - start;
+            ++t;
+            start = c;
+            kept = 0;
+        }
+        cur = sig[c];
+        ++kept;
+    }
+    tile_col0[t] = start;
+    tile_width[t] = N - start;
+    *n_tiles = t + 1;
     return TW_OK;
 }
 

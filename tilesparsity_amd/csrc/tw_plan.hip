@@ -621,9 +621,9 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     return tw_plan_from_mask_tiles(K, N, dtype, nt, col0.data(), width.data(), mask, B, out);
 }
 
-int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
-                            const int32_t *tile_width, const uint8_t *mask, const float *B,
-                            tw_plan **out)
+static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                               const int32_t *tile_width, const uint8_t *mask, const float *B,
+                               bool cover, tw_plan **out)
 {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
@@ -706,7 +706,7 @@ int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t 
     std::vector<int32_t> counts(2 * nt);
     TW_TRY(hipMemcpy(&mismatch, d_mismatch, sizeof(mismatch), hipMemcpyDeviceToHost));
     TW_TRY(hipMemcpy(counts.data(), d_counts, sizeof(int32_t) * 2 * nt, hipMemcpyDeviceToHost));
-    if (mismatch != 0) {
+    if (mismatch != 0 && !cover) {
         cleanup();
         return fail(TW_ERR_NOT_TW,
                     "%llu mask elements differ from (row kept) & (column kept) of their tile",
@@ -759,14 +759,68 @@ int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t 
                         p->kept_k_idx.data(), p->kept_n_ptr.data(), p->kept_n_idx.data());
     if (!st)
         st = finalize_plan_geometry(p);
-    if (!st)
+    if (!st && cover && mismatch != 0) {
+        // rows and columns of a tile are the union of its elements: the elements the mask
+        // drops inside that cover are stored as zeros
+        std::vector<float> Bm((size_t)K * N);
+        for (size_t i = 0; i < Bm.size(); ++i)
+            Bm[i] = mask[i] ? B[i] : 0.0f;
+        st = pack_host_weight(p, Bm.data());
+    } else if (!st) {
         st = pack_host_weight(p, B);
+    }
     if (st) {
         free_plan(p);
         return st;
     }
     *out = p;
     return TW_OK;
+}
+
+int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                            const int32_t *tile_width, const uint8_t *mask, const float *B,
+                            tw_plan **out)
+{
+    return plan_from_mask_impl(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, false, out);
+}
+
+int tw_plan_from_mask_cover(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                            const int32_t *tile_width, const uint8_t *mask, const float *B,
+                            tw_plan **out)
+{
+    return plan_from_mask_impl(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, true, out);
+}
+
+int tw_plan_from_export(int K, int N, int dtype, int n_kept_k, const int32_t *mask_i,
+                        int n_kept_n, const int32_t *mask_o, const float *kernel, tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (K <= 0 || N <= 0 || n_kept_k < 0 || n_kept_k > K || n_kept_n < 0 || n_kept_n > N)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d with %d kept rows and %d kept columns", K, N,
+                    n_kept_k, n_kept_n);
+    if ((n_kept_k > 0 && !mask_i) || (n_kept_n > 0 && !mask_o) ||
+        (n_kept_k > 0 && n_kept_n > 0 && !kernel))
+        return fail(TW_ERR_NULL, "mask_i, mask_o or kernel is NULL");
+    std::vector<int32_t> kk((size_t)std::max(n_kept_k, 1)), kn((size_t)std::max(n_kept_n, 1));
+    int st = tw_offsets_to_kept(mask_i, n_kept_k, K, kk.data());
+    if (!st)
+        st = tw_offsets_to_kept(mask_o, n_kept_n, N, kn.data());
+    if (st)
+        return st;
+    // one tile over all columns: every unit of 128 compact columns shares the kept rows
+    std::vector<float> B((size_t)K * N, 0.0f);
+    for (int i = 0; i < n_kept_k; ++i) {
+        float *dst = B.data() + (size_t)kk[i] * N;
+        const float *src = kernel + (size_t)i * n_kept_n;
+        for (int j = 0; j < n_kept_n; ++j)
+            dst[kn[j]] = src[j];
+    }
+    const int32_t col0 = 0, width = N;
+    const int32_t kp[2] = {0, n_kept_k}, np[2] = {0, n_kept_n};
+    return tw_plan_create(K, N, dtype, 1, &col0, &width, kp, kk.data(), np, kn.data(), B.data(),
+                          out);
 }
 
 int tw_plan_from_stream_operands(int M, int N, int K, int dtype, const void *B_stream,

@@ -422,6 +422,62 @@ __global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t
 }
 
 // ---------------------------------------------------------------------------------
+// mixed masks: a TW mask plus the largest remaining single elements
+
+struct MixLayer {
+    const float *score;
+    const uint8_t *mask0; // the TW mask of the layer
+    uint8_t *out;         // may be mask0 itself
+    int64_t begin;        // first element of the layer in the pooled vector
+};
+
+__device__ inline int find_mix_layer(const MixLayer *layers, int n_layers, int64_t idx)
+{
+    int lo = 0, hi = n_layers;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (layers[mid].begin <= idx)
+            lo = mid;
+        else
+            hi = mid;
+    }
+    return lo;
+}
+
+// pool[i] = ||x|| of the single element (sqrt(x*x) / 1, the reference's norm over a tile of one
+// column) minus 1 where the TW mask already keeps it (prune_algo.py:159-161)
+__global__ void __launch_bounds__(256)
+    mix_values_kernel(const MixLayer *layers, int n_layers, int64_t total, float *pool)
+{
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const MixLayer L = layers[find_mix_layer(layers, n_layers, i)];
+        const int64_t e = i - L.begin;
+        const float x = L.score[e];
+        const float sq = x * x;
+        const float nrm = sqrtf(sq) / 1.0f;
+        pool[i] = nrm - (L.mask0[e] ? 1.0f : 0.0f);
+    }
+}
+
+// out = mask0 | (pool > threshold)   (prune_algo.py:171-176)
+__global__ void __launch_bounds__(256)
+    mix_mask_kernel(const MixLayer *layers, int n_layers, int64_t total, const float *pool,
+                    const SelectState *st, int f64)
+{
+    const float thr32 = st->thr32;
+    const double thr64 = st->thr64;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+        const MixLayer L = layers[find_mix_layer(layers, n_layers, i)];
+        const int64_t e = i - L.begin;
+        const float v = pool[i];
+        const bool extra = f64 ? (double)v > thr64 : v > thr32;
+        L.out[e] = (L.mask0[e] || extra) ? 1 : 0;
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // host side
 
 namespace {
@@ -887,6 +943,54 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
         thresholds[0] = vc;
         thresholds[1] = vr;
     }
+    return st;
+}
+
+int tw_prune_mix(int n_layers, const int32_t *K, const int32_t *N, const float *const *scores,
+                 const uint8_t *const *layer_masks, double g1percent, int q_type,
+                 uint8_t *const *masks, double *threshold, void *stream)
+{
+    int st = check_layers(n_layers, K, N, scores, masks, 1);
+    if (st)
+        return st;
+    if (!layer_masks)
+        return fail(TW_ERR_NULL, "layer_masks is NULL");
+    if (q_type != TW_Q_F32 && q_type != TW_Q_F64)
+        return fail(TW_ERR_LAYOUT, "q_type=%d: unknown", q_type);
+    hipStream_t s = (hipStream_t)stream;
+    std::vector<MixLayer> ml(n_layers);
+    int64_t total = 0;
+    for (int l = 0; l < n_layers; ++l) {
+        if (!layer_masks[l])
+            return fail(TW_ERR_NULL, "layer %d: layer mask pointer is NULL", l);
+        ml[l].score = scores[l];
+        ml[l].mask0 = layer_masks[l];
+        ml[l].out = masks[l];
+        ml[l].begin = total;
+        total += (int64_t)K[l] * N[l];
+    }
+    Arena ar;
+    float *d_pool = ar.alloc_n<float>(total);
+    MixLayer *d_layers = ar.alloc_n<MixLayer>(n_layers);
+    if (!d_pool || !d_layers)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %lld element scores failed", (long long)total);
+    TW_HIP(hipMemcpyAsync(d_layers, ml.data(), sizeof(MixLayer) * n_layers, hipMemcpyHostToDevice, s));
+    TW_HIP(hipStreamSynchronize(s)); // `ml` is pageable host memory
+    const unsigned grid = (unsigned)std::min<int64_t>((total + 255) / 256, 256 * 64);
+    hipLaunchKernelGGL(mix_values_kernel, dim3(grid), dim3(256), 0, s, d_layers, n_layers, total,
+                       d_pool);
+    TW_HIP(hipGetLastError());
+    Threshold thr;
+    st = percentile_linear(ar, d_pool, total, 100.0 - g1percent, q_type, s, &thr);
+    if (st)
+        return st;
+    hipLaunchKernelGGL(mix_mask_kernel, dim3(grid), dim3(256), 0, s, d_layers, n_layers, total,
+                       d_pool, thr.state, thr.is_f64);
+    TW_HIP(hipGetLastError());
+    double value = 0.0;
+    st = read_threshold(thr, s, &value); // waits for the masks
+    if (!st && threshold)
+        *threshold = value;
     return st;
 }
 

@@ -46,7 +46,8 @@ EXPORTED_SYMBOLS = (
     "tw_plan_from_mask_tiles", "tw_prune_tiled_wise_1d", "tw_prune_tiled_wise_2d",
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
-    "tw_prune_granularity",
+    "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
+    "tw_prune_mix",
 )
 
 
@@ -137,6 +138,11 @@ def lib():
                                          ctypes.POINTER(ctypes.c_double), vp]),
         "tw_tiles_every_g_kept_columns": (c_int, [c_int, c_int, u8p, i32p, i32p,
                                                   ctypes.POINTER(c_int)]),
+        "tw_prune_mix": (c_int, [c_int, i32p, i32p, pp, pp, ctypes.c_double, c_int, pp,
+                                 ctypes.POINTER(ctypes.c_double), vp]),
+        "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
+        "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
+        "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -207,6 +213,20 @@ def tile_partition(M, N, K, N_pruned, K_pruned, n_dim=128, max_tiles=4096):
                 K_cal=K_cal[:n].tolist(), off_B=off_B[:n].tolist(), off_C=off_C[:n].tolist())
 
 
+def tiles_from_mask(mask, G=0):
+    """[(col0, width), ...] for a mask [K,N] whose tiling is not known: a tile takes columns
+    while their kept rows equal those of its first non-empty column, at most G of them (0: no
+    limit).  Host only."""
+    mask = np.ascontiguousarray(mask, dtype=np.uint8)
+    K, N = mask.shape
+    col0, width = np.zeros(N, np.int32), np.zeros(N, np.int32)
+    n = ctypes.c_int(0)
+    _check(lib().tw_tiles_from_mask(K, N, int(G), _ptr(mask, ctypes.c_uint8),
+                                    _ptr(col0, ctypes.c_int32), _ptr(width, ctypes.c_int32),
+                                    ctypes.byref(n)))
+    return [(int(col0[t]), int(width[t])) for t in range(n.value)]
+
+
 def tiles_to_csr(tiles):
     """list of tile dicts (col0, width, kept_k, kept_n) -> the six flat arrays."""
     col0 = _i32([t["col0"] for t in tiles])
@@ -275,8 +295,10 @@ class Plan:
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod
-    def from_mask_tiles(cls, mask, tile_table, dtype, B):
-        """From a dense 0/1 mask [K,N] and an explicit tile table [(col0, width), ...]."""
+    def from_mask_tiles(cls, mask, tile_table, dtype, B, cover=False):
+        """From a dense 0/1 mask [K,N] and an explicit tile table [(col0, width), ...].  With
+        ``cover`` a tile need not be rows x columns: it keeps every row and column that holds a
+        kept element and stores the dropped elements inside as zeros (any mask is accepted)."""
         mask = np.ascontiguousarray(mask, dtype=np.uint8)
         K, N = mask.shape
         B = np.ascontiguousarray(B, dtype=np.float32)
@@ -285,10 +307,26 @@ class Plan:
         col0 = _i32([t[0] for t in tile_table])
         width = _i32([t[1] for t in tile_table])
         h = ctypes.c_void_p()
-        _check(lib().tw_plan_from_mask_tiles(K, N, dtype_code(dtype), len(tile_table),
-                                             _ptr(col0, ctypes.c_int32), _ptr(width, ctypes.c_int32),
-                                             _ptr(mask, ctypes.c_uint8), _ptr(B, ctypes.c_float),
-                                             ctypes.byref(h)))
+        fn = lib().tw_plan_from_mask_cover if cover else lib().tw_plan_from_mask_tiles
+        _check(fn(K, N, dtype_code(dtype), len(tile_table), _ptr(col0, ctypes.c_int32),
+                  _ptr(width, ctypes.c_int32), _ptr(mask, ctypes.c_uint8), _ptr(B, ctypes.c_float),
+                  ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def from_export(cls, K, N, dtype, mask_i, mask_o, kernel):
+        """From one layer of an exported pruned model: relative offsets of the kept rows and
+        columns and the compacted fp32 weight [len(mask_i), len(mask_o)]."""
+        mask_i, mask_o = _i32(mask_i), _i32(mask_o)
+        kernel = np.ascontiguousarray(kernel, dtype=np.float32)
+        if kernel.size != mask_i.size * mask_o.size:
+            raise TwError(ERR_SHAPE, "kernel has %d elements, expected %d x %d"
+                          % (kernel.size, mask_i.size, mask_o.size))
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_from_export(K, N, dtype_code(dtype), mask_i.size,
+                                         _ptr(mask_i, ctypes.c_int32), mask_o.size,
+                                         _ptr(mask_o, ctypes.c_int32), _ptr(kernel, ctypes.c_float),
+                                         ctypes.byref(h)))
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod

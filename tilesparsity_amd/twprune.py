@@ -1,6 +1,7 @@
 """TW mask producers on the GPU, with the reference's function names and argument meaning
-(Pruning/VGG/prune_algo.py: img2col_forward, tiled_wise_1d, tiled_wise_2d; BERT pruning types 7
-and 8 of Pruning/BERT/utils/MyHook.py are tiled_wise_1d and tiled_wise_2d(transform=False)).
+(Pruning/VGG/prune_algo.py: img2col_forward, tiled_wise_1d, tiled_wise_2d, tw_mix_fn,
+tiled_wise_1d_mix, tiled_wise_2d_mix; BERT pruning types 7 and 8 of Pruning/BERT/utils/MyHook.py
+are tiled_wise_1d and tiled_wise_2d(transform=False)).
 
     masks = tiled_wise_1d(scores, sparsity, granularity)     # list of bool [K, N] arrays
 
@@ -100,6 +101,54 @@ def tiled_wise_2d(accumulated_scores, sparsity, granularity=128, transform=True,
         return masks
     tables = [tiles_every_g_kept_columns(c.cpu().numpy(), granularity) for c in d.d_cols]
     return masks, tables
+
+
+def _mix(d, g1percent, return_device):
+    """Second stage of the mixed producers on the device masks already in ``d``."""
+    thr = ctypes.c_double()
+    pm = ctypes.cast(d.p_masks, ctypes.POINTER(ctypes.c_void_p))
+    tw._check(tw.lib().tw_prune_mix(
+        len(d.shapes), tw._ptr(d.K, ctypes.c_int32), tw._ptr(d.N, ctypes.c_int32),
+        ctypes.cast(d.p_scores, ctypes.POINTER(ctypes.c_void_p)), pm, float(g1percent),
+        _q_type(100 - g1percent), pm, ctypes.byref(thr), d.stream))
+    tw_mix_fn.last_threshold = thr.value
+    return d.d_masks if return_device else d.masks()
+
+
+def tw_mix_fn(accumulated_scores, g1percent, layer_mask, return_device=False):
+    """prune_algo.py:151-179: the elements whose |score| (minus 1 where ``layer_mask`` keeps
+    them) lies above the (100 - g1percent)-th percentile of the whole network join the masks."""
+    d = _DeviceLayers(accumulated_scores)
+    for dst, m in zip(d.d_masks, layer_mask):
+        if isinstance(m, d.torch.Tensor):
+            dst.copy_(m.reshape(dst.shape).to(device="cuda", dtype=d.torch.uint8))
+        else:
+            dst.copy_(d.torch.from_numpy(np.ascontiguousarray(np.asarray(m) != 0).view(np.uint8)
+                                         .reshape(dst.shape)))
+    return _mix(d, g1percent, return_device)
+
+
+def tiled_wise_1d_mix(accumulated_scores, sparsity, granularity=128, g1percent=5, return_device=False):
+    """prune_algo.py:182-186: tiled_wise_1d at sparsity + g1percent, then tw_mix_fn."""
+    d = _DeviceLayers(accumulated_scores)
+    q = sparsity + g1percent
+    tw._check(tw.lib().tw_prune_tiled_wise_1d(
+        len(d.shapes), tw._ptr(d.K, ctypes.c_int32), tw._ptr(d.N, ctypes.c_int32),
+        ctypes.cast(d.p_scores, ctypes.POINTER(ctypes.c_void_p)), float(q), _q_type(q),
+        int(granularity), ctypes.cast(d.p_masks, ctypes.POINTER(ctypes.c_void_p)), None, d.stream))
+    return _mix(d, g1percent, return_device)
+
+
+def tiled_wise_2d_mix(accumulated_scores, sparsity, granularity=128, g1percent=1, return_device=False):
+    """prune_algo.py:189-193: tiled_wise_2d at sparsity + g1percent, then tw_mix_fn."""
+    d = _DeviceLayers(accumulated_scores)
+    q = sparsity + g1percent
+    tw._check(tw.lib().tw_prune_tiled_wise_2d(
+        len(d.shapes), tw._ptr(d.K, ctypes.c_int32), tw._ptr(d.N, ctypes.c_int32),
+        ctypes.cast(d.p_scores, ctypes.POINTER(ctypes.c_void_p)), float(q), _q_type(q), 1,
+        int(granularity), ctypes.cast(d.p_masks, ctypes.POINTER(ctypes.c_void_p)),
+        ctypes.cast(d.p_cols, ctypes.POINTER(ctypes.c_void_p)), None, d.stream))
+    return _mix(d, g1percent, return_device)
 
 
 def granularity_pruning(score, sparsity, granularity):

@@ -79,11 +79,14 @@ template <> struct Elem<TW_BF16> {
     }
 };
 
-// 16-byte chunk of column c, rows m..m+7 of a K-major matrix, honouring the M edge
+// 16-byte chunk of column c, rows m..m+7 of a K-major matrix, honouring the M edge.  The store
+// writes through to memory (sc0 sc1) and does not linger in the caches (nt): C is written once
+// and not read again by this launch, and lines left dirty in the L2s would otherwise all be
+// written back after the last wave has ended, where nothing overlaps them.
 __device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M)
 {
     if (m + 8 <= M) {
-        *reinterpret_cast<u32x4 *>(dst) = v;
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
     } else if (m < M) {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         for (int e = 0; e < M - m; ++e)

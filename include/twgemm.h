@@ -256,6 +256,21 @@ int tw_delete_row(const void *matrix, void *matrix_2, int rows, int columns,
 int tw_insert_row(void *matrix, const void *matrix_2, int rows, int columns,
                   const int32_t *mask, void *stream);
 
+/* LSTM gate arithmetic of the reference's NMT model, whose cells are TensorFlow 1.x
+ * tf.contrib.rnn.BasicLSTMCell (Pruning/NMT/nmt/model_helper.py:400-402; BasicLSTMCell.call in
+ * tensorflow/python/ops/rnn_cell_impl.py): with i, j, f, o the four H-wide blocks of the gate
+ * pre-activations (inputs and h concatenated, times the masked kernel, plus bias: one
+ * tw_gemm_ex with N = 4H),
+ *   c_new = c_prev * sigmoid(f + forget_bias) + sigmoid(i) * tanh(j)
+ *   h_new = tanh(c_new) * sigmoid(o)
+ * All matrices are K-major device buffers: gates [4H][ldg] of `dtype` (the GEMM's C), c_prev and
+ * c_new fp32 [H][ld] (may be the same buffer), h_new [H][ldh] of `dtype`, which may point into
+ * the rows of the next time step's A that hold h (the cell input is concat([x, h])), so that
+ * the recurrence needs no transpose or copy.  fp32 arithmetic, one rounding of h. */
+int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg, float forget_bias,
+                  const float *c_prev, int64_t ldc_prev, float *c_new, int64_t ldc_new,
+                  void *h_new, int64_t ldh, void *stream);
+
 /* ---- TW mask producers ---------------------------------------------------------------
  * The reference derives its masks from importance scores with NumPy: per layer a 2-D score
  * matrix [K,N] (|w|; conv kernels HWIO reshaped to (H*W*I) x O, Pruning/VGG/prune_algo.py:16-24),

@@ -20,6 +20,8 @@ Pins (the reference holds no golden vectors for this path):
                          gather -> GEMM -> scatter form (stream_gemm_nn)
   mask_dense             numpy.matmul
   export_pruned_model    hand known answer; export -> scatter back == kernel * outer(mi, mo)
+  basic_lstm_cell        closed form of a third-party routine (TensorFlow is absent): limits
+                         (saturated gates), zero input, scipy.special.expit / numpy.tanh
   checkout               hand cases
 """
 import ctypes
@@ -271,6 +273,17 @@ def mask_dense(x, kernel, mask, bias=None, activation=None):
     if bias is not None:
         y = y + bias
     return ACTIVATIONS[activation](y)
+
+
+def basic_lstm_cell(gate_inputs, c, forget_bias=1.0):
+    """The gate arithmetic of TensorFlow 1.x BasicLSTMCell.call, the cell of the reference's NMT
+    model (Pruning/NMT/nmt/model_helper.py:400-402): gate_inputs [M, 4H] = concat([x, h]) @
+    kernel + bias, split into i, j, f, o; returns (new_c, new_h) in the input's precision."""
+    g = np.asarray(gate_inputs)
+    i, j, f, o = np.split(g, 4, axis=1)
+    sig = lambda v: 1.0 / (1.0 + np.exp(-v))
+    new_c = c * sig(f + forget_bias) + sig(i) * np.tanh(j)
+    return new_c, np.tanh(new_c) * sig(o)
 
 
 def tw_gemm_reference(A, B, tiles, alpha=1.0, beta=0.0, C=None, acc=np.float64):

@@ -1,0 +1,111 @@
+"""GPU parity of the LSTM gate arithmetic (tw_lstm_gates) against the oracle's BasicLSTMCell
+restatement, alone and inside a two-step recurrence that runs the reference's NMT gate GEMM
+(concat([x, h]) @ (kernel * mask) + bias) through tw_gemm_ex with the new h written straight
+into the next step's K-major A.
+
+Tolerances: c (fp32) 1e-5 relative to max |c|; h (16-bit) max relative error 1e-2 (fp16) /
+2e-2 (bf16) with the 1e-2 * rms floor, as for the GEMM."""
+import numpy as np
+import pytest
+
+from tests.helpers import from_device_bits, random_tiles, to_device_bits
+
+pytestmark = pytest.mark.gpu
+
+TOL = {"f16": 1e-2, "bf16": 2e-2}
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,H", [(128, 256), (100, 96), (7, 8), (264, 1024)])
+def test_gates_match_oracle(tw, oracle, M, H, dtype):
+    import torch
+    rng = np.random.default_rng(M * 1000 + H)
+    ld = (M + 7) // 8 * 8
+    g = (rng.standard_normal((M, 4 * H)) * 2).astype(np.float32)
+    c = rng.standard_normal((M, H)).astype(np.float32)
+    gb = np.zeros((4 * H, ld), np.uint16)
+    gb[:, :M] = oracle.cast_bits(g, dtype).reshape(M, 4 * H).T
+    cp = np.zeros((H, ld), np.float32)
+    cp[:, :M] = c.T
+    dg, dc = to_device_bits(gb, gb.shape), torch.from_numpy(cp).cuda()
+    dcn = torch.full((H, ld), 7.0, dtype=torch.float32, device="cuda")
+    dh = torch.full((H, ld), 0x3C00, dtype=torch.int16, device="cuda")
+    print("gates", M, H, dtype, flush=True)
+    tw.lstm_gates(M, H, dtype, dg.data_ptr(), ld, 1.0, dc.data_ptr(), ld, dcn.data_ptr(), ld,
+                  dh.data_ptr(), ld, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    want_c, want_h = oracle.basic_lstm_cell(oracle.quantize(g, dtype).astype(np.float64), c.astype(np.float64), 1.0)
+    got_c = dcn.cpu().numpy()
+    got_h = oracle.bits_to_f32(from_device_bits(dh), dtype).reshape(H, ld)
+    assert np.max(np.abs(got_c[:, :M].T - want_c)) <= 1e-5 * np.max(np.abs(want_c))
+    assert oracle.rel_error(got_h[:, :M].T, want_h) <= TOL[dtype]
+    # padding beyond M is not written
+    if ld > M:
+        assert np.all(got_c[:, M:] == 7.0) and np.all(from_device_bits(dh)[:, M:] == 0x3C00)
+    # in place on c
+    tw.lstm_gates(M, H, dtype, dg.data_ptr(), ld, 1.0, dc.data_ptr(), ld, dc.data_ptr(), ld,
+                  dh.data_ptr(), ld, torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert np.array_equal(dc.cpu().numpy()[:, :M], got_c[:, :M])
+
+
+def test_gate_argument_errors(tw):
+    with pytest.raises(tw.TwError):
+        tw.lstm_gates(8, 8, "f16", 0, 8, 1.0, 0, 8, 0, 8, 0, 8)
+    with pytest.raises(tw.TwError):
+        tw.lstm_gates(8, 8, "f16", 16, 4, 1.0, 16, 8, 16, 8, 16, 8)      # ldg < M
+    with pytest.raises(tw.TwError):
+        tw.lstm_gates(8, 8, "f16", 16, 12, 1.0, 16, 8, 16, 8, 16, 8)     # ldg not a multiple of 8
+    with pytest.raises(tw.TwError):
+        tw.lstm_gates(8, 0, "f16", 16, 8, 1.0, 16, 8, 16, 8, 16, 8)
+    tw.lstm_gates(0, 8, "f16", 0, 8, 1.0, 0, 8, 0, 8, 0, 8)               # M = 0: no-op
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_two_step_recurrence(tw, oracle, dtype):
+    """x_t and h_{t-1} share one K-major A; the gate kernel writes h_t into the rows of the next
+    step's A, the masked gate GEMM adds the bias in its epilogue."""
+    import torch
+    rng = np.random.default_rng(91)
+    M, I, H, G = 128, 192, 256, 128
+    K, N = I + H, 4 * H
+    W = (rng.standard_normal((K, N)) * 0.08).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.5).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.5, n_keep=1.0)
+    mask = oracle.plan_mask(K, N, tiles)
+    xs = [rng.standard_normal((M, I)).astype(np.float32) for _ in range(2)]
+    h0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    ld = M
+    s = torch.cuda.current_stream().cuda_stream
+    # A_t = [x_t ; h_{t-1}] as K-major rows
+    A = []
+    for t in range(3):
+        a = np.zeros((K, ld), np.uint16)
+        if t < 2:
+            a[:I] = oracle.cast_bits(xs[t], dtype).reshape(M, I).T
+        A.append(a)
+    A[0][I:] = oracle.cast_bits(h0, dtype).reshape(M, H).T
+    dA = [to_device_bits(a, a.shape) for a in A]
+    dC = torch.from_numpy(np.ascontiguousarray(c0.T)).cuda()
+    dG = torch.zeros((N, ld), dtype=torch.int16, device="cuda")
+    dbias = torch.from_numpy(bias).cuda()
+    esz = 2
+    with tw.Plan.create(K, N, dtype, tiles, W) as plan:
+        for t in range(2):
+            plan.gemm(dA[t].data_ptr(), dG.data_ptr(), M, lda=ld, ldc=ld, pruned_cols=tw.PRUNED_ZERO,
+                      stream=s, bias_ptr=dbias.data_ptr())
+            tw.lstm_gates(M, H, dtype, dG.data_ptr(), ld, 1.0, dC.data_ptr(), ld, dC.data_ptr(), ld,
+                          dA[t + 1].data_ptr() + I * ld * esz, ld, s)
+        torch.cuda.synchronize()
+    # oracle: the same recurrence with the 16-bit hand-overs
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+    h, c = q(h0), c0.astype(np.float64)
+    for t in range(2):
+        gates = oracle.mask_dense(np.concatenate([q(xs[t]), h], 1), q(W), mask, bias.astype(np.float64))
+        c, h = oracle.basic_lstm_cell(q(gates), c, 1.0)
+        h = q(h)
+    got_h = oracle.bits_to_f32(from_device_bits(dA[2])[I:], dtype).reshape(H, M).T
+    got_c = dC.cpu().numpy().T
+    assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
+    assert oracle.rel_error(got_c, c) <= 2 * TOL[dtype]

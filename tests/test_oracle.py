@@ -368,3 +368,32 @@ def test_gelu_and_mask_dense_epilogue():
     # a fully pruned column still gets its bias
     m[:, 2] = 0
     assert np.allclose(o.mask_dense(x, w, m, b)[:, 2], b[2])
+
+
+def test_basic_lstm_cell_closed_forms(oracle):
+    """BasicLSTMCell's gate arithmetic against library routines and its limits."""
+    from scipy.special import expit
+    rng = np.random.default_rng(77)
+    M, H = 9, 16
+    g = rng.standard_normal((M, 4 * H)) * 2
+    c = rng.standard_normal((M, H))
+    nc, nh = oracle.basic_lstm_cell(g, c, 1.0)
+    i, j, f, o = g[:, :H], g[:, H:2 * H], g[:, 2 * H:3 * H], g[:, 3 * H:]
+    want_c = c * expit(f + 1.0) + expit(i) * np.tanh(j)
+    assert np.allclose(nc, want_c, rtol=1e-12, atol=1e-12)
+    assert np.allclose(nh, np.tanh(want_c) * expit(o), rtol=1e-12, atol=1e-12)
+    # saturated gates: forget open / input shut keeps c; the opposite replaces it by tanh(j)
+    big = 40.0
+    keep = np.concatenate([np.full((M, H), -big), g[:, H:2 * H], np.full((M, H), big), np.full((M, H), big)], 1)
+    nc, nh = oracle.basic_lstm_cell(keep, c, 0.0)
+    assert np.allclose(nc, c) and np.allclose(nh, np.tanh(c))
+    repl = np.concatenate([np.full((M, H), big), g[:, H:2 * H], np.full((M, H), -big), np.full((M, H), -big)], 1)
+    nc, nh = oracle.basic_lstm_cell(repl, c, 0.0)
+    assert np.allclose(nc, np.tanh(j)) and np.allclose(nh, 0.0, atol=1e-15)
+    # zero pre-activations: c/2 (+ forget bias 0), h = tanh(c/2)/2
+    nc, nh = oracle.basic_lstm_cell(np.zeros((M, 4 * H)), c, 0.0)
+    assert np.allclose(nc, c / 2) and np.allclose(nh, np.tanh(c / 2) / 2)
+    # the gate order is i, j, f, o: a transposed split would fail this
+    one = np.zeros((1, 4)); one[0, 2] = big                    # only f saturated, H = 1
+    nc, _ = oracle.basic_lstm_cell(one, np.array([[3.0]]), 0.0)
+    assert np.allclose(nc, 3.0)

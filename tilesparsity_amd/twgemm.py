@@ -47,7 +47,7 @@ EXPORTED_SYMBOLS = (
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
-    "tw_prune_mix",
+    "tw_prune_mix", "tw_lstm_gates",
 )
 
 
@@ -140,6 +140,7 @@ def lib():
                                                   ctypes.POINTER(c_int)]),
         "tw_prune_mix": (c_int, [c_int, i32p, i32p, pp, pp, ctypes.c_double, c_int, pp,
                                  ctypes.POINTER(ctypes.c_double), vp]),
+        "tw_lstm_gates": (c_int, [c_int, c_int, c_int, vp, c_i64, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
@@ -428,6 +429,15 @@ def stream_gemm_nn(M, N, K, dtype, alpha, A_ptr, B_ptr, beta, C_ptr, N_cal, K_ca
                                    bn, _ptr(N_cal, ctypes.c_int32), _ptr(K_cal, ctypes.c_int32),
                                    mn, mk, _ptr(off_B, ctypes.c_int64), _ptr(off_C, ctypes.c_int64),
                                    ctypes.c_void_p(int(stream or 0))))
+
+
+def lstm_gates(M, H, dtype, gates_ptr, ldg, forget_bias, c_prev_ptr, ldc_prev, c_new_ptr, ldc_new,
+               h_new_ptr, ldh, stream=0):
+    """BasicLSTMCell gate arithmetic on K-major device buffers (see tw_lstm_gates)."""
+    vp = ctypes.c_void_p
+    _check(lib().tw_lstm_gates(M, H, dtype_code(dtype), vp(int(gates_ptr or 0)), ldg, forget_bias,
+                               vp(int(c_prev_ptr or 0)), ldc_prev, vp(int(c_new_ptr or 0)), ldc_new,
+                               vp(int(h_new_ptr or 0)), ldh, vp(int(stream or 0))))
 
 
 def cast_f32(src_ptr, dst_ptr, n, dtype, stream=0):

@@ -1457,8 +1457,10 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
             (int64_t)plan->n_units * ((M + kShapes[shape].bm - 1) / kShapes[shape].bm);
         if (forced >= 0 && forced < 5 && (forced == 2 || forced == 3) == narrow && (forced != 4 || ws_ok))
             shape = forced;
-        else if (big_items * 5 < 3 * (int64_t)plan->cu_count)
-            shape = narrow ? 3 : 1; // too few large items to occupy the chip
+        else if (big_items * 5 < 3 * (int64_t)plan->cu_count && (narrow || M <= 128))
+            shape = narrow ? 3 : 1; // too few large items to occupy the chip (for wide tiles the
+                                    // wave-specialised kernel still wins unless a 128-row block
+                                    // holds all of M)
     }
     const int BM = kShapes[shape].bm;
     GemmArgs a;

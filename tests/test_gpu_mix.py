@@ -126,3 +126,37 @@ def test_cover_plan_runs_mixed_masks(tw, twprune, po, oracle, dtype):
         assert np.array_equal(b1, b2)
         for a, b in zip(t1, t2):
             assert np.array_equal(a["kept_k"], b["kept_k"]) and np.array_equal(a["kept_n"], b["kept_n"])
+
+
+VGG16_LAYERS = [(27, 64), (576, 64), (576, 128), (1152, 128), (1152, 256), (2304, 256), (2304, 256),
+                (2304, 512), (4608, 512), (4608, 512), (4608, 512), (4608, 512), (4608, 512),
+                (4096, 4096)]
+
+
+def test_full_size_network_all_producers(twprune, po):
+    """A VGG16-sized list of score matrices (31.6 M elements, the 13 conv layers as im2col
+    matrices and one 4096 x 4096 dense layer): every producer returns the oracle's masks bit for
+    bit, and the kept fractions are the requested ones."""
+    rng = np.random.default_rng(20200615)
+    scores = [np.abs(rng.standard_normal(s)).astype(np.float32) for s in VGG16_LAYERS]
+    total = sum(k * n for k, n in VGG16_LAYERS)
+    print("full size: 1d", flush=True)
+    want, _, _ = po.tiled_wise_1d(scores, 75, 128)
+    got = twprune.tiled_wise_1d(scores, 75, 128)
+    assert all(np.array_equal(w, g) for w, g in zip(want, got))
+    assert abs(sum(int(g.sum()) for g in got) / total - 0.25) < 0.01
+    print("full size: 2d", flush=True)
+    want = po.tiled_wise_2d(scores, 75, 128)[0]
+    got = twprune.tiled_wise_2d(scores, 75, 128)
+    assert all(np.array_equal(w, g) for w, g in zip(want, got))
+    print("full size: 1d mix", flush=True)
+    want = po.tiled_wise_1d_mix(scores, 75, 128, 5)
+    got = twprune.tiled_wise_1d_mix(scores, 75, 128, 5)
+    assert all(np.array_equal(w, g) for w, g in zip(want, got))
+    # TW at 80 % plus the top 5 % of the shifted element scores: between 20 % and 25 % kept
+    kept = sum(int(g.sum()) for g in got) / total
+    assert 0.20 < kept <= 0.2501
+    print("full size: 2d mix", flush=True)
+    want = po.tiled_wise_2d_mix(scores, 75, 128, 1)
+    got = twprune.tiled_wise_2d_mix(scores, 75, 128, 1)
+    assert all(np.array_equal(w, g) for w, g in zip(want, got))

@@ -169,8 +169,21 @@ def bench_producers(steps, warmup, torch):
                                            ctypes.cast(d.p_masks, pp), ctypes.cast(d.p_cols, pp),
                                            thr, d.stream))
 
+    def run1dmix():
+        # tiled_wise_1d at 75 + 5 %, then the element-wise remainder (5 %) over all elements
+        tw._check(L.tw_prune_tiled_wise_1d(len(d.shapes), tw._ptr(d.K, i32), tw._ptr(d.N, i32),
+                                           ctypes.cast(d.p_scores, pp), 80.0, 0, 128,
+                                           ctypes.cast(d.p_masks, pp), None, d.stream))
+        thr = ctypes.c_double()
+        tw._check(L.tw_prune_mix(len(d.shapes), tw._ptr(d.K, i32), tw._ptr(d.N, i32),
+                                 ctypes.cast(d.p_scores, pp), ctypes.cast(d.p_masks, pp), 5.0, 0,
+                                 ctypes.cast(d.p_masks, pp), ctypes.byref(thr), d.stream))
+
     out = {}
-    for name, fn, passes in (("tiled_wise_1d", run1d, 1), ("tiled_wise_2d", run2d, 2)):
+    # bytes: scores read once per stage, one mask byte written; the mixed producer also writes and
+    # reads the 4-byte element scores, reads the TW mask and rewrites it
+    for name, fn, passes in (("tiled_wise_1d", run1d, 1), ("tiled_wise_2d", run2d, 2),
+                             ("tiled_wise_1d_mix", run1dmix, 4)):
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
@@ -194,6 +207,7 @@ def bench_producers(steps, warmup, torch):
         "config": {"workload": "mask producers, %d layers, %.1f M score elements" % (
             len(PRODUCER_LAYERS), elems / 1e6)},
         "tiled_wise_2d": out["tiled_wise_2d"],
+        "tiled_wise_1d_mix": out["tiled_wise_1d_mix"],
         "roofline": {"bound": "hbm", "achieved": one["gbs"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": one["gbs"] / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes": one["algorithmic_bytes"]},

@@ -340,3 +340,42 @@ def test_stream_gemm_nn_drop_in(tw, oracle):
         for g, t in zip(got, tiles):
             assert np.array_equal(g["kept_k"], t["kept_k"]) and np.array_equal(g["mask_n"], t["mask_n"])
         assert np.array_equal(Bs, from_device_bits(dB))
+
+
+def test_graph_capture_replays_bitwise(tw, oracle):
+    """tw_gemm allocates nothing, clears nothing from the host and re-arms its work queue inside
+    the kernel, so a sequence of launches can be captured into a HIP graph; every replay (with
+    eager launches and synchronisations in between) gives the eager result bit for bit."""
+    import torch
+    rng = np.random.default_rng(77)
+    M, K, N, G = 384, 256, 512, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.9)
+    At = np.ascontiguousarray(oracle.cast_bits(A, "f16").reshape(M, K).T)
+    dA = to_device_bits(At, At.shape)
+    dH = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+    dC = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+    s = torch.cuda.Stream()
+    with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+        def chain():
+            # two dependent launches: C = A (B.mask), then C += 0.5 * A (B.mask) on top of it
+            plan.gemm(dA.data_ptr(), dH.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO, stream=s.cuda_stream)
+            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=0.5, beta=0.0, pruned_cols=tw.PRUNED_ZERO,
+                      stream=s.cuda_stream)
+            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=1.0, beta=1.0, stream=s.cuda_stream)
+        with torch.cuda.stream(s):
+            chain()
+            s.synchronize()
+            want_h, want_c = dH.clone(), dC.clone()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=s):
+                chain()
+            for rep in range(4):
+                dH.fill_(0x1234)
+                dC.fill_(0x1234)
+                plan.gemm(dA.data_ptr(), dH.data_ptr(), M, stream=s.cuda_stream)   # eager work between replays
+                s.synchronize()
+                g.replay()
+                s.synchronize()
+                assert torch.equal(dH, want_h) and torch.equal(dC, want_c), rep

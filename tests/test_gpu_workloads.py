@@ -96,3 +96,21 @@ def test_config5_imbalance_stress(tw, oracle):
     kts = [len(t["kept_k"]) for t in wl["tiles"]]
     assert kts.count(0) >= 13 and max(kts) > 2500      # empty tiles and near-dense tiles
     check_workload(tw, oracle, wl)
+
+
+def test_cpp_driver_reference_command_line():
+    """The C++ perf driver with the reference's command line (`./test_basic_nn M N K N_kept K_kept`,
+    StreamMaskedGEMM/README.md:12-13) at a reduced M: its three self-checks (fused == gather /
+    dense / scatter bit for bit, fused vs a host fp32 product, dense baseline vs fused) pass."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                       "tilesparsity_amd", "test_basic_nn")
+    assert os.path.exists(exe), "build the driver with `python -m tilesparsity_amd.build`"
+    for args in (["1280", "768", "768", "384", "384"], ["520", "768", "3072", "384", "1536"]):
+        print("driver", args, flush=True)
+        res = subprocess.run([exe] + args, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                             timeout=100)
+        assert res.returncode == 0, res.stdout[-2000:]
+        assert res.stdout.count("PASSED !!!") == 3 and "FAILED" not in res.stdout, res.stdout[-2000:]
+        assert "Stream  GEMM :" in res.stdout and "Dense   GEMM :" in res.stdout

@@ -157,3 +157,31 @@ def test_tiles_from_mask_accepts_any_mask(tw):
         got = tw.tiles_from_mask(mask, 32)
         assert got == po.tiles_from_mask(mask, 32)
         check_table(mask, got, 32)
+
+
+# --------------------------------------------------------------------------------------
+# host logic of the producer mirror (no GPU call)
+# --------------------------------------------------------------------------------------
+def test_percentile_type_follows_the_type_of_q():
+    """np.percentile keeps float32 arithmetic for a Python number and switches to float64 for a
+    NumPy float64; the mirror passes that choice to the library."""
+    from tilesparsity_amd import twprune
+    assert twprune._q_type(75) == twprune.Q_F32 and twprune._q_type(75.0) == twprune.Q_F32
+    assert twprune._q_type(np.float64(75)) == twprune.Q_F64
+    assert twprune._q_type(np.float32(75)) == twprune.Q_F32
+    assert twprune._q_type(100 - np.sqrt(10000 - 75 * 100)) == twprune.Q_F64   # tiled_wise_2d's own
+    assert twprune._q_type(100 - 5) == twprune.Q_F32 and twprune._q_type(75 + np.float64(5)) == twprune.Q_F64
+    # and NumPy really behaves that way (the reason the switch exists)
+    v = np.random.default_rng(3).random(1001).astype(np.float32)
+    assert np.percentile(v, 33.3).dtype == np.float32 and np.percentile(v, np.float64(33.3)).dtype == np.float64
+
+
+def test_img2col_forward_shapes_and_sign():
+    from tilesparsity_amd import twprune
+    rng = np.random.default_rng(4)
+    conv, dense = rng.standard_normal((3, 3, 8, 16)).astype(np.float32), rng.standard_normal((5, 7)).astype(np.float32)
+    out = twprune.img2col_forward([conv, dense])
+    assert out[0].shape == (72, 16) and out[1].shape == (5, 7)
+    assert np.array_equal(out[0], po.img2col(conv)) and np.array_equal(out[1], np.abs(dense))
+    # HWIO -> (H*W*I) x O keeps the output channel as the column
+    assert np.array_equal(out[0][:, 3], np.abs(conv[..., 3]).ravel())

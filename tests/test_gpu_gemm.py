@@ -379,3 +379,26 @@ def test_graph_capture_replays_bitwise(tw, oracle):
                 g.replay()
                 s.synchronize()
                 assert torch.equal(dH, want_h) and torch.equal(dC, want_c), rep
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_every_kernel_shape_agrees(tw, oracle, dtype, monkeypatch):
+    """The launch picks one of five kernel shapes from the plan and M; TWGEMM_SHAPE forces each of
+    them in turn (wide tiles: 256x128, 128x128, wave-specialised 256x128; narrow tiles: 512x64,
+    256x64): all match the oracle, and each shape repeats itself bit for bit."""
+    rng = np.random.default_rng(88)
+    for (M, K, N, G, shapes) in ((600, 320, 384, 128, (0, 1, 4)), (1100, 200, 256, 64, (2, 3))):
+        A = rng.standard_normal((M, K)).astype(np.float32)
+        B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+        tiles = random_tiles(rng, K, N, G, k_keep=0.45, n_keep=0.85)
+        ref = reference(oracle, A, B, tiles, dtype)
+        keep = kept_columns(tiles, N)
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            for shape in shapes:
+                monkeypatch.setenv("TWGEMM_SHAPE", str(shape))
+                print("shape", shape, M, K, N, G, dtype, flush=True)
+                C1, bits1 = run_gemm(tw, oracle, plan, A, dtype, N)
+                C2, bits2 = run_gemm(tw, oracle, plan, A, dtype, N)
+                assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL[dtype], shape
+                assert np.array_equal(bits1, bits2), shape
+        monkeypatch.delenv("TWGEMM_SHAPE", raising=False)

@@ -402,3 +402,33 @@ def test_every_kernel_shape_agrees(tw, oracle, dtype, monkeypatch):
                 assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL[dtype], shape
                 assert np.array_equal(bits1, bits2), shape
         monkeypatch.delenv("TWGEMM_SHAPE", raising=False)
+
+
+def test_operand_beyond_four_gib(tw, oracle):
+    """A of 4.4 GiB: byte offsets into A no longer fit 32 bits, the launch falls back to the
+    kernel with 64-bit addressing.  Checked on sampled rows (a row of C depends on the same row
+    of A only) at both ends of M."""
+    import torch
+    K, N, G = 2304, 128, 128
+    M = 1024 * 1000                        # K * M * 2 bytes = 4.4 GiB
+    rng = np.random.default_rng(99)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.25, n_keep=0.9)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    dA = torch.empty((K, M), dtype=torch.float16, device="cuda")
+    for k0 in range(0, K, 256):            # filled in slabs: no 2x temporary
+        dA[k0:k0 + 256].normal_(generator=g)
+    dC = torch.full((N, M), 7.0, dtype=torch.float16, device="cuda")
+    print("4 GiB operand: launch", flush=True)
+    with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+        plan.gemm(dA.data_ptr(), dC.data_ptr(), M, stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+    rows = np.concatenate([np.arange(0, 40), rng.integers(0, M, 60), np.arange(M - 40, M)])
+    idx = torch.from_numpy(rows).cuda()
+    A_rows = dA[:, idx].float().cpu().numpy().T          # [rows, K], exact fp16 values
+    C_rows = dC[:, idx].float().cpu().numpy().T
+    ref = oracle.tw_gemm_reference(A_rows, oracle.quantize(B, "f16"), tiles)
+    keep = kept_columns(tiles, N)
+    assert oracle.rel_error(C_rows[:, keep], ref[:, keep]) <= 1e-2
+    assert np.all(C_rows[:, ~keep] == 7.0)               # pruned columns untouched

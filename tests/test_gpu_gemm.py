@@ -432,3 +432,43 @@ def test_operand_beyond_four_gib(tw, oracle):
     keep = kept_columns(tiles, N)
     assert oracle.rel_error(C_rows[:, keep], ref[:, keep]) <= 1e-2
     assert np.all(C_rows[:, ~keep] == 7.0)               # pruned columns untouched
+
+
+def test_concurrent_host_threads_and_streams(tw, oracle):
+    """One immutable plan, four host threads, each launching on its own stream into its own C:
+    every thread gets the single-stream result bit for bit."""
+    import threading
+    import torch
+    rng = np.random.default_rng(111)
+    M, K, N, G = 1024, 384, 512, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.9)
+    At = np.ascontiguousarray(oracle.cast_bits(A, "f16").reshape(M, K).T)
+    dA = to_device_bits(At, At.shape)
+    with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+        want = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+        plan.gemm(dA.data_ptr(), want.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
+                  stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        outs = [torch.full((N, M), 0x1234, dtype=torch.int16, device="cuda") for _ in range(4)]
+        streams = [torch.cuda.Stream() for _ in range(4)]
+        errors = []
+
+        def work(i):
+            try:
+                for _ in range(60):
+                    plan.gemm(dA.data_ptr(), outs[i].data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
+                              stream=streams[i].cuda_stream)
+                streams[i].synchronize()
+            except Exception as e:           # surfaced by the main thread
+                errors.append(e)
+
+        threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+        for t in threads:
+            t.start()
+        for t in threads:
+            t.join()
+        assert not errors, errors
+        for o in outs:
+            assert torch.equal(o, want)

@@ -135,6 +135,46 @@ def cpu_baseline(wl, A, B, budget_s=20.0):
                        % (rows, M, len(times), t))
 
 
+def bench_prepass(wl, steps, warmup):
+    """The integer pre-pass behind tw_plan_from_mask on the workload's mask: host mask and fp32
+    weight in, device plan out (upload, row / column flags, tile-wise check, compaction of the
+    kept lists and relative offsets, weight packing and cast).  A step is one plan build; the
+    CPU baseline is the oracle's NumPy restatement of the same pre-pass."""
+    from tilesparsity_amd import twgemm as tw
+    from oracle import tw_oracle
+    K, N, G, tiles = wl["K"], wl["N"], wl["G"], wl["tiles"]
+    _, B = wl["values"]()
+    mask = tw_oracle.plan_mask(K, N, tiles).astype(np.uint8)
+    for _ in range(warmup):
+        tw.Plan.from_mask(mask, G, wl["dtype"], B).destroy()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tw.Plan.from_mask(mask, G, wl["dtype"], B).destroy()
+    t = (time.perf_counter() - t0) / steps
+    with tw.Plan.from_mask(mask, G, wl["dtype"], B) as plan:
+        info = plan.info()
+    # bytes the device must move: the mask is read three times (row flags, column flags, check),
+    # the fp32 weight once at the kept positions, the packed 16-bit weight is written once
+    by = 3 * K * N + 4 * info["kept_elems"] + info["packed_bytes"]
+    t1 = time.perf_counter()
+    got = tw_oracle.plan_from_mask(mask, G)
+    tw_oracle.cast_bits(tw_oracle.stream_weight(B, got), wl["dtype"])
+    t_cpu = time.perf_counter() - t1
+    return {
+        "metric": "TW pre-pass: plan builds per second (mask -> lists -> offsets -> packed weight)",
+        "value": 1.0 / t, "unit": "plans/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": t * 1e3, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "u8", "data": "synthetic",
+        "config": {"workload": "%s mask %d x %d, G=%d, %d tiles" % (wl["name"], K, N, G, len(tiles))},
+        "host_to_plan_ms": t * 1e3, "uploaded_bytes": K * N * 5,
+        "roofline": {"bound": "hbm", "achieved": by / t / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": by / t / 1e9 / HBM_PEAK_GBS, "traffic": None, "algorithmic_bytes": by},
+        "cpu_baseline": {"value": 1.0 / t_cpu, "unit": "plans/s", "cores": 1, "kind": "port",
+                         "sample": "NumPy oracle: lists from the mask, compacted weight and cast, "
+                                   "one run (%.1f ms)" % (t_cpu * 1e3)},
+    }
+
+
 # VGG16's 13 conv layers as im2col score matrices (H*W*I) x O, plus a 4096 x 4096 dense layer
 PRODUCER_LAYERS = [(27, 64), (576, 64), (576, 128), (1152, 128), (1152, 256), (2304, 256),
                    (2304, 256), (2304, 512), (4608, 512), (4608, 512), (4608, 512), (4608, 512),
@@ -229,6 +269,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--producers", action="store_true",
                     help="benchmark the TW mask producers instead of the GEMM (one JSON line)")
+    ap.add_argument("--prepass", action="store_true",
+                    help="time the mask -> kept lists -> offsets -> compaction pre-pass instead")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (4 launches over rotating buffers), "
                          "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
@@ -246,6 +288,10 @@ def main():
     tw.lib()  # fails loudly if the HIP library has not been built
     if args.producers:
         print(json.dumps(bench_producers(min(args.steps, 20), min(args.warmup, 3), torch)), flush=True)
+        return 0
+    if args.prepass:
+        print(json.dumps(bench_prepass(make_workload(args.workload), min(args.steps, 20),
+                                       min(args.warmup, 3))), flush=True)
         return 0
 
     if args.copy_calibration:

@@ -110,3 +110,41 @@ def test_delete_insert_row_kernels(tw):
     expect = np.zeros_like(src)
     expect[kept] = src[kept]
     assert np.array_equal(from_device_bits(d_back), expect)
+
+
+def test_device_operands_give_the_same_plan(tw, oracle):
+    """tw_plan_from_device_mask on device copies of the mask and the weight builds the plan the
+    host entry points build: same lists, same packed weight bits; also for covering plans and
+    for the masks a producer leaves on the device."""
+    import torch
+    from oracle import tw_prune_oracle as po
+    from tilesparsity_amd import twprune
+    rng = np.random.default_rng(17)
+    for K, N, G in ((192, 320, 64), (300, 200, 128), (64, 64, 16)):
+        W = rng.standard_normal((K, N)).astype(np.float32)
+        scores = twprune.img2col_forward([W])
+        dW = torch.from_numpy(W).cuda()
+        table = po.tiles_every_g_columns(N, G)
+        # a producer's device mask goes straight into the plan
+        dmask = twprune.tiled_wise_1d(scores, 70, G, return_device=True)[0]
+        print("device pre-pass", K, N, G, flush=True)
+        with tw.Plan.from_device_mask(K, N, dmask.data_ptr(), table, "f16", dW.data_ptr()) as pd, \
+                tw.Plan.from_mask_tiles(dmask.cpu().numpy(), table, "f16", W) as ph:
+            (td, bd), (th, bh) = pd.export(), ph.export()
+            assert np.array_equal(bd, bh)
+            for a, b in zip(td, th):
+                assert np.array_equal(a["kept_k"], b["kept_k"]) and np.array_equal(a["kept_n"], b["kept_n"])
+                assert np.array_equal(a["mask_k"], b["mask_k"]) and np.array_equal(a["mask_n"], b["mask_n"])
+        # an arbitrary mask: refused without cover, identical to the host path with it
+        m = (rng.random((K, N)) < 0.1).astype(np.uint8)
+        dm = torch.from_numpy(m).cuda()
+        with pytest.raises(tw.TwError) as e:
+            tw.Plan.from_device_mask(K, N, dm.data_ptr(), table, "bf16", dW.data_ptr())
+        assert e.value.status == tw.ERR_NOT_TW
+        with tw.Plan.from_device_mask(K, N, dm.data_ptr(), table, "bf16", dW.data_ptr(), cover=True) as pd, \
+                tw.Plan.from_mask_tiles(m, table, "bf16", W, cover=True) as ph:
+            (td, bd), (th, bh) = pd.export(), ph.export()
+            assert np.array_equal(bd, bh)
+            assert np.array_equal(bd, oracle.cast_bits(oracle.stream_weight(np.where(m != 0, W, np.float32(0)), po.cover_tiles_from_mask(m, table)), "bf16"))
+    with pytest.raises(tw.TwError):
+        tw.Plan.from_device_mask(8, 8, 0, [(0, 8)], "f16", 0)

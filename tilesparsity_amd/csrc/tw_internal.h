@@ -119,7 +119,7 @@ int validate_lists(int K, int N, int n_tiles, const int32_t *tile_col0, const in
 int finalize_plan_geometry(tw_plan *p);
 
 // device pack: packed weight from a row-major fp32 [K,N] device buffer
-int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s);
+int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s, const uint8_t *d_mask = nullptr);
 // device pack: packed weight from the reference's compacted stream layout (16-bit, device)
 int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStream_t s);
 // device unpack: compacted stream layout (K*N 16-bit, zero elsewhere) from the packed weight

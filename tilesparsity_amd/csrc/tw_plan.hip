@@ -47,9 +47,11 @@ __device__ __forceinline__ uint16_t cast16(float f, int dtype)
 // ---------------------------------------------------------------------------------
 // packing
 
+// `mask` (optional, K x N bytes): elements whose mask byte is zero are stored as zeros (covering
+// plans of masks that are not rows x columns per tile)
 __global__ void pack_dense_kernel(const PackTile *tiles, const int32_t *kept_k,
                                   const int32_t *kept_n, const float *B, int N, int dtype,
-                                  uint16_t *Bp)
+                                  uint16_t *Bp, const uint8_t *mask)
 {
     const PackTile t = tiles[blockIdx.y];
     const int64_t groups = (int64_t)t.k_pad * t.n_pad / 8;
@@ -72,8 +74,11 @@ __global__ void pack_dense_kernel(const PackTile *tiles, const int32_t *kept_k,
     for (int e = 0; e < 8; ++e) {
         const int kk = kk0 + e;
         float f = 0.0f;
-        if (col >= 0 && kk < t.k_kept)
-            f = B[(int64_t)kept_k[t.kk_off + kk] * N + col];
+        if (col >= 0 && kk < t.k_kept) {
+            const int64_t src = (int64_t)kept_k[t.kk_off + kk] * N + col;
+            if (!mask || mask[src])
+                f = B[src];
+        }
         v[e] = cast16(f, dtype);
     }
     uint4 out;
@@ -419,14 +424,25 @@ int finalize_plan_geometry(tw_plan *p)
     if (hipMalloc((void **)&p->d_tickets, sizeof(int32_t) * 2 * kTicketSlots + 2048) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of the ticket slots failed");
     TW_HIP(hipMemset(p->d_tickets, 0, sizeof(int32_t) * 2 * kTicketSlots + 2048));
-    hipDeviceProp_t prop;
     TW_HIP(hipGetDevice(&p->device));
-    TW_HIP(hipGetDeviceProperties(&prop, p->device));
-    p->cu_count = prop.multiProcessorCount;
+    {
+        // the CU count of a device does not change: ask once per device
+        static std::mutex mu;
+        static std::vector<int> cu_of;
+        std::lock_guard<std::mutex> lock(mu);
+        if ((int)cu_of.size() <= p->device)
+            cu_of.resize(p->device + 1, 0);
+        if (cu_of[p->device] == 0) {
+            int n = 0;
+            TW_HIP(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, p->device));
+            cu_of[p->device] = n;
+        }
+        p->cu_count = cu_of[p->device];
+    }
     return TW_OK;
 }
 
-int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s)
+int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s, const uint8_t *d_mask)
 {
     const int64_t mg = max_groups(p);
     if (mg == 0)
@@ -438,7 +454,7 @@ int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s)
         return st;
     dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
     hipLaunchKernelGGL(pack_dense_kernel, grid, dim3(256), 0, s, d_pt, p->d_kept_k, p->d_kept_n,
-                       d_B, p->N, p->dtype, (uint16_t *)p->d_Bp);
+                       d_B, p->N, p->dtype, (uint16_t *)p->d_Bp, d_mask);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
         e = hipStreamSynchronize(s);
@@ -621,9 +637,11 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     return tw_plan_from_mask_tiles(K, N, dtype, nt, col0.data(), width.data(), mask, B, out);
 }
 
-static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
-                               const int32_t *tile_width, const uint8_t *mask, const float *B,
-                               bool cover, tw_plan **out)
+// The pre-pass on device operands: d_mask is K x N bytes, d_B the fp32 weight, both row-major in
+// device memory.  Temporaries (flags, counters, the tile table) share one allocation.
+static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                                 const int32_t *tile_width, const uint8_t *d_mask, const float *d_B,
+                                 bool cover, tw_plan **out)
 {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
@@ -633,7 +651,7 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
         return st;
     if (K <= 0 || N <= 0 || n_tiles <= 0)
         return fail(TW_ERR_SHAPE, "K=%d N=%d n_tiles=%d must all be positive", K, N, n_tiles);
-    if (!mask || !B || !tile_col0 || !tile_width)
+    if (!d_mask || !d_B || !tile_col0 || !tile_width)
         return fail(TW_ERR_NULL, "mask, B or the tile table is NULL");
     const int nt = n_tiles;
     std::vector<int32_t> tcol0(nt + 1);
@@ -652,21 +670,19 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
         tcol0[nt] = N;
     }
 
-    uint8_t *d_mask = nullptr, *d_rowflag = nullptr;
-    uint32_t *d_colflag = nullptr;
-    unsigned long long *d_mismatch = nullptr;
-    int32_t *d_counts = nullptr, *d_kptr = nullptr, *d_nptr = nullptr, *d_tcol0 = nullptr;
+    // one allocation for all temporaries, carved at 256-byte boundaries
+    auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+    const size_t o_rowflag = 0;
+    const size_t o_colflag = o_rowflag + up((size_t)nt * K);
+    const size_t o_mismatch = o_colflag + up(sizeof(uint32_t) * N);
+    const size_t o_counts = o_mismatch + up(sizeof(unsigned long long));
+    const size_t o_tcol0 = o_counts + up(sizeof(int32_t) * 2 * nt);
+    const size_t o_kptr = o_tcol0 + up(sizeof(int32_t) * (nt + 1));
+    const size_t o_nptr = o_kptr + up(sizeof(int32_t) * (nt + 1));
+    const size_t ws_bytes = o_nptr + up(sizeof(int32_t) * (nt + 1));
+    char *ws = nullptr;
     tw_plan *p = nullptr;
-    auto cleanup = [&]() {
-        hipFree(d_tcol0);
-        hipFree(d_mask);
-        hipFree(d_rowflag);
-        hipFree(d_colflag);
-        hipFree(d_mismatch);
-        hipFree(d_counts);
-        hipFree(d_kptr);
-        hipFree(d_nptr);
-    };
+    auto cleanup = [&]() { hipFree(ws); };
 #define TW_TRY(call)                                                                       \
     do {                                                                                   \
         hipError_t e_ = (call);                                                            \
@@ -677,17 +693,17 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
         }                                                                                  \
     } while (0)
 
-    const size_t mask_bytes = (size_t)K * N;
-    TW_TRY(hipMalloc((void **)&d_mask, mask_bytes));
-    TW_TRY(hipMalloc((void **)&d_rowflag, (size_t)nt * K));
-    TW_TRY(hipMalloc((void **)&d_colflag, sizeof(uint32_t) * N));
-    TW_TRY(hipMalloc((void **)&d_mismatch, sizeof(unsigned long long)));
-    TW_TRY(hipMalloc((void **)&d_counts, sizeof(int32_t) * 2 * nt));
-    TW_TRY(hipMalloc((void **)&d_tcol0, sizeof(int32_t) * (nt + 1)));
+    TW_TRY(hipMalloc((void **)&ws, ws_bytes));
+    uint8_t *d_rowflag = reinterpret_cast<uint8_t *>(ws + o_rowflag);
+    uint32_t *d_colflag = reinterpret_cast<uint32_t *>(ws + o_colflag);
+    unsigned long long *d_mismatch = reinterpret_cast<unsigned long long *>(ws + o_mismatch);
+    int32_t *d_counts = reinterpret_cast<int32_t *>(ws + o_counts);
+    int32_t *d_tcol0 = reinterpret_cast<int32_t *>(ws + o_tcol0);
+    int32_t *d_kptr = reinterpret_cast<int32_t *>(ws + o_kptr);
+    int32_t *d_nptr = reinterpret_cast<int32_t *>(ws + o_nptr);
     TW_TRY(hipMemcpy(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
-    TW_TRY(hipMemcpy(d_mask, mask, mask_bytes, hipMemcpyHostToDevice));
-    TW_TRY(hipMemset(d_colflag, 0, sizeof(uint32_t) * N));
-    TW_TRY(hipMemset(d_mismatch, 0, sizeof(unsigned long long)));
+    // column flags and the mismatch counter start at zero (they are adjacent in the workspace)
+    TW_TRY(hipMemset(d_colflag, 0, o_counts - o_colflag));
 
     {
         const int64_t n_rt = (int64_t)K * nt;
@@ -702,10 +718,12 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
                            d_colflag, K, d_tcol0, nt, d_counts);
         TW_TRY(hipGetLastError());
     }
+    // mismatch counter and the 2 * nt counts come back with one copy (they are adjacent)
+    std::vector<char> back(o_tcol0 - o_mismatch);
+    TW_TRY(hipMemcpy(back.data(), ws + o_mismatch, back.size(), hipMemcpyDeviceToHost));
     unsigned long long mismatch = 0;
-    std::vector<int32_t> counts(2 * nt);
-    TW_TRY(hipMemcpy(&mismatch, d_mismatch, sizeof(mismatch), hipMemcpyDeviceToHost));
-    TW_TRY(hipMemcpy(counts.data(), d_counts, sizeof(int32_t) * 2 * nt, hipMemcpyDeviceToHost));
+    std::memcpy(&mismatch, back.data(), sizeof(mismatch));
+    const int32_t *counts = reinterpret_cast<const int32_t *>(back.data() + (o_counts - o_mismatch));
     if (mismatch != 0 && !cover) {
         cleanup();
         return fail(TW_ERR_NOT_TW,
@@ -733,8 +751,6 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
         p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + counts[nt + t];
     }
     const size_t sk = std::max(p->kept_k_ptr[nt], 1), sn = std::max(p->kept_n_ptr[nt], 1);
-    TW_TRY(hipMalloc((void **)&d_kptr, sizeof(int32_t) * (nt + 1)));
-    TW_TRY(hipMalloc((void **)&d_nptr, sizeof(int32_t) * (nt + 1)));
     TW_TRY(hipMemcpy(d_kptr, p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
     TW_TRY(hipMemcpy(d_nptr, p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
     TW_TRY(hipMalloc((void **)&p->d_kept_k, sizeof(int32_t) * sk));
@@ -759,22 +775,55 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
                         p->kept_k_idx.data(), p->kept_n_ptr.data(), p->kept_n_idx.data());
     if (!st)
         st = finalize_plan_geometry(p);
-    if (!st && cover && mismatch != 0) {
-        // rows and columns of a tile are the union of its elements: the elements the mask
-        // drops inside that cover are stored as zeros
-        std::vector<float> Bm((size_t)K * N);
-        for (size_t i = 0; i < Bm.size(); ++i)
-            Bm[i] = mask[i] ? B[i] : 0.0f;
-        st = pack_host_weight(p, Bm.data());
-    } else if (!st) {
-        st = pack_host_weight(p, B);
-    }
+    // rows and columns of a covering tile are the union of its elements: the elements the mask
+    // drops inside that cover are stored as zeros
+    if (!st && p->packed_elems > 0)
+        st = pack_from_dense(p, d_B, nullptr, cover && mismatch != 0 ? d_mask : nullptr);
     if (st) {
         free_plan(p);
         return st;
     }
     *out = p;
     return TW_OK;
+}
+
+// host operands: one upload buffer for the mask and the weight, then the device pre-pass
+static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                               const int32_t *tile_width, const uint8_t *mask, const float *B,
+                               bool cover, tw_plan **out)
+{
+    if (!out)
+        return fail(TW_ERR_NULL, "out is NULL");
+    *out = nullptr;
+    if (int st = check_dtype(dtype))
+        return st;
+    if (K <= 0 || N <= 0 || n_tiles <= 0)
+        return fail(TW_ERR_SHAPE, "K=%d N=%d n_tiles=%d must all be positive", K, N, n_tiles);
+    if (!mask || !B || !tile_col0 || !tile_width)
+        return fail(TW_ERR_NULL, "mask, B or the tile table is NULL");
+    const size_t b_bytes = (size_t)K * N * sizeof(float), m_bytes = (size_t)K * N;
+    char *buf = nullptr;
+    if (hipMalloc((void **)&buf, b_bytes + m_bytes) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the mask and weight upload failed",
+                    b_bytes + m_bytes);
+    hipError_t e = hipMemcpy(buf, B, b_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess)
+        e = hipMemcpy(buf + b_bytes, mask, m_bytes, hipMemcpyHostToDevice);
+    int st = e == hipSuccess
+                 ? plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width,
+                                         reinterpret_cast<const uint8_t *>(buf + b_bytes),
+                                         reinterpret_cast<const float *>(buf), cover, out)
+                 : fail(TW_ERR_DEVICE, "mask / weight upload failed: %s", hipGetErrorString(e));
+    hipFree(buf);
+    return st;
+}
+
+int tw_plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
+                             const int32_t *tile_width, const uint8_t *mask, const float *B,
+                             int cover, tw_plan **out)
+{
+    return plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, cover != 0,
+                                 out);
 }
 
 int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,

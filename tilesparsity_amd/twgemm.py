@@ -47,7 +47,7 @@ EXPORTED_SYMBOLS = (
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
-    "tw_prune_mix", "tw_lstm_gates",
+    "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask",
 )
 
 
@@ -141,6 +141,7 @@ def lib():
         "tw_prune_mix": (c_int, [c_int, i32p, i32p, pp, pp, ctypes.c_double, c_int, pp,
                                  ctypes.POINTER(ctypes.c_double), vp]),
         "tw_lstm_gates": (c_int, [c_int, c_int, c_int, vp, c_i64, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
+        "tw_plan_from_device_mask": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, vp, vp, c_int, pp]),
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
@@ -312,6 +313,20 @@ class Plan:
         _check(fn(K, N, dtype_code(dtype), len(tile_table), _ptr(col0, ctypes.c_int32),
                   _ptr(width, ctypes.c_int32), _ptr(mask, ctypes.c_uint8), _ptr(B, ctypes.c_float),
                   ctypes.byref(h)))
+        return cls(h.value, K, N, dtype_code(dtype))
+
+    @classmethod
+    def from_device_mask(cls, K, N, mask_ptr, tile_table, dtype, B_ptr, cover=False):
+        """As from_mask_tiles, with the mask (K x N bytes) and the fp32 weight in device memory
+        (raw pointers): nothing is uploaded."""
+        col0 = _i32([t[0] for t in tile_table])
+        width = _i32([t[1] for t in tile_table])
+        h = ctypes.c_void_p()
+        _check(lib().tw_plan_from_device_mask(K, N, dtype_code(dtype), len(tile_table),
+                                              _ptr(col0, ctypes.c_int32), _ptr(width, ctypes.c_int32),
+                                              ctypes.c_void_p(int(mask_ptr or 0)),
+                                              ctypes.c_void_p(int(B_ptr or 0)), 1 if cover else 0,
+                                              ctypes.byref(h)))
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod

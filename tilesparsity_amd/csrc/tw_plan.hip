@@ -151,66 +151,146 @@ __global__ void unpack_stream_kernel(const PackTile *tiles, const uint16_t *Bp, 
 
 // The tile table on the device: tcol0[t] is the first column of tile t, tcol0[n_tiles] == N.
 
-// rowflag[t*K + k] = any byte of mask[k][tcol0[t] .. tcol0[t+1]) is non-zero
-__global__ void row_flags_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0,
-                                 int n_tiles, uint8_t *rowflag)
-{
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)K * n_tiles)
-        return;
-    const int t = (int)(idx % n_tiles);
-    const int k = (int)(idx / n_tiles);
-    const int c0 = tcol0[t];
-    const int w = tcol0[t + 1] - c0;
-    const uint8_t *row = mask + (int64_t)k * N + c0;
-    uint32_t any = 0;
-    for (int j = 0; j < w; ++j)
-        any |= row[j];
-    rowflag[(int64_t)t * K + k] = any ? 1 : 0;
-}
+// Both flag kernels walk the mask in 16-byte column chunks: thread (slice, chunk) of a block
+// handles chunk `chunk` of the rows slice, slice + 256/cw, ... of a 64-row slab, so that the cw
+// lanes next to each other read cw * 16 contiguous bytes of one row.  A chunk usually lies inside
+// one tile; chunks that straddle a tile boundary, ragged ends and unaligned masks take the
+// byte-wise path.
 
-// colflag[c] |= any of mask[k][c] over a 64-row slab (colflag holds 32-bit words)
-__global__ void col_flags_kernel(const uint8_t *mask, int K, int N, uint32_t *colflag)
-{
-    const int c = blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= N)
-        return;
-    const int k0 = blockIdx.y * 64;
-    const int k1 = min(K, k0 + 64);
-    uint32_t any = 0;
-    for (int k = k0; k < k1; ++k)
-        any |= mask[(int64_t)k * N + c];
-    if (any)
-        atomicOr(&colflag[c], 1u);
-}
+struct ChunkPos {
+    int c0, w;       // first column and width (1..16) of the chunk
+    int t0;          // tile of the chunk's first column
+    bool one_tile;   // the whole chunk lies in tile t0
+    bool vec;        // 16-byte loads are possible
+    int k_begin, k_end, k_step;
+};
 
-// counts the elements where mask != rowflag & colflag (a TW mask has none)
-__global__ void validate_tw_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0,
-                                   int n_tiles, const uint8_t *rowflag, const uint32_t *colflag,
-                                   unsigned long long *mismatch)
+__device__ __forceinline__ bool chunk_pos(const uint8_t *mask, int K, int N, const int32_t *tcol0,
+                                          int n_tiles, int cw, ChunkPos &q)
 {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (int64_t)K * N)
-        return;
-    const int c = (int)(idx % N);
-    const int k = (int)(idx / N);
-    int lo = 0, hi = n_tiles; // the tile with tcol0[t] <= c < tcol0[t+1]
+    const int nchunk = (N + 15) >> 4;
+    const int chunk = blockIdx.x * cw + (int)(threadIdx.x % cw);
+    if (chunk >= nchunk)
+        return false;
+    q.c0 = chunk << 4;
+    q.w = min(16, N - q.c0);
+    int lo = 0, hi = n_tiles; // the tile with tcol0[t] <= c0 < tcol0[t+1]
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
-        if (tcol0[mid] <= c)
+        if (tcol0[mid] <= q.c0)
             lo = mid;
         else
             hi = mid;
     }
-    const int t = lo;
-    const bool m = mask[idx] != 0;
-    const bool e = rowflag[(int64_t)t * K + k] && colflag[c];
-    if (m != e)
-        atomicAdd(mismatch, 1ull);
+    q.t0 = lo;
+    q.one_tile = tcol0[lo + 1] >= q.c0 + q.w;
+    q.vec = q.w == 16 && (N & 15) == 0 && ((uintptr_t)mask & 15) == 0;
+    q.k_step = 256 / cw;
+    q.k_begin = blockIdx.y * 64 + (int)(threadIdx.x / cw);
+    q.k_end = min(K, (int)blockIdx.y * 64 + 64);
+    return true;
+}
+
+// the chunk's bytes as four words, byte j of the chunk in bits 8*(j%4) of word j/4; 0 beyond w
+__device__ __forceinline__ void load_chunk(const uint8_t *src, const ChunkPos &q, uint32_t (&v)[4])
+{
+    if (q.vec) {
+        const uint4 x = *reinterpret_cast<const uint4 *>(src);
+        v[0] = x.x;
+        v[1] = x.y;
+        v[2] = x.z;
+        v[3] = x.w;
+    } else {
+        v[0] = v[1] = v[2] = v[3] = 0u;
+        for (int j = 0; j < q.w; ++j)
+            v[j >> 2] |= (uint32_t)src[j] << ((j & 3) * 8);
+    }
+}
+
+__device__ __forceinline__ uint32_t chunk_byte(const uint32_t (&v)[4], int j)
+{
+    return (v[j >> 2] >> ((j & 3) * 8)) & 0xFFu;
+}
+
+// rowflag[t*K + k] = 1 where any byte of mask[k][tcol0[t] .. tcol0[t+1]) is non-zero,
+// colflag[c] = 1 where any byte of column c is; both arrays start zeroed and only receive ones.
+__global__ void __launch_bounds__(256)
+    mask_flags_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0, int n_tiles, int cw,
+                      uint8_t *rowflag, uint8_t *colflag)
+{
+    ChunkPos q;
+    if (!chunk_pos(mask, K, N, tcol0, n_tiles, cw, q))
+        return;
+    uint32_t acc[4] = {0u, 0u, 0u, 0u};
+    for (int k = q.k_begin; k < q.k_end; k += q.k_step) {
+        uint32_t v[4];
+        load_chunk(mask + (int64_t)k * N + q.c0, q, v);
+        if (q.one_tile) {
+            if (v[0] | v[1] | v[2] | v[3])
+                rowflag[(int64_t)q.t0 * K + k] = 1;
+        } else {
+            int t = q.t0, t_end = tcol0[t + 1];
+            uint32_t any = 0;
+            for (int j = 0; j < q.w; ++j) {
+                if (q.c0 + j >= t_end) {
+                    if (any)
+                        rowflag[(int64_t)t * K + k] = 1;
+                    any = 0;
+                    ++t;
+                    t_end = tcol0[t + 1];
+                }
+                any |= chunk_byte(v, j);
+            }
+            if (any)
+                rowflag[(int64_t)t * K + k] = 1;
+        }
+        acc[0] |= v[0];
+        acc[1] |= v[1];
+        acc[2] |= v[2];
+        acc[3] |= v[3];
+    }
+    for (int j = 0; j < q.w; ++j)
+        if (chunk_byte(acc, j))
+            colflag[q.c0 + j] = 1;
+}
+
+// counts the elements where mask != rowflag & colflag (a TW mask has none)
+__global__ void __launch_bounds__(256)
+    validate_tw_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0, int n_tiles, int cw,
+                       const uint8_t *rowflag, const uint8_t *colflag, unsigned long long *mismatch)
+{
+    ChunkPos q;
+    unsigned bad = 0;
+    if (chunk_pos(mask, K, N, tcol0, n_tiles, cw, q)) {
+        uint32_t cf = 0; // bit j: column c0 + j is kept
+        for (int j = 0; j < q.w; ++j)
+            cf |= (colflag[q.c0 + j] ? 1u : 0u) << j;
+        for (int k = q.k_begin; k < q.k_end; k += q.k_step) {
+            uint32_t v[4];
+            load_chunk(mask + (int64_t)k * N + q.c0, q, v);
+            int t = q.t0, t_end = tcol0[t + 1];
+            bool rf = rowflag[(int64_t)t * K + k] != 0;
+            for (int j = 0; j < q.w; ++j) {
+                if (q.c0 + j >= t_end) {
+                    ++t;
+                    t_end = tcol0[t + 1];
+                    rf = rowflag[(int64_t)t * K + k] != 0;
+                }
+                const bool m = chunk_byte(v, j) != 0;
+                const bool e = rf && ((cf >> j) & 1u);
+                bad += m != e;
+            }
+        }
+    }
+    // one atomic per wave that saw a mismatch
+    for (int off = 32; off > 0; off >>= 1)
+        bad += __shfl_down(bad, off);
+    if ((threadIdx.x & 63) == 0 && bad)
+        atomicAdd(mismatch, (unsigned long long)bad);
 }
 
 // counts[t] = kept rows of tile t, counts[n_tiles + t] = kept columns of tile t
-__global__ void count_flags_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K,
+__global__ void count_flags_kernel(const uint8_t *rowflag, const uint8_t *colflag, int K,
                                    const int32_t *tcol0, int n_tiles, int32_t *counts)
 {
     __shared__ int s_sum[2];
@@ -272,7 +352,7 @@ __device__ void block_compact(const uint8_t *flag8, const uint32_t *flag32, int 
 
 // grid (n_tiles, 2): y == 0 rows, y == 1 columns
 __global__ void __launch_bounds__(256)
-    compact_lists_kernel(const uint8_t *rowflag, const uint32_t *colflag, int K,
+    compact_lists_kernel(const uint8_t *rowflag, const uint8_t *colflag, int K,
                          const int32_t *tcol0, const int32_t *k_ptr, const int32_t *n_ptr,
                          int32_t *kept_k, int32_t *rel_k, int32_t *kept_n, int32_t *rel_n)
 {
@@ -281,7 +361,7 @@ __global__ void __launch_bounds__(256)
         block_compact(rowflag + (int64_t)t * K, nullptr, K, kept_k + k_ptr[t], rel_k + k_ptr[t]);
     } else {
         const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
-        block_compact(nullptr, colflag + c0, w, kept_n + n_ptr[t], rel_n + n_ptr[t]);
+        block_compact(colflag + c0, nullptr, w, kept_n + n_ptr[t], rel_n + n_ptr[t]);
     }
 }
 
@@ -674,7 +754,7 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     auto up = [](size_t b) { return (b + 255) / 256 * 256; };
     const size_t o_rowflag = 0;
     const size_t o_colflag = o_rowflag + up((size_t)nt * K);
-    const size_t o_mismatch = o_colflag + up(sizeof(uint32_t) * N);
+    const size_t o_mismatch = o_colflag + up((size_t)N);
     const size_t o_counts = o_mismatch + up(sizeof(unsigned long long));
     const size_t o_tcol0 = o_counts + up(sizeof(int32_t) * 2 * nt);
     const size_t o_kptr = o_tcol0 + up(sizeof(int32_t) * (nt + 1));
@@ -695,25 +775,26 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
 
     TW_TRY(hipMalloc((void **)&ws, ws_bytes));
     uint8_t *d_rowflag = reinterpret_cast<uint8_t *>(ws + o_rowflag);
-    uint32_t *d_colflag = reinterpret_cast<uint32_t *>(ws + o_colflag);
+    uint8_t *d_colflag = reinterpret_cast<uint8_t *>(ws + o_colflag);
     unsigned long long *d_mismatch = reinterpret_cast<unsigned long long *>(ws + o_mismatch);
     int32_t *d_counts = reinterpret_cast<int32_t *>(ws + o_counts);
     int32_t *d_tcol0 = reinterpret_cast<int32_t *>(ws + o_tcol0);
     int32_t *d_kptr = reinterpret_cast<int32_t *>(ws + o_kptr);
     int32_t *d_nptr = reinterpret_cast<int32_t *>(ws + o_nptr);
     TW_TRY(hipMemcpy(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
-    // column flags and the mismatch counter start at zero (they are adjacent in the workspace)
-    TW_TRY(hipMemset(d_colflag, 0, o_counts - o_colflag));
+    // row flags, column flags and the mismatch counter start at zero (adjacent in the workspace)
+    TW_TRY(hipMemset(ws, 0, o_counts));
 
     {
-        const int64_t n_rt = (int64_t)K * nt;
-        hipLaunchKernelGGL(row_flags_kernel, dim3((unsigned)((n_rt + 255) / 256)), dim3(256), 0,
-                           nullptr, d_mask, K, N, d_tcol0, nt, d_rowflag);
-        hipLaunchKernelGGL(col_flags_kernel, dim3((N + 255) / 256, (K + 63) / 64), dim3(256), 0,
-                           nullptr, d_mask, K, N, d_colflag);
-        const int64_t n_el = (int64_t)K * N;
-        hipLaunchKernelGGL(validate_tw_kernel, dim3((unsigned)((n_el + 255) / 256)), dim3(256), 0,
-                           nullptr, d_mask, K, N, d_tcol0, nt, d_rowflag, d_colflag, d_mismatch);
+        // lanes next to each other take the chunks of one row: 64 of them where a row has that
+        // many, else 32 or 16 (two or four rows per wave)
+        const int nchunk = (N + 15) / 16;
+        const int cw = nchunk > 32 ? 64 : (nchunk > 16 ? 32 : 16);
+        const dim3 grid((unsigned)((nchunk + cw - 1) / cw), (unsigned)((K + 63) / 64));
+        hipLaunchKernelGGL(mask_flags_kernel, grid, dim3(256), 0, nullptr, d_mask, K, N, d_tcol0, nt,
+                           cw, d_rowflag, d_colflag);
+        hipLaunchKernelGGL(validate_tw_kernel, grid, dim3(256), 0, nullptr, d_mask, K, N, d_tcol0, nt,
+                           cw, d_rowflag, d_colflag, d_mismatch);
         hipLaunchKernelGGL(count_flags_kernel, dim3(nt), dim3(256), 0, nullptr, d_rowflag,
                            d_colflag, K, d_tcol0, nt, d_counts);
         TW_TRY(hipGetLastError());

@@ -262,23 +262,35 @@ __global__ void __launch_bounds__(256)
     ChunkPos q;
     unsigned bad = 0;
     if (chunk_pos(mask, K, N, tcol0, n_tiles, cw, q)) {
-        uint32_t cf = 0; // bit j: column c0 + j is kept
+        // 0x01 in every byte of the chunk whose column is kept
+        uint32_t cf[4] = {0u, 0u, 0u, 0u};
         for (int j = 0; j < q.w; ++j)
-            cf |= (colflag[q.c0 + j] ? 1u : 0u) << j;
+            cf[j >> 2] |= (colflag[q.c0 + j] ? 1u : 0u) << ((j & 3) * 8);
         for (int k = q.k_begin; k < q.k_end; k += q.k_step) {
             uint32_t v[4];
             load_chunk(mask + (int64_t)k * N + q.c0, q, v);
-            int t = q.t0, t_end = tcol0[t + 1];
-            bool rf = rowflag[(int64_t)t * K + k] != 0;
-            for (int j = 0; j < q.w; ++j) {
-                if (q.c0 + j >= t_end) {
-                    ++t;
-                    t_end = tcol0[t + 1];
-                    rf = rowflag[(int64_t)t * K + k] != 0;
+            if (q.one_tile) {
+                // byte-parallel: 0x01 where the mask byte is non-zero, against (row kept) & cf
+                const uint32_t rf = rowflag[(int64_t)q.t0 * K + k] ? 0xFFFFFFFFu : 0u;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t x = v[i];
+                    const uint32_t nz = ((x | ((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu)) >> 7) & 0x01010101u;
+                    bad += __popc(nz ^ (cf[i] & rf));
                 }
-                const bool m = chunk_byte(v, j) != 0;
-                const bool e = rf && ((cf >> j) & 1u);
-                bad += m != e;
+            } else {
+                int t = q.t0, t_end = tcol0[t + 1];
+                bool rf = rowflag[(int64_t)t * K + k] != 0;
+                for (int j = 0; j < q.w; ++j) {
+                    if (q.c0 + j >= t_end) {
+                        ++t;
+                        t_end = tcol0[t + 1];
+                        rf = rowflag[(int64_t)t * K + k] != 0;
+                    }
+                    const bool m = chunk_byte(v, j) != 0;
+                    const bool e = rf && chunk_byte(cf, j);
+                    bad += m != e;
+                }
             }
         }
     }

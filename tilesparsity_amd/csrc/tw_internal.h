@@ -93,6 +93,13 @@ struct tw_plan {
     tw::TileDev *d_tiles = nullptr;
     void *d_Bp = nullptr;
     int32_t *d_tickets = nullptr; // kTicketSlots pairs
+    // Ownership: every pointer above points into one of these two allocations.  d_lists holds the
+    // four index arrays when the pre-pass compacted them on the device (else they sit in d_slab);
+    // d_slab holds the unit / tile tables, the pruned-column and padded kept-K lists, the packing
+    // table, the ticket slots and the packed weight.
+    void *d_lists = nullptr;
+    void *d_slab = nullptr;
+    void *d_pack_tiles = nullptr; // tw::PackTile[n_tiles] for packing from a dense weight
     mutable unsigned next_slot = 0;
     int cu_count = 0;
 };

@@ -493,29 +493,65 @@ int finalize_plan_geometry(tw_plan *p)
         p->n_pipe_units += u.k_pad > 0;
     p->n_zero_tiles = (int)ztiles.size();
 
-    int st;
-    if (!p->d_kept_k) {
-        std::vector<int32_t> rel_k(p->kept_k_idx.size()), rel_n(p->kept_n_idx.size());
+    // One device allocation for everything the plan owns besides lists that were compacted on
+    // the device: [staged tables, uploaded with one copy][ticket slots][packed weight], the last
+    // two zeroed with one memset.
+    std::vector<int32_t> rel_k, rel_n;
+    const bool lists_here = p->d_kept_k == nullptr;
+    if (lists_here) {
+        rel_k.resize(p->kept_k_idx.size());
+        rel_n.resize(p->kept_n_idx.size());
         for (int t = 0; t < nt; ++t) {
             for (int i = p->kept_k_ptr[t]; i < p->kept_k_ptr[t + 1]; ++i)
                 rel_k[i] = p->kept_k_idx[i] - (i - p->kept_k_ptr[t]);
             for (int i = p->kept_n_ptr[t]; i < p->kept_n_ptr[t + 1]; ++i)
                 rel_n[i] = p->kept_n_idx[i] - (i - p->kept_n_ptr[t]);
         }
-        if ((st = upload(&p->d_kept_k, p->kept_k_idx)) || (st = upload(&p->d_kept_n, p->kept_n_idx)) ||
-            (st = upload(&p->d_rel_k, rel_k)) || (st = upload(&p->d_rel_n, rel_n)))
-            return st;
     }
-    if ((st = upload(&p->d_units, units)) || (st = upload(&p->d_tiles, ztiles)) ||
-        (st = upload(&p->d_pruned_n, pruned_n)) || (st = upload(&p->d_kept_k_pad, kept_k_pad)))
-        return st;
-    size_t bp_bytes = std::max<int64_t>(p->packed_elems, 8) * 2;
-    if (hipMalloc(&p->d_Bp, bp_bytes) != hipSuccess)
-        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the packed weight failed", bp_bytes);
-    TW_HIP(hipMemset(p->d_Bp, 0, bp_bytes));
-    if (hipMalloc((void **)&p->d_tickets, sizeof(int32_t) * 2 * kTicketSlots + 2048) != hipSuccess)
-        return fail(TW_ERR_ALLOC, "hipMalloc of the ticket slots failed");
-    TW_HIP(hipMemset(p->d_tickets, 0, sizeof(int32_t) * 2 * kTicketSlots + 2048));
+    const std::vector<PackTile> ptab = pack_tiles(p, nullptr);
+    std::vector<char> stage;
+    auto put = [&stage](const void *src, size_t bytes) { // returns the 256-aligned offset
+        const size_t off = (stage.size() + 255) / 256 * 256;
+        stage.resize(off + std::max<size_t>(bytes, 4), 0);
+        if (bytes)
+            std::memcpy(stage.data() + off, src, bytes);
+        return off;
+    };
+    const size_t o_units = put(units.data(), units.size() * sizeof(UnitDev));
+    const size_t o_tiles = put(ztiles.data(), ztiles.size() * sizeof(TileDev));
+    const size_t o_pruned = put(pruned_n.data(), pruned_n.size() * sizeof(int32_t));
+    const size_t o_kkpad = put(kept_k_pad.data(), kept_k_pad.size() * sizeof(int32_t));
+    const size_t o_ptab = put(ptab.data(), ptab.size() * sizeof(PackTile));
+    size_t o_kk = 0, o_kn = 0, o_rk = 0, o_rn = 0;
+    if (lists_here) {
+        o_kk = put(p->kept_k_idx.data(), p->kept_k_idx.size() * sizeof(int32_t));
+        o_kn = put(p->kept_n_idx.data(), p->kept_n_idx.size() * sizeof(int32_t));
+        o_rk = put(rel_k.data(), rel_k.size() * sizeof(int32_t));
+        o_rn = put(rel_n.data(), rel_n.size() * sizeof(int32_t));
+    }
+    const size_t o_tickets = (stage.size() + 255) / 256 * 256;
+    const size_t ticket_bytes = sizeof(int32_t) * 2 * kTicketSlots + 2048;
+    const size_t o_bp = (o_tickets + ticket_bytes + 1023) / 1024 * 1024;
+    const size_t bp_bytes = (size_t)std::max<int64_t>(p->packed_elems, 8) * 2;
+    char *slab = nullptr;
+    if (hipMalloc((void **)&slab, o_bp + bp_bytes) != hipSuccess)
+        return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the plan failed", o_bp + bp_bytes);
+    p->d_slab = slab;
+    TW_HIP(hipMemcpy(slab, stage.data(), stage.size(), hipMemcpyHostToDevice));
+    TW_HIP(hipMemset(slab + o_tickets, 0, o_bp + bp_bytes - o_tickets));
+    p->d_units = reinterpret_cast<UnitDev *>(slab + o_units);
+    p->d_tiles = reinterpret_cast<TileDev *>(slab + o_tiles);
+    p->d_pruned_n = reinterpret_cast<int32_t *>(slab + o_pruned);
+    p->d_kept_k_pad = reinterpret_cast<int32_t *>(slab + o_kkpad);
+    p->d_pack_tiles = slab + o_ptab;
+    if (lists_here) {
+        p->d_kept_k = reinterpret_cast<int32_t *>(slab + o_kk);
+        p->d_kept_n = reinterpret_cast<int32_t *>(slab + o_kn);
+        p->d_rel_k = reinterpret_cast<int32_t *>(slab + o_rk);
+        p->d_rel_n = reinterpret_cast<int32_t *>(slab + o_rn);
+    }
+    p->d_tickets = reinterpret_cast<int32_t *>(slab + o_tickets);
+    p->d_Bp = slab + o_bp;
     TW_HIP(hipGetDevice(&p->device));
     {
         // the CU count of a device does not change: ask once per device
@@ -539,18 +575,13 @@ int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s, const uint8_t *
     const int64_t mg = max_groups(p);
     if (mg == 0)
         return TW_OK;
-    std::vector<PackTile> pt = pack_tiles(p, nullptr);
-    PackTile *d_pt = nullptr;
-    int st = upload(&d_pt, pt);
-    if (st)
-        return st;
     dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
-    hipLaunchKernelGGL(pack_dense_kernel, grid, dim3(256), 0, s, d_pt, p->d_kept_k, p->d_kept_n,
-                       d_B, p->N, p->dtype, (uint16_t *)p->d_Bp, d_mask);
+    hipLaunchKernelGGL(pack_dense_kernel, grid, dim3(256), 0, s,
+                       static_cast<const PackTile *>(p->d_pack_tiles), p->d_kept_k, p->d_kept_n, d_B,
+                       p->N, p->dtype, (uint16_t *)p->d_Bp, d_mask);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
         e = hipStreamSynchronize(s);
-    hipFree(d_pt);
     if (e != hipSuccess)
         return fail(TW_ERR_DEVICE, "weight packing kernel failed: %s", hipGetErrorString(e));
     return TW_OK;
@@ -606,16 +637,8 @@ static void free_plan(tw_plan *p)
 {
     if (!p)
         return;
-    hipFree(p->d_kept_k);
-    hipFree(p->d_kept_n);
-    hipFree(p->d_rel_k);
-    hipFree(p->d_rel_n);
-    hipFree(p->d_pruned_n);
-    hipFree(p->d_kept_k_pad);
-    hipFree(p->d_units);
-    hipFree(p->d_tiles);
-    hipFree(p->d_Bp);
-    hipFree(p->d_tickets);
+    hipFree(p->d_lists);
+    hipFree(p->d_slab);
     delete p;
 }
 
@@ -844,24 +867,38 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
         p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + counts[nt + t];
     }
     const size_t sk = std::max(p->kept_k_ptr[nt], 1), sn = std::max(p->kept_n_ptr[nt], 1);
-    TW_TRY(hipMemcpy(d_kptr, p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
-    TW_TRY(hipMemcpy(d_nptr, p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
-    TW_TRY(hipMalloc((void **)&p->d_kept_k, sizeof(int32_t) * sk));
-    TW_TRY(hipMalloc((void **)&p->d_rel_k, sizeof(int32_t) * sk));
-    TW_TRY(hipMalloc((void **)&p->d_kept_n, sizeof(int32_t) * sn));
-    TW_TRY(hipMalloc((void **)&p->d_rel_n, sizeof(int32_t) * sn));
+    {
+        // the two prefix arrays are adjacent in the workspace: one upload
+        std::vector<char> ptrs(o_nptr - o_kptr + sizeof(int32_t) * (nt + 1), 0);
+        std::memcpy(ptrs.data(), p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1));
+        std::memcpy(ptrs.data() + (o_nptr - o_kptr), p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1));
+        TW_TRY(hipMemcpy(d_kptr, ptrs.data(), ptrs.size(), hipMemcpyHostToDevice));
+    }
+    // [kept_k | kept_n | rel_k | rel_n], each at a 256-byte boundary: the first two come back
+    // to the host with one copy
+    const size_t l_kn = up(sizeof(int32_t) * sk), l_rk = l_kn + up(sizeof(int32_t) * sn);
+    const size_t l_rn = l_rk + up(sizeof(int32_t) * sk);
+    char *lists = nullptr;
+    TW_TRY(hipMalloc((void **)&lists, l_rn + up(sizeof(int32_t) * sn)));
+    p->d_lists = lists;
+    p->d_kept_k = reinterpret_cast<int32_t *>(lists);
+    p->d_kept_n = reinterpret_cast<int32_t *>(lists + l_kn);
+    p->d_rel_k = reinterpret_cast<int32_t *>(lists + l_rk);
+    p->d_rel_n = reinterpret_cast<int32_t *>(lists + l_rn);
     hipLaunchKernelGGL(compact_lists_kernel, dim3(nt, 2), dim3(256), 0, nullptr, d_rowflag,
                        d_colflag, K, d_tcol0, d_kptr, d_nptr, p->d_kept_k, p->d_rel_k, p->d_kept_n,
                        p->d_rel_n);
     TW_TRY(hipGetLastError());
     p->kept_k_idx.resize(p->kept_k_ptr[nt]);
     p->kept_n_idx.resize(p->kept_n_ptr[nt]);
-    if (!p->kept_k_idx.empty())
-        TW_TRY(hipMemcpy(p->kept_k_idx.data(), p->d_kept_k, sizeof(int32_t) * p->kept_k_idx.size(),
-                         hipMemcpyDeviceToHost));
-    if (!p->kept_n_idx.empty())
-        TW_TRY(hipMemcpy(p->kept_n_idx.data(), p->d_kept_n, sizeof(int32_t) * p->kept_n_idx.size(),
-                         hipMemcpyDeviceToHost));
+    {
+        std::vector<char> both(l_kn + sizeof(int32_t) * sn);
+        TW_TRY(hipMemcpy(both.data(), lists, both.size(), hipMemcpyDeviceToHost));
+        if (!p->kept_k_idx.empty())
+            std::memcpy(p->kept_k_idx.data(), both.data(), sizeof(int32_t) * p->kept_k_idx.size());
+        if (!p->kept_n_idx.empty())
+            std::memcpy(p->kept_n_idx.data(), both.data() + l_kn, sizeof(int32_t) * p->kept_n_idx.size());
+    }
     cleanup();
 #undef TW_TRY
     st = validate_lists(K, N, nt, p->tile_col0.data(), p->tile_width.data(), p->kept_k_ptr.data(),

@@ -159,7 +159,8 @@ int tw_plan_from_mask_cover(int K, int N, int dtype, int n_tiles, const int32_t 
  * memory, e.g. the masks tw_prune_* leave on the device and a weight that already lives there, so
  * nothing but the tile table, the list lengths and the lists' host copies crosses the host
  * boundary.  cover != 0 as tw_plan_from_mask_cover, else as tw_plan_from_mask_tiles.  The call
- * works on the default stream and returns when the plan is complete. */
+ * works on the default stream and returns when the plan is complete; work that writes mask or B
+ * on a stream that does not synchronise with the default stream must have finished before. */
 int tw_plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                              const int32_t *tile_width, const uint8_t *mask, const float *B,
                              int cover, tw_plan **out);

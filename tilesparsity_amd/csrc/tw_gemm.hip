@@ -1403,6 +1403,14 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
                     (long long)lda, (long long)ldc);
     if (((uintptr_t)A & 15) || ((uintptr_t)C & 15))
         return fail(TW_ERR_ALIGNMENT, "A and C must be 16-byte aligned");
+    {
+        // the plan's tables and packed weight live on the device it was built on
+        int dev = -1;
+        TW_HIP(hipGetDevice(&dev));
+        if (dev != plan->device)
+            return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d",
+                        plan->device, dev);
+    }
     if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR) {
         // layout-generic path (element strides), 128-row blocks, one workgroup per item
         GemmArgs a;
@@ -1517,17 +1525,14 @@ int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A
                       const int32_t *K_cal, const int32_t *const *mask_n,
                       const int32_t *const *mask_k, const int64_t *off_B, const int64_t *off_C,
                       void *stream)
-{
+try {
+    if (M > 0 && (M & 7))
+        return fail(TW_ERR_ALIGNMENT, "M=%d must be a multiple of 8 here (lda = ldc = M)", M);
     tw_plan *plan = nullptr;
     int st = tw_plan_from_stream_operands(M, N, K, dtype, B, block_num, N_cal, K_cal, mask_n,
                                           mask_k, off_B, off_C, &plan);
     if (st)
         return st;
-    const int64_t ld = (M + 7) / 8 * 8;
-    if (ld != M) {
-        tw_plan_destroy(plan);
-        return fail(TW_ERR_ALIGNMENT, "M=%d must be a multiple of 8 here (lda = ldc = M)", M);
-    }
     st = tw_gemm(plan, A, TW_LAYOUT_KMAJOR, M, C, TW_LAYOUT_KMAJOR, M, M, alpha, beta,
                  TW_PRUNED_UNTOUCHED, stream);
     if (!st) {
@@ -1538,6 +1543,7 @@ int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A
     tw_plan_destroy(plan);
     return st;
 }
+TW_CATCH_TO_STATUS
 
 int tw_cast_f32(const float *src, void *dst, int64_t n, int dtype, void *stream)
 {

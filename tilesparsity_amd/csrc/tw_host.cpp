@@ -152,7 +152,7 @@ int tw_offsets_to_kept(const int32_t *offsets, int n_kept, int limit, int32_t *k
 int tw_tile_partition(int M, int N, int K, int N_pruned, int K_pruned, int n_dim, int max_tiles,
                       int *block_num, int32_t *N_ori, int32_t *N_cal, int32_t *K_cal,
                       int64_t *off_B, int64_t *off_C)
-{
+try {
     if (!block_num || !N_ori || !N_cal || !K_cal || !off_B || !off_C)
         return tw::fail(TW_ERR_NULL, "an output array is NULL");
     if (M < 0 || N <= 0 || K <= 0 || n_dim <= 0 || N_pruned <= 0 || N_pruned > N || K_pruned < 0 ||
@@ -184,10 +184,11 @@ int tw_tile_partition(int M, int N, int K, int N_pruned, int K_pruned, int n_dim
     *block_num = bn;
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_tiles_from_mask(int K, int N, int G, const uint8_t *mask, int32_t *tile_col0,
                        int32_t *tile_width, int32_t *n_tiles)
-{
+try {
     if (K <= 0 || N <= 0)
         return tw::fail(TW_ERR_SHAPE, "K=%d N=%d must be positive", K, N);
     if (!mask || !tile_col0 || !tile_width || !n_tiles)
@@ -225,5 +226,6 @@ int tw_tiles_from_mask(int K, int N, int G, const uint8_t *mask, int32_t *tile_c
     *n_tiles = t + 1;
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 } // extern "C"

@@ -6,6 +6,8 @@
 #include <cstdarg>
 #include <cstdint>
 #include <cstdio>
+#include <exception>
+#include <new>
 #include <string>
 #include <vector>
 
@@ -115,6 +117,17 @@ int fail(int status, const char *fmt, ...);
         if (e_ != hipSuccess)                                                            \
             return ::tw::fail(TW_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(e_)); \
     } while (0)
+
+// Closes a function-try-block of a C-ABI entry point: no C++ exception crosses the boundary.
+#define TW_CATCH_TO_STATUS                                                               \
+    catch (const std::bad_alloc &)                                                       \
+    {                                                                                    \
+        return ::tw::fail(TW_ERR_ALLOC, "out of host memory");                           \
+    }                                                                                    \
+    catch (const std::exception &e)                                                      \
+    {                                                                                    \
+        return ::tw::fail(TW_ERR_ALLOC, "host-side failure: %s", e.what());              \
+    }
 
 // validation shared by the plan builders (host only)
 int validate_lists(int K, int N, int n_tiles, const int32_t *tile_col0, const int32_t *tile_width,

@@ -414,8 +414,14 @@ template <typename T> static int upload(T **dst, const std::vector<T> &src)
     size_t bytes = std::max<size_t>(src.size(), 1) * sizeof(T);
     if (hipMalloc((void **)dst, bytes) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes failed", bytes);
-    if (!src.empty())
-        TW_HIP(hipMemcpy(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice));
+    if (!src.empty()) {
+        hipError_t e = hipMemcpy(*dst, src.data(), src.size() * sizeof(T), hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            hipFree(*dst);
+            *dst = nullptr;
+            return fail(TW_ERR_DEVICE, "upload of %zu bytes failed: %s", bytes, hipGetErrorString(e));
+        }
+    }
     return TW_OK;
 }
 
@@ -675,7 +681,7 @@ int tw_plan_create(int K, int N, int dtype, int n_tiles, const int32_t *tile_col
                    const int32_t *tile_width, const int32_t *kept_k_ptr, const int32_t *kept_k_idx,
                    const int32_t *kept_n_ptr, const int32_t *kept_n_idx, const float *B,
                    tw_plan **out)
-{
+try {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
@@ -708,9 +714,10 @@ int tw_plan_create(int K, int N, int dtype, int n_tiles, const int32_t *tile_col
     *out = p;
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_create_dense(int K, int N, int G, int dtype, const float *B, tw_plan **out)
-{
+try {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
@@ -734,10 +741,11 @@ int tw_plan_create_dense(int K, int N, int G, int dtype, const float *B, tw_plan
     return tw_plan_create(K, N, dtype, nt, col0.data(), width.data(), kp.data(), ki.data(),
                           np.data(), ni.data(), B, out);
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const float *B,
                       tw_plan **out)
-{
+try {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
@@ -751,6 +759,7 @@ int tw_plan_from_mask(int K, int N, int G, int dtype, const uint8_t *mask, const
     }
     return tw_plan_from_mask_tiles(K, N, dtype, nt, col0.data(), width.data(), mask, B, out);
 }
+TW_CATCH_TO_STATUS
 
 // The pre-pass on device operands: d_mask is K x N bytes, d_B the fp32 weight, both row-major in
 // device memory.  Temporaries (flags, counters, the tile table) share one allocation.
@@ -951,28 +960,31 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
 int tw_plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                              const int32_t *tile_width, const uint8_t *mask, const float *B,
                              int cover, tw_plan **out)
-{
+try {
     return plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, cover != 0,
                                  out);
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_from_mask_tiles(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                             const int32_t *tile_width, const uint8_t *mask, const float *B,
                             tw_plan **out)
-{
+try {
     return plan_from_mask_impl(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, false, out);
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_from_mask_cover(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                             const int32_t *tile_width, const uint8_t *mask, const float *B,
                             tw_plan **out)
-{
+try {
     return plan_from_mask_impl(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, true, out);
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_from_export(int K, int N, int dtype, int n_kept_k, const int32_t *mask_i,
                         int n_kept_n, const int32_t *mask_o, const float *kernel, tw_plan **out)
-{
+try {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
@@ -1001,12 +1013,13 @@ int tw_plan_from_export(int K, int N, int dtype, int n_kept_k, const int32_t *ma
     return tw_plan_create(K, N, dtype, 1, &col0, &width, kp, kk.data(), np, kn.data(), B.data(),
                           out);
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_from_stream_operands(int M, int N, int K, int dtype, const void *B_stream,
                                  int block_num, const int32_t *N_cal, const int32_t *K_cal,
                                  const int32_t *const *mask_n, const int32_t *const *mask_k,
                                  const int64_t *off_B, const int64_t *off_C, tw_plan **out)
-{
+try {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
     *out = nullptr;
@@ -1079,6 +1092,7 @@ int tw_plan_from_stream_operands(int M, int N, int K, int dtype, const void *B_s
     *out = p;
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_info(const tw_plan *p, int64_t *info, int n_info)
 {
@@ -1109,7 +1123,7 @@ int tw_plan_info(const tw_plan *p, int64_t *info, int n_info)
 int tw_plan_export(const tw_plan *p, int32_t *tile_col0, int32_t *tile_width, int32_t *kept_k_ptr,
                    int32_t *kept_k_idx, int32_t *mask_k_rel, int32_t *kept_n_ptr,
                    int32_t *kept_n_idx, int32_t *mask_n_rel, uint16_t *B_stream)
-{
+try {
     if (!p)
         return fail(TW_ERR_NULL, "plan is NULL");
     const int nt = p->n_tiles;
@@ -1148,6 +1162,7 @@ int tw_plan_export(const tw_plan *p, int32_t *tile_col0, int32_t *tile_width, in
     }
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_plan_destroy(tw_plan *plan)
 {

@@ -707,7 +707,7 @@ int tw_tiles_every_g_columns(int N, int G, int32_t *tile_col0, int32_t *tile_wid
 
 int tw_tiles_every_g_kept_columns(int N, int G, const uint8_t *col_mask, int32_t *tile_col0,
                                   int32_t *tile_width, int32_t *n_tiles)
-{
+try {
     if (N <= 0 || G <= 0)
         return fail(TW_ERR_SHAPE, "N=%d G=%d must be positive", N, G);
     if (!col_mask || !tile_col0 || !tile_width || !n_tiles)
@@ -728,11 +728,12 @@ int tw_tiles_every_g_kept_columns(int N, int G, const uint8_t *col_mask, int32_t
     *n_tiles = t + 1;
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_tile_row_norms(int K, int N, const float *scores, int n_tiles,
                             const int32_t *tile_col0, const int32_t *tile_width,
                             const uint8_t *col_keep, float *norms, void *stream)
-{
+try {
     if (K <= 0 || N <= 0 || n_tiles <= 0)
         return fail(TW_ERR_SHAPE, "K=%d N=%d n_tiles=%d must be positive", K, N, n_tiles);
     if (!scores || !tile_col0 || !tile_width || !norms)
@@ -776,9 +777,10 @@ int tw_prune_tile_row_norms(int K, int N, const float *scores, int n_tiles,
     TW_HIP(hipStreamSynchronize(s));
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_col_norms(int K, int N, const float *scores, float *norms, void *stream)
-{
+try {
     if (K <= 0 || N <= 0)
         return fail(TW_ERR_SHAPE, "K=%d N=%d must be positive", K, N);
     if (!scores || !norms)
@@ -796,10 +798,11 @@ int tw_prune_col_norms(int K, int N, const float *scores, float *norms, void *st
     TW_HIP(hipStreamSynchronize(s));
     return TW_OK;
 }
+TW_CATCH_TO_STATUS
 
 int tw_percentile_linear(const float *values, int64_t n, double q, int q_type, double *result,
                          void *stream)
-{
+try {
     if (!values || !result)
         return fail(TW_ERR_NULL, "a pointer is NULL");
     if (q_type != TW_Q_F32 && q_type != TW_Q_F64)
@@ -811,11 +814,12 @@ int tw_percentile_linear(const float *values, int64_t n, double q, int q_type, d
         st = read_threshold(t, (hipStream_t)stream, result);
     return st;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_tiled_wise_1d(int n_layers, const int32_t *K, const int32_t *N,
                            const float *const *scores, double sparsity, int q_type,
                            int granularity, uint8_t *const *masks, double *threshold, void *stream)
-{
+try {
     int st = check_layers(n_layers, K, N, scores, masks, granularity);
     if (st)
         return st;
@@ -838,10 +842,11 @@ int tw_prune_tiled_wise_1d(int n_layers, const int32_t *K, const int32_t *N,
         *threshold = value;
     return st;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_granularity(int K, int N, const float *scores, double sparsity, int q_type,
                          int granularity, uint8_t *mask, void *stream)
-{
+try {
     const float *const sc[1] = {scores};
     uint8_t *const mk[1] = {mask};
     int st = check_layers(1, &K, &N, sc, mk, granularity);
@@ -863,12 +868,13 @@ int tw_prune_granularity(int K, int N, const float *scores, double sparsity, int
         st = read_threshold(thr, (hipStream_t)stream, &value); // waits for the mask
     return st;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
                            const float *const *scores, double sparsity, int q_type, int transform,
                            int granularity, uint8_t *const *masks, uint8_t *const *col_masks,
                            double *thresholds, void *stream)
-{
+try {
     int st = check_layers(n_layers, K, N, scores, masks, granularity);
     if (st)
         return st;
@@ -945,11 +951,12 @@ int tw_prune_tiled_wise_2d(int n_layers, const int32_t *K, const int32_t *N,
     }
     return st;
 }
+TW_CATCH_TO_STATUS
 
 int tw_prune_mix(int n_layers, const int32_t *K, const int32_t *N, const float *const *scores,
                  const uint8_t *const *layer_masks, double g1percent, int q_type,
                  uint8_t *const *masks, double *threshold, void *stream)
-{
+try {
     int st = check_layers(n_layers, K, N, scores, masks, 1);
     if (st)
         return st;
@@ -993,5 +1000,6 @@ int tw_prune_mix(int n_layers, const int32_t *K, const int32_t *N, const float *
         *threshold = value;
     return st;
 }
+TW_CATCH_TO_STATUS
 
 } // extern "C"

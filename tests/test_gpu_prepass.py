@@ -148,3 +148,36 @@ def test_device_operands_give_the_same_plan(tw, oracle):
             assert np.array_equal(bd, oracle.cast_bits(oracle.stream_weight(np.where(m != 0, W, np.float32(0)), po.cover_tiles_from_mask(m, table)), "bf16"))
     with pytest.raises(tw.TwError):
         tw.Plan.from_device_mask(8, 8, 0, [(0, 8)], "f16", 0)
+
+
+def test_long_rows_and_wide_tiles_span_several_segments(tw, oracle):
+    """Counting and compaction work on segments of 1024 flags: a mask with more rows than that,
+    tiles wider than that (one of them not starting at a multiple of 16) and a narrow tile between
+    them gives the oracle's lists and packed weight."""
+    rng = np.random.default_rng(23)
+    K, widths = 2500, [1500, 40, 2101, 7]
+    N = sum(widths)
+    table, tiles, c0 = [], [], 0
+    for w in widths:
+        kk = np.sort(rng.choice(K, int(K * 0.3), replace=False)).astype(np.int32)
+        kn = np.sort(rng.choice(w, max(1, int(w * 0.7)), replace=False)).astype(np.int32)
+        table.append((c0, w))
+        tiles.append(dict(col0=c0, width=w, kept_k=kk, kept_n=kn))
+        c0 += w
+    B = rng.standard_normal((K, N)).astype(np.float32)
+    mask = oracle.plan_mask(K, N, tiles)
+    print("segmented pre-pass", K, N, widths, flush=True)
+    with tw.Plan.from_mask_tiles(mask, table, "f16", B) as plan:
+        check_export(oracle, plan, tiles, B, "f16")
+    # rows kept only in the last segment, columns only in a tile's last segment
+    mask2 = np.zeros((K, N), np.uint8)
+    mask2[2400:2500:3, 1400:1500:2] = 1
+    mask2[5, 1540 + 2090] = 1
+    with tw.Plan.from_mask_tiles(mask2, table, "bf16", B) as plan:
+        got, _ = plan.export()
+        assert np.array_equal(got[0]["kept_k"], np.arange(2400, 2500, 3))
+        assert np.array_equal(got[0]["kept_n"], np.arange(1400, 1500, 2))
+        assert len(got[1]["kept_k"]) == 0 and len(got[1]["kept_n"]) == 0
+        assert np.array_equal(got[2]["kept_k"], [5]) and np.array_equal(got[2]["kept_n"], [2090])
+        assert np.array_equal(got[2]["mask_k"], [5]) and np.array_equal(got[2]["mask_n"], [2090])
+        assert len(got[3]["kept_k"]) == 0

@@ -212,42 +212,74 @@ __device__ __forceinline__ uint32_t chunk_byte(const uint32_t (&v)[4], int j)
     return (v[j >> 2] >> ((j & 3) * 8)) & 0xFFu;
 }
 
+// Rows a thread loads before it looks at any of them, so that this many 16-byte loads are in
+// flight per lane.
+constexpr int kFlagBatch = 8;
+
 // rowflag[t*K + k] = 1 where any byte of mask[k][tcol0[t] .. tcol0[t+1]) is non-zero,
 // colflag[c] = 1 where any byte of column c is; both arrays start zeroed and only receive ones.
 __global__ void __launch_bounds__(256)
-    mask_flags_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0, int n_tiles, int cw,
-                      uint8_t *rowflag, uint8_t *colflag)
+    mask_flags_kernel(const uint8_t *__restrict__ mask, int K, int N,
+                      const int32_t *__restrict__ tcol0, int n_tiles, int cw,
+                      uint8_t *__restrict__ rowflag, uint8_t *__restrict__ colflag)
 {
     ChunkPos q;
     if (!chunk_pos(mask, K, N, tcol0, n_tiles, cw, q))
         return;
+    // Of the lanes that hold chunks of one row inside one tile, only the lowest one with a
+    // non-zero chunk stores the row flag.  seg_mask: the lanes below this one from the tile's
+    // first whole chunk in this row on (they all lie in tile t0 when this chunk does).
+    const int lane = (int)(threadIdx.x & 63u);
+    unsigned long long seg_mask = 0ull;
+    if (q.one_tile) {
+        const int in_row = (int)(threadIdx.x % cw);
+        const int first_chunk = (tcol0[q.t0] + 15) >> 4;
+        const int seg_lane = lane - in_row + max(0, first_chunk - (int)blockIdx.x * cw);
+        seg_mask = ((1ull << lane) - 1ull) & ~((1ull << seg_lane) - 1ull);
+    }
     uint32_t acc[4] = {0u, 0u, 0u, 0u};
-    for (int k = q.k_begin; k < q.k_end; k += q.k_step) {
-        uint32_t v[4];
-        load_chunk(mask + (int64_t)k * N + q.c0, q, v);
-        if (q.one_tile) {
-            if (v[0] | v[1] | v[2] | v[3])
-                rowflag[(int64_t)q.t0 * K + k] = 1;
-        } else {
-            int t = q.t0, t_end = tcol0[t + 1];
-            uint32_t any = 0;
-            for (int j = 0; j < q.w; ++j) {
-                if (q.c0 + j >= t_end) {
-                    if (any)
-                        rowflag[(int64_t)t * K + k] = 1;
-                    any = 0;
-                    ++t;
-                    t_end = tcol0[t + 1];
-                }
-                any |= chunk_byte(v, j);
-            }
-            if (any)
-                rowflag[(int64_t)t * K + k] = 1;
+    for (int k0 = q.k_begin; k0 < q.k_end; k0 += kFlagBatch * q.k_step) {
+        uint32_t v[kFlagBatch][4];
+#pragma unroll
+        for (int i = 0; i < kFlagBatch; ++i) {
+            const int k = k0 + i * q.k_step;
+            if (k < q.k_end)
+                load_chunk(mask + (int64_t)k * N + q.c0, q, v[i]);
+            else
+                v[i][0] = v[i][1] = v[i][2] = v[i][3] = 0u;
         }
-        acc[0] |= v[0];
-        acc[1] |= v[1];
-        acc[2] |= v[2];
-        acc[3] |= v[3];
+#pragma unroll
+        for (int i = 0; i < kFlagBatch; ++i) {
+            const int k = k0 + i * q.k_step;
+            const bool nz = (v[i][0] | v[i][1] | v[i][2] | v[i][3]) != 0u;
+            // lanes of one row run the same iterations, so a row's lanes all vote here
+            const unsigned long long votes = __ballot(nz && q.one_tile);
+            if (!nz)
+                continue; // also every row past k_end
+            if (q.one_tile) {
+                if ((votes & seg_mask) == 0ull)
+                    rowflag[(int64_t)q.t0 * K + k] = 1;
+            } else {
+                int t = q.t0, t_end = tcol0[t + 1];
+                uint32_t any = 0;
+                for (int j = 0; j < q.w; ++j) {
+                    if (q.c0 + j >= t_end) {
+                        if (any)
+                            rowflag[(int64_t)t * K + k] = 1;
+                        any = 0;
+                        ++t;
+                        t_end = tcol0[t + 1];
+                    }
+                    any |= chunk_byte(v[i], j);
+                }
+                if (any)
+                    rowflag[(int64_t)t * K + k] = 1;
+            }
+            acc[0] |= v[i][0];
+            acc[1] |= v[i][1];
+            acc[2] |= v[i][2];
+            acc[3] |= v[i][3];
+        }
     }
     for (int j = 0; j < q.w; ++j)
         if (chunk_byte(acc, j))
@@ -256,8 +288,10 @@ __global__ void __launch_bounds__(256)
 
 // counts the elements where mask != rowflag & colflag (a TW mask has none)
 __global__ void __launch_bounds__(256)
-    validate_tw_kernel(const uint8_t *mask, int K, int N, const int32_t *tcol0, int n_tiles, int cw,
-                       const uint8_t *rowflag, const uint8_t *colflag, unsigned long long *mismatch)
+    validate_tw_kernel(const uint8_t *__restrict__ mask, int K, int N,
+                       const int32_t *__restrict__ tcol0, int n_tiles, int cw,
+                       const uint8_t *__restrict__ rowflag, const uint8_t *__restrict__ colflag,
+                       unsigned long long *__restrict__ mismatch)
 {
     ChunkPos q;
     unsigned bad = 0;
@@ -266,30 +300,46 @@ __global__ void __launch_bounds__(256)
         uint32_t cf[4] = {0u, 0u, 0u, 0u};
         for (int j = 0; j < q.w; ++j)
             cf[j >> 2] |= (colflag[q.c0 + j] ? 1u : 0u) << ((j & 3) * 8);
-        for (int k = q.k_begin; k < q.k_end; k += q.k_step) {
-            uint32_t v[4];
-            load_chunk(mask + (int64_t)k * N + q.c0, q, v);
-            if (q.one_tile) {
-                // byte-parallel: 0x01 where the mask byte is non-zero, against (row kept) & cf
-                const uint32_t rf = rowflag[(int64_t)q.t0 * K + k] ? 0xFFFFFFFFu : 0u;
+        for (int k0 = q.k_begin; k0 < q.k_end; k0 += kFlagBatch * q.k_step) {
+            uint32_t v[kFlagBatch][4];
+            uint32_t rf[kFlagBatch]; // all ones where the row of tile t0 is kept
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const uint32_t x = v[i];
-                    const uint32_t nz = ((x | ((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu)) >> 7) & 0x01010101u;
-                    bad += __popc(nz ^ (cf[i] & rf));
+            for (int i = 0; i < kFlagBatch; ++i) {
+                const int k = k0 + i * q.k_step;
+                if (k < q.k_end) {
+                    load_chunk(mask + (int64_t)k * N + q.c0, q, v[i]);
+                    rf[i] = rowflag[(int64_t)q.t0 * K + k] ? 0xFFFFFFFFu : 0u;
+                } else {
+                    v[i][0] = v[i][1] = v[i][2] = v[i][3] = 0u;
+                    rf[i] = 0u;
                 }
-            } else {
-                int t = q.t0, t_end = tcol0[t + 1];
-                bool rf = rowflag[(int64_t)t * K + k] != 0;
-                for (int j = 0; j < q.w; ++j) {
-                    if (q.c0 + j >= t_end) {
-                        ++t;
-                        t_end = tcol0[t + 1];
-                        rf = rowflag[(int64_t)t * K + k] != 0;
+            }
+#pragma unroll
+            for (int i = 0; i < kFlagBatch; ++i) {
+                const int k = k0 + i * q.k_step;
+                if (q.one_tile) {
+                    // byte-parallel: 0x01 where the mask byte is non-zero, against (row kept) & cf;
+                    // a row past k_end has v == 0 and rf == 0 and adds nothing
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        const uint32_t x = v[i][w];
+                        const uint32_t nz =
+                            ((x | ((x & 0x7F7F7F7Fu) + 0x7F7F7F7Fu)) >> 7) & 0x01010101u;
+                        bad += __popc(nz ^ (cf[w] & rf[i]));
                     }
-                    const bool m = chunk_byte(v, j) != 0;
-                    const bool e = rf && chunk_byte(cf, j);
-                    bad += m != e;
+                } else if (k < q.k_end) {
+                    int t = q.t0, t_end = tcol0[t + 1];
+                    bool r = rf[i] != 0u;
+                    for (int j = 0; j < q.w; ++j) {
+                        if (q.c0 + j >= t_end) {
+                            ++t;
+                            t_end = tcol0[t + 1];
+                            r = rowflag[(int64_t)t * K + k] != 0;
+                        }
+                        const bool m = chunk_byte(v[i], j) != 0;
+                        const bool e = r && chunk_byte(cf, j);
+                        bad += m != e;
+                    }
                 }
             }
         }
@@ -301,79 +351,123 @@ __global__ void __launch_bounds__(256)
         atomicAdd(mismatch, (unsigned long long)bad);
 }
 
-// counts[t] = kept rows of tile t, counts[n_tiles + t] = kept columns of tile t
-__global__ void count_flags_kernel(const uint8_t *rowflag, const uint8_t *colflag, int K,
-                                   const int32_t *tcol0, int n_tiles, int32_t *counts)
+// Counting and compaction work on segments of kSegFlags flags (rows of one tile, or columns of
+// one tile), one workgroup per segment: grid (n_tiles, n_seg_k + n_seg_n), y < n_seg_k rows.
+// seg_counts holds the kept flags per segment, tile-major: first the n_tiles * n_seg_k row
+// entries, then the n_tiles * n_seg_n column entries.
+constexpr int kSegFlags = 1024;
+constexpr int kSegRounds = kSegFlags / 256;
+
+struct FlagSegment {
+    const uint8_t *flag; // the tile's flag vector
+    int n;               // its length
+    int first;           // first flag of this segment
+    int entry;           // index of this segment among the row (or column) entries
+    bool rows;
+};
+
+__device__ __forceinline__ FlagSegment flag_segment(const uint8_t *rowflag, const uint8_t *colflag,
+                                                    int K, const int32_t *tcol0, int n_seg_k,
+                                                    int n_seg_n)
 {
-    __shared__ int s_sum[2];
+    FlagSegment g;
     const int t = blockIdx.x;
-    if (threadIdx.x == 0) {
-        s_sum[0] = 0;
-        s_sum[1] = 0;
-    }
-    __syncthreads();
-    int rk = 0, ck = 0;
-    for (int k = threadIdx.x; k < K; k += blockDim.x)
-        rk += rowflag[(int64_t)t * K + k];
-    const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
-    for (int j = threadIdx.x; j < w; j += blockDim.x)
-        ck += colflag[c0 + j] ? 1 : 0;
-    atomicAdd(&s_sum[0], rk);
-    atomicAdd(&s_sum[1], ck);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        counts[t] = s_sum[0];
-        counts[n_tiles + t] = s_sum[1];
-    }
+    g.rows = (int)blockIdx.y < n_seg_k;
+    const int seg = g.rows ? (int)blockIdx.y : (int)blockIdx.y - n_seg_k;
+    g.flag = g.rows ? rowflag + (int64_t)t * K : colflag + tcol0[t];
+    g.n = g.rows ? K : tcol0[t + 1] - tcol0[t];
+    g.first = seg * kSegFlags;
+    g.entry = t * (g.rows ? n_seg_k : n_seg_n) + seg;
+    return g;
 }
 
-// Ordered compaction of one flag vector by one 256-thread block: writes the
-// ascending kept indices and the relative offsets kept[i] - i.
-__device__ void block_compact(const uint8_t *flag8, const uint32_t *flag32, int n, int32_t *kept,
-                              int32_t *rel)
+__global__ void __launch_bounds__(256)
+    count_flags_kernel(const uint8_t *__restrict__ rowflag, const uint8_t *__restrict__ colflag,
+                       int K, const int32_t *__restrict__ tcol0, int n_tiles, int n_seg_k,
+                       int n_seg_n, int32_t *__restrict__ seg_counts)
 {
     __shared__ int s_wave[4];
-    __shared__ int s_base;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    if (threadIdx.x == 0)
-        s_base = 0;
-    __syncthreads();
-    for (int i0 = 0; i0 < n; i0 += 256) {
-        const int i = i0 + threadIdx.x;
-        bool f = false;
-        if (i < n)
-            f = flag8 ? flag8[i] != 0 : flag32[i] != 0;
-        const unsigned long long b = __ballot(f);
-        const int before = __popcll(b & ((1ull << lane) - 1ull));
-        if (lane == 0)
-            s_wave[wave] = __popcll(b);
-        __syncthreads();
-        int off = s_base;
-        for (int w = 0; w < wave; ++w)
-            off += s_wave[w];
-        if (f) {
-            kept[off + before] = i;
-            rel[off + before] = i - (off + before);
-        }
-        __syncthreads();
-        if (threadIdx.x == 0)
-            s_base += s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
-        __syncthreads();
+    const FlagSegment g = flag_segment(rowflag, colflag, K, tcol0, n_seg_k, n_seg_n);
+    int c = 0;
+#pragma unroll
+    for (int j = 0; j < kSegRounds; ++j) {
+        const int i = g.first + j * 256 + (int)threadIdx.x;
+        if (i < g.n)
+            c += g.flag[i] != 0;
     }
+    for (int off = 32; off > 0; off >>= 1)
+        c += __shfl_down(c, off);
+    if ((threadIdx.x & 63) == 0)
+        s_wave[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0)
+        seg_counts[(g.rows ? 0 : n_tiles * n_seg_k) + g.entry] =
+            s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
 }
 
-// grid (n_tiles, 2): y == 0 rows, y == 1 columns
+// Ordered compaction of one segment: the ascending kept indices and the relative offsets
+// kept[i] - i land where the segments before it (seg_counts, tile-major) leave off.
 __global__ void __launch_bounds__(256)
-    compact_lists_kernel(const uint8_t *rowflag, const uint8_t *colflag, int K,
-                         const int32_t *tcol0, const int32_t *k_ptr, const int32_t *n_ptr,
-                         int32_t *kept_k, int32_t *rel_k, int32_t *kept_n, int32_t *rel_n)
+    compact_lists_kernel(const uint8_t *__restrict__ rowflag, const uint8_t *__restrict__ colflag,
+                         int K, const int32_t *__restrict__ tcol0, int n_tiles, int n_seg_k,
+                         int n_seg_n, const int32_t *__restrict__ seg_counts,
+                         int32_t *__restrict__ kept_k, int32_t *__restrict__ rel_k,
+                         int32_t *__restrict__ kept_n, int32_t *__restrict__ rel_n)
 {
-    const int t = blockIdx.x;
-    if (blockIdx.y == 0) {
-        block_compact(rowflag + (int64_t)t * K, nullptr, K, kept_k + k_ptr[t], rel_k + k_ptr[t]);
-    } else {
-        const int c0 = tcol0[t], w = tcol0[t + 1] - c0;
-        block_compact(colflag + c0, nullptr, w, kept_n + n_ptr[t], rel_n + n_ptr[t]);
+    __shared__ int s_sum[2][4];
+    __shared__ int s_round[kSegRounds][4];
+    const FlagSegment g = flag_segment(rowflag, colflag, K, tcol0, n_seg_k, n_seg_n);
+    const int lane = (int)(threadIdx.x & 63u), wave = (int)(threadIdx.x >> 6);
+    bool f[kSegRounds];
+#pragma unroll
+    for (int j = 0; j < kSegRounds; ++j) {
+        const int i = g.first + j * 256 + (int)threadIdx.x;
+        f[j] = i < g.n && g.flag[i] != 0;
+    }
+    // kept flags before this segment: in the tiles before (a) and earlier in this tile (b)
+    const int32_t *cnt = seg_counts + (g.rows ? 0 : n_tiles * n_seg_k);
+    const int tile_first = (int)blockIdx.x * (g.rows ? n_seg_k : n_seg_n);
+    int a = 0, b = 0;
+    for (int i = (int)threadIdx.x; i < g.entry; i += 256) {
+        const int v = cnt[i];
+        if (i < tile_first)
+            a += v;
+        else
+            b += v;
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        a += __shfl_down(a, off);
+        b += __shfl_down(b, off);
+    }
+    int before[kSegRounds];
+#pragma unroll
+    for (int j = 0; j < kSegRounds; ++j) {
+        const unsigned long long votes = __ballot(f[j]);
+        before[j] = __popcll(votes & ((1ull << lane) - 1ull));
+        if (lane == 0)
+            s_round[j][wave] = __popcll(votes);
+    }
+    if (lane == 0) {
+        s_sum[0][wave] = a;
+        s_sum[1][wave] = b;
+    }
+    __syncthreads();
+    const int in_tile = s_sum[1][0] + s_sum[1][1] + s_sum[1][2] + s_sum[1][3];
+    const int tile_base = s_sum[0][0] + s_sum[0][1] + s_sum[0][2] + s_sum[0][3];
+    int32_t *kept = (g.rows ? kept_k : kept_n) + tile_base;
+    int32_t *rel = (g.rows ? rel_k : rel_n) + tile_base;
+    int rank = in_tile; // position in the tile's list of this round's first kept flag
+#pragma unroll
+    for (int j = 0; j < kSegRounds; ++j) {
+        int mine = rank + before[j];
+        for (int w = 0; w < wave; ++w)
+            mine += s_round[j][w];
+        if (f[j]) {
+            const int i = g.first + j * 256 + (int)threadIdx.x;
+            kept[mine] = i;
+            rel[mine] = i - mine;
+        }
+        rank += s_round[j][0] + s_round[j][1] + s_round[j][2] + s_round[j][3];
     }
 }
 
@@ -544,7 +638,11 @@ int finalize_plan_geometry(tw_plan *p)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the plan failed", o_bp + bp_bytes);
     p->d_slab = slab;
     TW_HIP(hipMemcpy(slab, stage.data(), stage.size(), hipMemcpyHostToDevice));
-    TW_HIP(hipMemset(slab + o_tickets, 0, o_bp + bp_bytes - o_tickets));
+    // asynchronous: the packing kernel follows on the same (default) stream and the builders wait
+    // for it; a plan with nothing to pack waits here
+    TW_HIP(hipMemsetAsync(slab + o_tickets, 0, o_bp + bp_bytes - o_tickets, nullptr));
+    if (p->packed_elems == 0)
+        TW_HIP(hipStreamSynchronize(nullptr));
     p->d_units = reinterpret_cast<UnitDev *>(slab + o_units);
     p->d_tiles = reinterpret_cast<TileDev *>(slab + o_tiles);
     p->d_pruned_n = reinterpret_cast<int32_t *>(slab + o_pruned);
@@ -796,14 +894,19 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
 
     // one allocation for all temporaries, carved at 256-byte boundaries
     auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+    int max_width = 0;
+    for (int t = 0; t < nt; ++t)
+        max_width = std::max(max_width, tile_width[t]);
+    const int n_seg_k = (K + kSegFlags - 1) / kSegFlags, n_seg_n = (max_width + kSegFlags - 1) / kSegFlags;
+    if ((int64_t)nt * (n_seg_k + n_seg_n) > INT32_MAX || n_seg_k + n_seg_n > 65535)
+        return fail(TW_ERR_SHAPE, "K=%d rows in %d tiles are more than the pre-pass indexes", K, nt);
+    const size_t n_seg = (size_t)nt * (n_seg_k + n_seg_n);
     const size_t o_rowflag = 0;
     const size_t o_colflag = o_rowflag + up((size_t)nt * K);
     const size_t o_mismatch = o_colflag + up((size_t)N);
     const size_t o_counts = o_mismatch + up(sizeof(unsigned long long));
-    const size_t o_tcol0 = o_counts + up(sizeof(int32_t) * 2 * nt);
-    const size_t o_kptr = o_tcol0 + up(sizeof(int32_t) * (nt + 1));
-    const size_t o_nptr = o_kptr + up(sizeof(int32_t) * (nt + 1));
-    const size_t ws_bytes = o_nptr + up(sizeof(int32_t) * (nt + 1));
+    const size_t o_tcol0 = o_counts + up(sizeof(int32_t) * n_seg);
+    const size_t ws_bytes = o_tcol0 + up(sizeof(int32_t) * (nt + 1));
     char *ws = nullptr;
     tw_plan *p = nullptr;
     auto cleanup = [&]() { hipFree(ws); };
@@ -821,14 +924,13 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     uint8_t *d_rowflag = reinterpret_cast<uint8_t *>(ws + o_rowflag);
     uint8_t *d_colflag = reinterpret_cast<uint8_t *>(ws + o_colflag);
     unsigned long long *d_mismatch = reinterpret_cast<unsigned long long *>(ws + o_mismatch);
-    int32_t *d_counts = reinterpret_cast<int32_t *>(ws + o_counts);
+    int32_t *d_seg_counts = reinterpret_cast<int32_t *>(ws + o_counts);
     int32_t *d_tcol0 = reinterpret_cast<int32_t *>(ws + o_tcol0);
-    int32_t *d_kptr = reinterpret_cast<int32_t *>(ws + o_kptr);
-    int32_t *d_nptr = reinterpret_cast<int32_t *>(ws + o_nptr);
     TW_TRY(hipMemcpy(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
     // row flags, column flags and the mismatch counter start at zero (adjacent in the workspace)
-    TW_TRY(hipMemset(ws, 0, o_counts));
+    TW_TRY(hipMemsetAsync(ws, 0, o_counts, nullptr));
 
+    const dim3 seg_grid((unsigned)nt, (unsigned)(n_seg_k + n_seg_n));
     {
         // lanes next to each other take the chunks of one row: 64 of them where a row has that
         // many, else 32 or 16 (two or four rows per wave)
@@ -839,16 +941,16 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
                            cw, d_rowflag, d_colflag);
         hipLaunchKernelGGL(validate_tw_kernel, grid, dim3(256), 0, nullptr, d_mask, K, N, d_tcol0, nt,
                            cw, d_rowflag, d_colflag, d_mismatch);
-        hipLaunchKernelGGL(count_flags_kernel, dim3(nt), dim3(256), 0, nullptr, d_rowflag,
-                           d_colflag, K, d_tcol0, nt, d_counts);
+        hipLaunchKernelGGL(count_flags_kernel, seg_grid, dim3(256), 0, nullptr, d_rowflag, d_colflag,
+                           K, d_tcol0, nt, n_seg_k, n_seg_n, d_seg_counts);
         TW_TRY(hipGetLastError());
     }
-    // mismatch counter and the 2 * nt counts come back with one copy (they are adjacent)
+    // the mismatch counter and the segment counts come back with one copy (they are adjacent)
     std::vector<char> back(o_tcol0 - o_mismatch);
     TW_TRY(hipMemcpy(back.data(), ws + o_mismatch, back.size(), hipMemcpyDeviceToHost));
     unsigned long long mismatch = 0;
     std::memcpy(&mismatch, back.data(), sizeof(mismatch));
-    const int32_t *counts = reinterpret_cast<const int32_t *>(back.data() + (o_counts - o_mismatch));
+    const int32_t *seg_counts = reinterpret_cast<const int32_t *>(back.data() + (o_counts - o_mismatch));
     if (mismatch != 0 && !cover) {
         cleanup();
         return fail(TW_ERR_NOT_TW,
@@ -872,17 +974,15 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     for (int t = 0; t < nt; ++t) {
         p->tile_col0[t] = tile_col0[t];
         p->tile_width[t] = tile_width[t];
-        p->kept_k_ptr[t + 1] = p->kept_k_ptr[t] + counts[t];
-        p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + counts[nt + t];
+        int rows = 0, cols = 0;
+        for (int g = 0; g < n_seg_k; ++g)
+            rows += seg_counts[(size_t)t * n_seg_k + g];
+        for (int g = 0; g < n_seg_n; ++g)
+            cols += seg_counts[(size_t)nt * n_seg_k + (size_t)t * n_seg_n + g];
+        p->kept_k_ptr[t + 1] = p->kept_k_ptr[t] + rows;
+        p->kept_n_ptr[t + 1] = p->kept_n_ptr[t] + cols;
     }
     const size_t sk = std::max(p->kept_k_ptr[nt], 1), sn = std::max(p->kept_n_ptr[nt], 1);
-    {
-        // the two prefix arrays are adjacent in the workspace: one upload
-        std::vector<char> ptrs(o_nptr - o_kptr + sizeof(int32_t) * (nt + 1), 0);
-        std::memcpy(ptrs.data(), p->kept_k_ptr.data(), sizeof(int32_t) * (nt + 1));
-        std::memcpy(ptrs.data() + (o_nptr - o_kptr), p->kept_n_ptr.data(), sizeof(int32_t) * (nt + 1));
-        TW_TRY(hipMemcpy(d_kptr, ptrs.data(), ptrs.size(), hipMemcpyHostToDevice));
-    }
     // [kept_k | kept_n | rel_k | rel_n], each at a 256-byte boundary: the first two come back
     // to the host with one copy
     const size_t l_kn = up(sizeof(int32_t) * sk), l_rk = l_kn + up(sizeof(int32_t) * sn);
@@ -894,9 +994,9 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     p->d_kept_n = reinterpret_cast<int32_t *>(lists + l_kn);
     p->d_rel_k = reinterpret_cast<int32_t *>(lists + l_rk);
     p->d_rel_n = reinterpret_cast<int32_t *>(lists + l_rn);
-    hipLaunchKernelGGL(compact_lists_kernel, dim3(nt, 2), dim3(256), 0, nullptr, d_rowflag,
-                       d_colflag, K, d_tcol0, d_kptr, d_nptr, p->d_kept_k, p->d_rel_k, p->d_kept_n,
-                       p->d_rel_n);
+    hipLaunchKernelGGL(compact_lists_kernel, seg_grid, dim3(256), 0, nullptr, d_rowflag, d_colflag, K,
+                       d_tcol0, nt, n_seg_k, n_seg_n, d_seg_counts, p->d_kept_k, p->d_rel_k,
+                       p->d_kept_n, p->d_rel_n);
     TW_TRY(hipGetLastError());
     p->kept_k_idx.resize(p->kept_k_ptr[nt]);
     p->kept_n_idx.resize(p->kept_n_ptr[nt]);

@@ -79,14 +79,19 @@ template <> struct Elem<TW_BF16> {
     }
 };
 
-// 16-byte chunk of column c, rows m..m+7 of a K-major matrix, honouring the M edge.  The store
-// writes through to memory (sc0 sc1) and does not linger in the caches (nt): C is written once
-// and not read again by this launch, and lines left dirty in the L2s would otherwise all be
-// written back after the last wave has ended, where nothing overlaps them.
-__device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M)
+// 16-byte chunk of column c, rows m..m+7 of a K-major matrix, honouring the M edge.  With
+// `through` the store writes through to memory (sc0 sc1) and does not linger in the caches (nt):
+// C is written once and not read again by this launch, and lines left dirty in the L2s would
+// otherwise all be written back after the last wave has ended, where nothing overlaps them.  A
+// small output is better left in the L2s: that write-back is short then, and shorter than the
+// last stores' way to memory.
+__device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M, bool through)
 {
     if (m + 8 <= M) {
-        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+        if (through)
+            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+        else
+            *reinterpret_cast<u32x4 *>(dst) = v;
     } else if (m < M) {
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         for (int e = 0; e < M - m; ++e)
@@ -268,17 +273,30 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     // shared counter (which starts at 0 for every launch) one item ahead, with the atomic of
     // the claim after that already in flight.
     const int ticket_base = gridDim.x;
-    int t_pending = 0; // thread 0: claim in flight
+    int t_pending = 0;   // thread 0: claim in flight
+    bool closed = false; // thread 0: the queue is exhausted, no claim is in flight
+    int t_done = -1;     // thread 0: workgroups counted as done before this one
     if (tid == 0)
         t_pending = atomicAdd(&p.ticket[0], 1);
     Item cur = make_item(blockIdx.x);
     Item nxt = cur;
     bool have_next = false; // nxt is known for the current item
-    // Publishes the claim in flight as the next item and starts the claim after it.
+    // Publishes the claim in flight as the next item and starts the claim after it.  A ticket
+    // past the end makes the current item the workgroup's last: all its claims have returned, so
+    // it counts itself as done right away (the workgroup counted last re-arms the slot when it
+    // leaves) and that count's round trip is over before the item ends.
     auto claim_next = [&]() {
         if (tid == 0) {
-            s_tk[0] = ticket_base + t_pending;
-            t_pending = atomicAdd(&p.ticket[0], 1);
+            const int t = closed ? p.n_items : ticket_base + t_pending;
+            s_tk[0] = t;
+            if (!closed) {
+                if (t < p.n_items) {
+                    t_pending = atomicAdd(&p.ticket[0], 1);
+                } else {
+                    closed = true;
+                    t_done = atomicAdd(&p.ticket[1], 1);
+                }
+            }
         }
         __syncthreads();
         // tickets are workgroup-uniform: keep them, and everything derived from them, scalar
@@ -319,7 +337,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                     v.z = w[2];
                     v.w = w[3];
                 }
-                store_chunk(dst, v, m, p.M);
+                store_chunk(dst, v, m, p.M, p.store_through != 0);
             }
         } else {
             // ---- GEMM item ------------------------------------------------------
@@ -536,7 +554,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 v.y = lo.y;
                 v.z = hi.x;
                 v.w = hi.y;
-                store_chunk(C + (int64_t)c * p.ldc + tc.m_ld, v, tc.m_ld, p.M);
+                store_chunk(C + (int64_t)c * p.ldc + tc.m_ld, v, tc.m_ld, p.M, p.store_through != 0);
             }
         }
 
@@ -553,16 +571,11 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     if (blockIdx.x == 0 && tid < 256)
         reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
 #endif
-    // the last workgroup to leave re-arms the ticket slot for the next launch; waiting for
-    // the pending ticket first keeps every atomic of this workgroup ahead of that reset
-    if (tid == 0) {
-        __threadfence();
-        const int done = atomicAdd(&p.ticket[1], t_pending >= 0 ? 1 : 1);
-        if (done == (int)gridDim.x - 1) {
-            p.ticket[0] = 0;
-            p.ticket[1] = 0;
-            __threadfence();
-        }
+    // the workgroup counted last re-arms the ticket slot for the next launch: every workgroup's
+    // claims had returned before it was counted
+    if (tid == 0 && t_done == (int)gridDim.x - 1) {
+        p.ticket[0] = 0;
+        p.ticket[1] = 0;
     }
 }
 
@@ -682,16 +695,42 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     const int ticket_base = 2 * gridDim.x;
     int t_pending = 0;                     // thread 0: result of the claim in flight
     int t_next = gridDim.x + blockIdx.x;   // thread 0: the next ticket once known, or -1
+    bool closed = false;    // thread 0: no claim of this workgroup is in flight, none will follow
+    bool announced = false; // thread 0: the workgroup has been counted as done with the counter
+    int t_done = -1;        // thread 0: workgroups counted before this one (atomic's result)
     if (tid == 0)
         t_pending = atomicAdd(&p.ticket[0], 1);
-    // Picks up the claim in flight and starts the one after it.  Called before an item's output
-    // stores are issued: memory operations complete in order, so waiting for an atomic issued
-    // after them (or overwriting its register) would wait for the stores as well.
+    // Picks up the claim in flight and starts the one after it, unless the queue is exhausted.
+    // Called before an item's output stores are issued: memory operations complete in order, so
+    // waiting for an atomic issued after them (or overwriting its register) would wait for the
+    // stores as well.
     auto pick_up = [&]() {
         if (tid == 0 && t_next < 0) {
-            t_next = ticket_base + t_pending;
-            asm volatile("" : "+v"(t_next)); // here, not where it is published
-            t_pending = atomicAdd(&p.ticket[0], 1);
+            if (closed) {
+                t_next = p.n_items;
+            } else {
+                t_next = ticket_base + t_pending;
+                asm volatile("" : "+v"(t_next)); // here, not where it is published
+                if (t_next < p.n_items)
+                    t_pending = atomicAdd(&p.ticket[0], 1);
+                else
+                    closed = true;
+            }
+        }
+    };
+    // Thread 0, when it hands out the ticket after the current item: a ticket past the end means
+    // that the current item is the workgroup's last.  All its claims have returned by then, so it
+    // counts itself as done with the counter right away and the count's round trip is over long
+    // before the item ends; the workgroup counted last re-arms the slot when it leaves.
+    auto announce = [&]() {
+        if (t_next >= p.n_items && !announced) {
+            if (!closed) {
+                // the second fixed item is already past the end: the first claim is in flight
+                asm volatile("" ::"v"(t_pending));
+                closed = true;
+            }
+            t_done = atomicAdd(&p.ticket[1], 1);
+            announced = true;
         }
     };
     // An item with at least one step learns its successor without barriers of its own: thread 0
@@ -700,6 +739,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         if (tid == 0) {
             pick_up();
             s_tk[0] = t_next;
+            announce();
             t_next = -1;
         }
     };
@@ -708,6 +748,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         if (tid == 0) {
             pick_up();
             s_tk[0] = t_next;
+            announce();
             t_next = -1;
         }
         TW_WS_STAMP(0, 6, 256)
@@ -743,7 +784,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 v.z = w[2];
                 v.w = w[3];
             }
-            store_chunk(dst, v, m, p.M);
+            store_chunk(dst, v, m, p.M, p.store_through != 0);
         }
     };
     // scatters the staged C tile (all threads): whole columns col0 + kept_n[j], 16-byte stores
@@ -760,7 +801,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             v.y = lo.y;
             v.z = hi.x;
             v.w = hi.y;
-            store_chunk(C + (int64_t)c * p.ldc + m_st, v, m_st, m_end);
+            store_chunk(C + (int64_t)c * p.ldc + m_st, v, m_st, m_end, p.store_through != 0);
         }
     };
 
@@ -1134,6 +1175,8 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     }
                 }
                 pick_up();
+                if (tid == 0 && announced)
+                    asm volatile("" : "+v"(t_done)); // the count has returned: read it before the stores
                 TW_LDS_BARRIER(); // the C tile is staged
                 store_tile(u, m0, cur.m_end);
             }
@@ -1158,15 +1201,11 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ws[tid];
 #endif
 #endif
-        // the last workgroup to leave re-arms the ticket slot for the next launch
-        if (tid == 0) {
-            __threadfence();
-            const int done = atomicAdd(&p.ticket[1], t_pending >= 0 ? 1 : 1);
-            if (done == (int)gridDim.x - 1) {
-                p.ticket[0] = 0;
-                p.ticket[1] = 0;
-                __threadfence();
-            }
+        // the workgroup counted last re-arms the ticket slot for the next launch: every
+        // workgroup's claims had returned before it was counted
+        if (tid == 0 && t_done == (int)gridDim.x - 1) {
+            p.ticket[0] = 0;
+            p.ticket[1] = 0;
         }
     }
 }
@@ -1325,6 +1364,9 @@ __global__ void insert_row_kernel(uint16_t *matrix, const uint16_t *matrix_2, in
         matrix[(int64_t)(i + mask[i]) * columns + j] = matrix_2[(int64_t)i * columns + j];
 }
 
+// outputs above this size are written through to memory: the size of one XCD's L2
+constexpr int64_t kStoreThroughBytes = 4 << 20;
+
 static int env_int(const char *name, int dflt)
 {
     const char *v = getenv(name);
@@ -1437,6 +1479,7 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
         a.n_arg_units = 0;
         a.bias = ep ? ep->bias : nullptr;
         a.act = ep ? ep->activation : TW_ACT_NONE;
+        a.store_through = 0;
         if (a.n_items == 0)
             return TW_OK;
         const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
@@ -1493,6 +1536,8 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
     a.beta = beta;
     a.bias = ep ? ep->bias : nullptr;
     a.act = ep ? ep->activation : TW_ACT_NONE;
+    // an output larger than one L2 is written through (see store_chunk)
+    a.store_through = (int64_t)M * plan->N * 2 > kStoreThroughBytes;
     if (a.n_items == 0)
         return TW_OK;
     const unsigned slot =

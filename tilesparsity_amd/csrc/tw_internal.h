@@ -66,6 +66,7 @@ struct GemmArgs {
     float alpha, beta;
     const float *bias;    // fp32 [N] added to every written column before the activation, or null
     int32_t act;          // TW_ACT_*
+    int32_t store_through; // output stores write through to memory (large outputs) or stay in L2
     int32_t *ticket;      // [0] next item, [1] finished workgroups
     void *dbg;            // 2 KiB scratch after the ticket slots (instrumented builds only)
     // Copy of `units` inside the kernel arguments for plans of at most kMaxArgUnits units

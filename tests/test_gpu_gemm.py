@@ -292,6 +292,46 @@ def test_repeated_launches_and_slot_reuse(tw, oracle):
         assert np.array_equal(from_device_bits(dC)[keep], first[keep, :M])
 
 
+def test_queue_is_rearmed_between_launches_of_different_sizes(tw, oracle):
+    """Launches with few items (one per workgroup), with several rounds of items per workgroup,
+    and with items that have no step or only fill zeros alternate on one plan, through every
+    ticket slot more than once: each launch re-arms the queue for the next, whatever its grid
+    was, so every result repeats bit for bit."""
+    import torch
+    rng = np.random.default_rng(27)
+    K, N, G, dtype = 320, 1536, 128, "bf16"
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.85, empty_every=5)
+    Ms = (8, 520, 33000)                  # 12 items; 36 items; 129 row blocks x 12 units
+    stream = torch.cuda.current_stream().cuda_stream
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        dA, dC, want = {}, {}, {}
+        for M in Ms:
+            ld = (M + 7) // 8 * 8
+            g = torch.Generator(device="cuda")
+            g.manual_seed(M)
+            dA[M] = torch.randn((K, ld), generator=g, device="cuda").to(torch.bfloat16)
+            dC[M] = torch.zeros((N, ld), dtype=torch.bfloat16, device="cuda")
+            plan.gemm(dA[M].data_ptr(), dC[M].data_ptr(), M, lda=ld, ldc=ld, stream=stream,
+                      pruned_cols=tw.PRUNED_ZERO)
+            torch.cuda.synchronize()
+            want[M] = dC[M].clone()
+            ref = (dA[M][:, :M].float().T.cpu().numpy() @
+                   (oracle.quantize(B, dtype) * oracle.plan_mask(K, N, tiles)))
+            got = dC[M][:, :M].float().T.cpu().numpy()
+            assert oracle.rel_error(got, ref) <= TOL[dtype], M
+        print("re-arm over mixed sizes", Ms, flush=True)
+        for i in range(3 * 256 + 5):
+            M = Ms[i % 3] if i % 7 else Ms[2 - i % 3]
+            ld = (M + 7) // 8 * 8
+            dC[M].fill_(1.0)
+            plan.gemm(dA[M].data_ptr(), dC[M].data_ptr(), M, lda=ld, ldc=ld, stream=stream,
+                      pruned_cols=tw.PRUNED_ZERO)
+            if i % 64 == 63 or i > 3 * 256:
+                torch.cuda.synchronize()
+                assert torch.equal(dC[M][:, :M], want[M][:, :M]), (i, M)
+
+
 def test_gemm_argument_errors(tw):
     import torch
     K, N, M = 64, 128, 64

@@ -572,7 +572,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
         reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
 #endif
     // the workgroup counted last re-arms the ticket slot for the next launch: every workgroup's
-    // claims had returned before it was counted
+    // claims had returned before it was counted.  Plain stores, made visible by the end of the
+    // kernel; a device-scope fence here would write back and invalidate this XCD's L2 under the
+    // workgroups that still stream through it.
     if (tid == 0 && t_done == (int)gridDim.x - 1) {
         p.ticket[0] = 0;
         p.ticket[1] = 0;
@@ -1202,7 +1204,9 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #endif
 #endif
         // the workgroup counted last re-arms the ticket slot for the next launch: every
-        // workgroup's claims had returned before it was counted
+        // workgroup's claims had returned before it was counted.  Plain stores, made visible by
+        // the end of the kernel; a device-scope fence here would write back and invalidate this
+        // XCD's L2 under the workgroups that still stream through it.
         if (tid == 0 && t_done == (int)gridDim.x - 1) {
             p.ticket[0] = 0;
             p.ticket[1] = 0;

@@ -155,6 +155,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 
     __shared__ __align__(16) uint16_t smem[SMEM];
     __shared__ int s_tk[2];
+    // Instrumented builds only (-DTW_EXP_TIMING): workgroup 0 records cycle stamps of its steps
+    // and phases in LDS and copies them behind the ticket slots, where tw_exp_read_debug reads
+    // them.  Not part of the shipped library.
 #ifdef TW_EXP_TIMING
     __shared__ unsigned long long s_ts[64 * 4];
 #define TW_STAMP(step, slot)                                                              \
@@ -240,9 +243,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     // loads pick their index out of that register with a cross-lane permute.
     auto load_idx = [&](const Thr &t, int s, int &ix) {
         ix = t.klist[s * BK + (lane & (BK - 1))];
-#ifdef TW_EXP_AWINDOW
-        ix &= 63;
-#endif
     };
     // No lane-dependent branches here: rows beyond K_t and chunks beyond M are loaded from a
     // valid address and replaced by zeros when they are staged (not here, so that nothing
@@ -426,19 +426,11 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     frags(s, ks, af, bf);
-#ifdef TW_EXP_NOMFMA
-#pragma unroll
-                    for (int ni = 0; ni < 2; ++ni)
-#pragma unroll
-                        for (int mi = 0; mi < 2; ++mi)
-                            acc[mi][ni][0] += __uint_as_float(af[mi].x ^ bf[ni].x);
-#else
 #pragma unroll
                     for (int ni = 0; ni < 2; ++ni)
 #pragma unroll
                         for (int mi = 0; mi < 2; ++mi)
                             acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
-#endif
                 }
                 TW_STAMP(s, 3)
             };
@@ -618,6 +610,8 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     __shared__ int s_tk[2];
     __shared__ int s_cols[BN];   // output columns of the current item's unit
     __shared__ float s_bias[BN]; // ... and their bias values (fused epilogue)
+    // Instrumented builds only (-DTW_EXP_TIMING=1: cycle stamps of workgroup 0's item number
+    // TW_EXP_ITEM; =2: start and end time of every workgroup), read back with tw_exp_read_debug.
 #ifdef TW_EXP_TIMING
     __shared__ unsigned long long s_ws[256];
 #ifndef TW_EXP_ITEM

@@ -200,12 +200,14 @@ __device__ __forceinline__ uint32_t sort_key(float v)
     return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
 }
 // Selection state in device memory, so that the passes follow each other on the stream without
-// a host round trip.
+// a host round trip.  Pass p (p = 0..3) counts, among the values whose key agrees with the digits
+// fixed by the passes before it, the digit at bit 24 - 8 p; which digit holds the rank is worked
+// out from the histograms by whoever needs it next (resolve_prefix).
 struct SelectState {
-    unsigned long long hist[256];
-    unsigned long long rank;      // rank still to find among the values matching the prefix
+    unsigned long long hist[4][256];
+    unsigned long long rank0;     // rank (0-based) of the wanted value
     unsigned long long count_le;  // values <= the k-th smallest
-    uint32_t prefix, mask;        // key bits fixed so far
+    uint32_t prefix;              // key of the k-th smallest (written with the threshold)
     uint32_t min_gt;              // smallest key above the k-th smallest's (0xFFFFFFFF: none)
     int32_t lost;                 // set if a pass found no digit (cannot happen for rank < n)
     float thr32;                  // the threshold, for the kernels that follow
@@ -215,31 +217,86 @@ struct SelectState {
 // The selection kernels work on segments of equal length laid end to end (one segment for the
 // network-wide thresholds, one per tile for per-tile thresholds): segment g = blockIdx.y (or
 // blockIdx.x for the one-workgroup kernels) uses state st[g] and values v[g*n .. g*n+n).
-__global__ void select_init_kernel(SelectState *st, unsigned long long rank)
+__global__ void __launch_bounds__(256) select_init_kernel(SelectState *st, unsigned long long rank)
 {
     st += blockIdx.x;
-    st->hist[threadIdx.x] = 0;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+        st->hist[p][threadIdx.x] = 0;
     if (threadIdx.x == 0) {
-        st->rank = rank;
+        st->rank0 = rank;
         st->count_le = 0;
         st->prefix = 0;
-        st->mask = 0;
         st->min_gt = 0xFFFFFFFFu;
         st->lost = 0;
     }
 }
 
-// hist[d] += number of values whose key matches the prefix in the masked bits and has digit d
-// at `shift`
+// The key digits that passes 0 .. npass-1 have fixed, the rank that is left among the values
+// matching them, and whether a pass found no digit.  Called by all 256 threads of a workgroup
+// (an inclusive scan of each histogram finds the digit whose count range holds the rank); every
+// thread returns the same values.
+__device__ void resolve_prefix(const SelectState *st, int npass, uint32_t &prefix, uint32_t &mask,
+                               unsigned long long &rank, bool &lost)
+{
+    __shared__ unsigned long long s_wave[4];
+    __shared__ unsigned long long s_before;
+    __shared__ int s_digit;
+    const int tid = (int)threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    prefix = 0;
+    mask = 0;
+    rank = st->rank0;
+    lost = false;
+    for (int p = 0; p < npass; ++p) {
+        const int shift = 24 - 8 * p;
+        const unsigned long long c = st->hist[p][tid];
+        unsigned long long incl = c;
+        for (int off = 1; off < 64; off <<= 1) {
+            const unsigned long long up = __shfl_up(incl, off);
+            if (lane >= off)
+                incl += up;
+        }
+        if (lane == 63)
+            s_wave[wave] = incl;
+        if (tid == 0)
+            s_digit = -1;
+        __syncthreads();
+        for (int w = 0; w < wave; ++w)
+            incl += s_wave[w];
+        const unsigned long long excl = incl - c;
+        if (c > 0 && excl <= rank && rank < incl) { // exactly one digit, if any
+            s_digit = tid;
+            s_before = excl;
+        }
+        __syncthreads();
+        int d = s_digit;
+        if (d < 0) {
+            lost = true;
+            d = 255;
+        } else {
+            rank -= s_before;
+        }
+        prefix |= (uint32_t)d << shift;
+        mask |= 255u << shift;
+        __syncthreads(); // the shared words are rewritten by the next pass
+    }
+}
+
+// hist[pass][d] += number of values whose key matches the digits fixed so far and has digit d
+// at bit 24 - 8 pass
 __global__ void __launch_bounds__(256)
-    select_hist_kernel(const float *v, int64_t n, int shift, SelectState *st)
+    select_hist_kernel(const float *v, int64_t n, int pass, SelectState *st)
 {
     st += blockIdx.y;
     v += (int64_t)blockIdx.y * n;
     __shared__ unsigned int s_h[256];
     s_h[threadIdx.x] = 0;
-    __syncthreads();
-    const uint32_t mask = st->mask, prefix = st->prefix;
+    uint32_t prefix, mask;
+    unsigned long long rank;
+    bool lost;
+    resolve_prefix(st, pass, prefix, mask, rank, lost);
+    __syncthreads(); // s_h is zeroed
+    const int shift = 24 - 8 * pass;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
          i += (int64_t)gridDim.x * blockDim.x) {
         const uint32_t key = sort_key(v[i]);
@@ -248,33 +305,7 @@ __global__ void __launch_bounds__(256)
     }
     __syncthreads();
     if (s_h[threadIdx.x])
-        atomicAdd(&st->hist[threadIdx.x], (unsigned long long)s_h[threadIdx.x]);
-}
-
-// one workgroup: picks the digit that holds the rank, fixes it in the prefix, clears the histogram
-__global__ void __launch_bounds__(256) select_digit_kernel(int shift, SelectState *st)
-{
-    st += blockIdx.x;
-    __shared__ unsigned long long s_c[256];
-    s_c[threadIdx.x] = st->hist[threadIdx.x];
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        unsigned long long rank = st->rank;
-        int d = 0;
-        for (; d < 256; ++d) {
-            if (rank < s_c[d])
-                break;
-            rank -= s_c[d];
-        }
-        if (d == 256) {
-            st->lost = 1;
-            d = 255;
-        }
-        st->rank = rank;
-        st->prefix |= (uint32_t)d << shift;
-        st->mask |= 255u << shift;
-    }
-    st->hist[threadIdx.x] = 0;
+        atomicAdd(&st->hist[pass][threadIdx.x], (unsigned long long)s_h[threadIdx.x]);
 }
 
 // count_le = number of values <= the selected one, min_gt = smallest key above it
@@ -282,7 +313,10 @@ __global__ void __launch_bounds__(256) rank_stats_kernel(const float *v, int64_t
 {
     st += blockIdx.y;
     v += (int64_t)blockIdx.y * n;
-    const uint32_t key_a = st->prefix;
+    uint32_t key_a, mask;
+    unsigned long long rank;
+    bool lost;
+    resolve_prefix(st, 4, key_a, mask, rank, lost);
     unsigned long long cnt = 0;
     unsigned int mn = 0xFFFFFFFFu;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
@@ -326,11 +360,20 @@ __device__ __forceinline__ float key_to_float(uint32_t key)
 // NumPy's two-sided linear interpolation between the k-th smallest value a and its upper
 // neighbour b (a again if it is repeated, or if the index is the last one): float32 throughout
 // for a float32 gamma, float64 with a float32 difference b - a otherwise.
-__global__ void select_lerp_kernel(SelectState *st, unsigned long long k, int top, int f64,
-                                   float gamma32, double gamma64)
+__global__ void __launch_bounds__(256)
+    select_lerp_kernel(SelectState *st, unsigned long long k, int top, int f64, float gamma32,
+                       double gamma64)
 {
     st += blockIdx.x;
-    const float a = key_to_float(st->prefix);
+    uint32_t key_a, mask;
+    unsigned long long rank;
+    bool lost;
+    resolve_prefix(st, 4, key_a, mask, rank, lost);
+    if (threadIdx.x != 0)
+        return;
+    st->prefix = key_a;
+    st->lost = lost ? 1 : 0;
+    const float a = key_to_float(key_a);
     float b = a;
     if (!top && st->count_le <= k + 1 && st->min_gt != 0xFFFFFFFFu)
         b = key_to_float(st->min_gt);
@@ -361,13 +404,36 @@ __global__ void col_keep_kernel(const float *cnorm, int N, const SelectState *st
 
 // mask[k][c] = (norm of row k in c's tile > threshold) and column c kept.  One thread per 16
 // consecutive columns of a row: one 16-byte store where the chunk is whole and aligned.
-__global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t n_chunks,
-                                 const SelectState *st, int f64)
+__global__ void __launch_bounds__(256)
+    fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t n_chunks,
+                     const SelectState *st, int f64)
 {
+    // the first chunk of every layer, so that a thread finds its layer without a chain of
+    // global loads (the first kFillCached layers; a search beyond them reads the table itself)
+    constexpr int kFillCached = 128;
+    __shared__ int64_t s_begin[kFillCached];
+    const int n_cached = min(n_layers, kFillCached);
+    for (int i = (int)threadIdx.x; i < n_cached; i += (int)blockDim.x)
+        s_begin[i] = layers[i].el_begin;
+    __syncthreads();
     const int64_t gidx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gidx >= n_chunks)
         return;
-    const PruneLayer L = layers[find_layer(layers, n_layers, gidx, true)];
+    int li;
+    if (n_layers > kFillCached && layers[kFillCached].el_begin <= gidx) {
+        li = kFillCached + find_layer(layers + kFillCached, n_layers - kFillCached, gidx, true);
+    } else {
+        int lo = 0, hi = n_cached;
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_begin[mid] <= gidx)
+                lo = mid;
+            else
+                hi = mid;
+        }
+        li = lo;
+    }
+    const PruneLayer L = layers[li];
     const bool per_tile = (L.flags & kPerTileThreshold) != 0;
     float thr32 = st->thr32;
     double thr64 = st->thr64;
@@ -375,14 +441,12 @@ __global__ void fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t
     const int cpr = (L.N + 15) >> 4; // chunks per row
     const int k = (int)(idx / cpr);
     const int c0 = (int)(idx - (int64_t)k * cpr) << 4;
-    int t = 0, hi = L.n_tiles;
-    while (hi - t > 1) {
-        const int mid = (t + hi) >> 1;
-        if (L.tcol0[mid] <= c0)
-            t = mid;
-        else
-            hi = mid;
-    }
+    // the tile of column c0: start where tiles of equal width would put it, then walk
+    int t = (int)((int64_t)c0 * L.n_tiles / L.N);
+    while (L.tcol0[t] > c0)
+        --t;
+    while (L.tcol0[t + 1] <= c0)
+        ++t;
     int t_end = L.tcol0[t + 1];
     float nv = L.norms[(int64_t)t * L.K + k];
     if (per_tile) {
@@ -580,12 +644,10 @@ int percentile_linear(Arena &ar, const float *d_v, int64_t n, double q, int q_is
     const int grid = (int)std::min<int64_t>(n_segments > 1 ? 64 : 1024, (n + 255) / 256);
     const dim3 g2(grid, n_segments), g1(n_segments);
     hipLaunchKernelGGL(select_init_kernel, g1, dim3(256), 0, s, st, k);
-    for (int shift = 24; shift >= 0; shift -= 8) {
-        hipLaunchKernelGGL(select_hist_kernel, g2, dim3(256), 0, s, d_v, n, shift, st);
-        hipLaunchKernelGGL(select_digit_kernel, g1, dim3(256), 0, s, shift, st);
-    }
+    for (int pass = 0; pass < 4; ++pass)
+        hipLaunchKernelGGL(select_hist_kernel, g2, dim3(256), 0, s, d_v, n, pass, st);
     hipLaunchKernelGGL(rank_stats_kernel, g2, dim3(256), 0, s, d_v, n, st);
-    hipLaunchKernelGGL(select_lerp_kernel, g1, dim3(1), 0, s, st, k, top ? 1 : 0, q_is_f64,
+    hipLaunchKernelGGL(select_lerp_kernel, g1, dim3(256), 0, s, st, k, top ? 1 : 0, q_is_f64,
                        gamma32, gamma64);
     TW_HIP(hipGetLastError());
     out->state = st;
@@ -596,8 +658,17 @@ int percentile_linear(Arena &ar, const float *d_v, int64_t n, double q, int q_is
 // waits for the stream and returns the threshold as a double
 int read_threshold(const Threshold &t, hipStream_t s, double *value)
 {
-    SelectState h;
-    TW_HIP(hipMemcpyAsync(&h, t.state, sizeof(h), hipMemcpyDeviceToHost, s));
+    // the words behind the histograms are all the host needs
+    struct Tail {
+        int32_t lost;
+        float thr32;
+        double thr64;
+    } h;
+    static_assert(offsetof(SelectState, thr64) - offsetof(SelectState, lost) == offsetof(Tail, thr64) &&
+                      sizeof(SelectState) - offsetof(SelectState, lost) == sizeof(Tail),
+                  "Tail mirrors the end of SelectState");
+    TW_HIP(hipMemcpyAsync(&h, reinterpret_cast<const char *>(t.state) + offsetof(SelectState, lost),
+                          sizeof(h), hipMemcpyDeviceToHost, s));
     TW_HIP(hipStreamSynchronize(s));
     if (h.lost)
         return fail(TW_ERR_DEVICE, "radix select lost its rank");
@@ -641,19 +712,24 @@ int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
         tab += (int64_t)lt[l].tcol0.size();
     }
     float *d_norms = ar.alloc_n<float>(total);
-    int32_t *d_tables = ar.alloc_n<int32_t>(tab);
-    PruneLayer *d_table = ar.alloc_n<PruneLayer>(n_layers);
-    if (!d_norms || !d_tables || !d_table)
+    // the layer table and the tile tables behind it share one buffer: one upload
+    const size_t table_bytes = (sizeof(PruneLayer) * n_layers + 15) / 16 * 16;
+    char *d_both = static_cast<char *>(ar.alloc(table_bytes + sizeof(int32_t) * tab));
+    if (!d_norms || !d_both)
         return fail(TW_ERR_ALLOC, "hipMalloc of %lld norms failed", (long long)total);
-    std::vector<int32_t> flat;
-    std::vector<PruneLayer> pl(n_layers);
+    PruneLayer *d_table = reinterpret_cast<PruneLayer *>(d_both);
+    int32_t *d_tables = reinterpret_cast<int32_t *>(d_both + table_bytes);
+    std::vector<char> both(table_bytes + sizeof(int32_t) * tab, 0);
+    PruneLayer *pl = reinterpret_cast<PruneLayer *>(both.data());
+    int32_t *flat = reinterpret_cast<int32_t *>(both.data() + table_bytes);
+    size_t n_flat = 0;
     int64_t n_pairs = 0, n_elems = 0;
     for (int l = 0; l < n_layers; ++l) {
-        PruneLayer &e = pl[l];
+        PruneLayer e;
         e.score = scores[l];
         e.mask = masks ? masks[l] : nullptr;
         e.colkeep = d_colkeep.empty() ? nullptr : d_colkeep[l];
-        e.tcol0 = d_tables + flat.size();
+        e.tcol0 = d_tables + n_flat;
         e.norms = d_norms + lt[l].norm_off;
         e.K = K[l];
         e.N = N[l];
@@ -663,12 +739,12 @@ int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
         e.el_begin = n_elems;
         n_pairs += (int64_t)e.K * e.n_tiles;
         n_elems += (int64_t)e.K * ((e.N + 15) / 16);
-        flat.insert(flat.end(), lt[l].tcol0.begin(), lt[l].tcol0.end());
+        std::memcpy(&pl[l], &e, sizeof(e));
+        std::memcpy(flat + n_flat, lt[l].tcol0.data(), sizeof(int32_t) * lt[l].tcol0.size());
+        n_flat += lt[l].tcol0.size();
     }
-    TW_HIP(hipMemcpyAsync(d_tables, flat.data(), sizeof(int32_t) * flat.size(),
-                          hipMemcpyHostToDevice, s));
-    TW_HIP(hipMemcpyAsync(d_table, pl.data(), sizeof(PruneLayer) * n_layers, hipMemcpyHostToDevice, s));
-    TW_HIP(hipStreamSynchronize(s)); // `flat` and `pl` are pageable host memory
+    TW_HIP(hipMemcpyAsync(d_both, both.data(), both.size(), hipMemcpyHostToDevice, s));
+    TW_HIP(hipStreamSynchronize(s)); // `both` is pageable host memory
     hipLaunchKernelGGL(tile_row_norms_kernel, dim3((unsigned)((n_pairs * 8 + 255) / 256)), dim3(256),
                        0, s, d_table, n_layers, n_pairs);
     TW_HIP(hipGetLastError());

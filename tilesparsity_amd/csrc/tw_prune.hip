@@ -107,7 +107,7 @@ struct PruneLayer {
     int32_t K, N, n_tiles;
     int32_t flags;          // kNormNotDivided, kPerTileThreshold
     int64_t rt_begin;       // first (row, tile) pair of this layer in the launch-wide numbering
-    int64_t el_begin;       // first 16-column chunk likewise (ceil(N/16) chunks per row)
+    int64_t el_begin;       // first item of the mask fill likewise (ceil(K/4) x ceil(N/16) items)
 };
 
 __device__ __forceinline__ int find_layer(const PruneLayer *layers, int n_layers, int64_t idx,
@@ -403,7 +403,9 @@ __global__ void col_keep_kernel(const float *cnorm, int N, const SelectState *st
 }
 
 // mask[k][c] = (norm of row k in c's tile > threshold) and column c kept.  One thread per 16
-// consecutive columns of a row: one 16-byte store where the chunk is whole and aligned.
+// consecutive columns of kFillRows consecutive rows: one 16-byte store per row where the chunk
+// is whole and aligned; the layer and tile look-ups are shared by the rows.
+constexpr int kFillRows = 4;
 __global__ void __launch_bounds__(256)
     fill_mask_kernel(const PruneLayer *layers, int n_layers, int64_t n_chunks,
                      const SelectState *st, int f64)
@@ -439,49 +441,67 @@ __global__ void __launch_bounds__(256)
     double thr64 = st->thr64;
     const int64_t idx = gidx - L.el_begin;
     const int cpr = (L.N + 15) >> 4; // chunks per row
-    const int k = (int)(idx / cpr);
-    const int c0 = (int)(idx - (int64_t)k * cpr) << 4;
-    // the tile of column c0: start where tiles of equal width would put it, then walk
-    int t = (int)((int64_t)c0 * L.n_tiles / L.N);
+    // (a 32-bit division where the layer's item count allows it: the 64-bit one is long)
+    const int kg = (idx >> 31) == 0 ? (int)((uint32_t)idx / (uint32_t)cpr) : (int)(idx / cpr);
+    const int c0 = (int)(idx - (int64_t)kg * cpr) << 4;
+    const int k0 = kg * kFillRows;
+    const int nrows = min(kFillRows, L.K - k0);
+    // the tile of column c0: start near where tiles of equal width would put it, then walk
+    int t = min(L.n_tiles - 1, (int)((float)c0 * (float)L.n_tiles / (float)L.N));
     while (L.tcol0[t] > c0)
         --t;
     while (L.tcol0[t + 1] <= c0)
         ++t;
     int t_end = L.tcol0[t + 1];
-    float nv = L.norms[(int64_t)t * L.K + k];
-    if (per_tile) {
-        thr32 = st[t].thr32;
-        thr64 = st[t].thr64;
-    }
-    bool row_keep = f64 ? (double)nv > thr64 : nv > thr32;
-    uint32_t w[4] = {0u, 0u, 0u, 0u};
-    const int n = min(16, L.N - c0);
-    for (int e = 0; e < n; ++e) {
-        const int c = c0 + e;
-        if (c >= t_end) {
-            ++t;
-            t_end = L.tcol0[t + 1];
-            nv = L.norms[(int64_t)t * L.K + k];
-            if (per_tile) {
-                thr32 = st[t].thr32;
-                thr64 = st[t].thr64;
-            }
-            row_keep = f64 ? (double)nv > thr64 : nv > thr32;
+    bool row_keep[kFillRows];
+    auto enter_tile = [&]() { // the rows' norms in tile t against its threshold
+        if (per_tile) {
+            thr32 = st[t].thr32;
+            thr64 = st[t].thr64;
         }
-        const bool keep = row_keep && (!L.colkeep || L.colkeep[c]);
-        w[e >> 2] |= (keep ? 1u : 0u) << ((e & 3) * 8);
+#pragma unroll
+        for (int r = 0; r < kFillRows; ++r) {
+            const float nv = r < nrows ? L.norms[(int64_t)t * L.K + k0 + r] : 0.0f;
+            row_keep[r] = r < nrows && (f64 ? (double)nv > thr64 : nv > thr32);
+        }
+    };
+    enter_tile();
+    uint32_t w[kFillRows][4];
+#pragma unroll
+    for (int r = 0; r < kFillRows; ++r)
+        w[r][0] = w[r][1] = w[r][2] = w[r][3] = 0u;
+    const int n = min(16, L.N - c0);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        if (e < n) {
+            const int c = c0 + e;
+            if (c >= t_end) {
+                ++t;
+                t_end = L.tcol0[t + 1];
+                enter_tile();
+            }
+            const bool col = !L.colkeep || L.colkeep[c];
+#pragma unroll
+            for (int r = 0; r < kFillRows; ++r)
+                w[r][e >> 2] |= (col && row_keep[r] ? 1u : 0u) << ((e & 3) * 8);
+        }
     }
-    uint8_t *dst = L.mask + (int64_t)k * L.N + c0;
-    if (n == 16 && (((uintptr_t)dst) & 15) == 0) {
-        uint4 v;
-        v.x = w[0];
-        v.y = w[1];
-        v.z = w[2];
-        v.w = w[3];
-        *reinterpret_cast<uint4 *>(dst) = v;
-    } else {
-        for (int e = 0; e < n; ++e)
-            dst[e] = (uint8_t)(w[e >> 2] >> ((e & 3) * 8));
+#pragma unroll
+    for (int r = 0; r < kFillRows; ++r) {
+        if (r >= nrows)
+            break;
+        uint8_t *dst = L.mask + (int64_t)(k0 + r) * L.N + c0;
+        if (n == 16 && (((uintptr_t)dst) & 15) == 0) {
+            uint4 v;
+            v.x = w[r][0];
+            v.y = w[r][1];
+            v.z = w[r][2];
+            v.w = w[r][3];
+            *reinterpret_cast<uint4 *>(dst) = v;
+        } else {
+            for (int e = 0; e < n; ++e)
+                dst[e] = (uint8_t)(w[r][e >> 2] >> ((e & 3) * 8));
+        }
     }
 }
 
@@ -738,7 +758,7 @@ int rows_stage(Arena &ar, int n_layers, const int32_t *K, const int32_t *N,
         e.rt_begin = n_pairs;
         e.el_begin = n_elems;
         n_pairs += (int64_t)e.K * e.n_tiles;
-        n_elems += (int64_t)e.K * ((e.N + 15) / 16);
+        n_elems += (int64_t)((e.K + kFillRows - 1) / kFillRows) * ((e.N + 15) / 16);
         std::memcpy(&pl[l], &e, sizeof(e));
         std::memcpy(flat + n_flat, lt[l].tcol0.data(), sizeof(int32_t) * lt[l].tcol0.size());
         n_flat += lt[l].tcol0.size();

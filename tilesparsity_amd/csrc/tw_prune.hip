@@ -282,6 +282,34 @@ __device__ void resolve_prefix(const SelectState *st, int npass, uint32_t &prefi
     }
 }
 
+// Calls f(value) for every element of v[0..n) once, the workgroups of blockIdx.x sharing the
+// work: 16-byte loads over the aligned middle (four of them in flight per thread), single
+// elements at the ragged ends.
+template <class F> __device__ __forceinline__ void for_each_value(const float *v, int64_t n, F f)
+{
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t nthr = (int64_t)gridDim.x * blockDim.x;
+    const int64_t head = min(n, (int64_t)((16 - ((uintptr_t)v & 15)) & 15) >> 2);
+    const int64_t nvec = (n - head) >> 2;
+    const float4 *v4 = reinterpret_cast<const float4 *>(v + head);
+    int64_t i = tid;
+    for (; i + 3 * nthr < nvec; i += 4 * nthr) {
+        const float4 a = v4[i], b = v4[i + nthr], c = v4[i + 2 * nthr], d = v4[i + 3 * nthr];
+        f(a.x); f(a.y); f(a.z); f(a.w);
+        f(b.x); f(b.y); f(b.z); f(b.w);
+        f(c.x); f(c.y); f(c.z); f(c.w);
+        f(d.x); f(d.y); f(d.z); f(d.w);
+    }
+    for (; i < nvec; i += nthr) {
+        const float4 a = v4[i];
+        f(a.x); f(a.y); f(a.z); f(a.w);
+    }
+    // the elements before the first and after the last whole vector
+    const int64_t tail0 = head + 4 * nvec;
+    for (int64_t j = tid; j < head + (n - tail0); j += nthr)
+        f(v[j < head ? j : tail0 + (j - head)]);
+}
+
 // hist[pass][d] += number of values whose key matches the digits fixed so far and has digit d
 // at bit 24 - 8 pass
 __global__ void __launch_bounds__(256)
@@ -297,12 +325,11 @@ __global__ void __launch_bounds__(256)
     resolve_prefix(st, pass, prefix, mask, rank, lost);
     __syncthreads(); // s_h is zeroed
     const int shift = 24 - 8 * pass;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-         i += (int64_t)gridDim.x * blockDim.x) {
-        const uint32_t key = sort_key(v[i]);
+    for_each_value(v, n, [&](float x) {
+        const uint32_t key = sort_key(x);
         if ((key & mask) == prefix)
             atomicAdd(&s_h[(key >> shift) & 255u], 1u);
-    }
+    });
     __syncthreads();
     if (s_h[threadIdx.x])
         atomicAdd(&st->hist[pass][threadIdx.x], (unsigned long long)s_h[threadIdx.x]);
@@ -319,14 +346,13 @@ __global__ void __launch_bounds__(256) rank_stats_kernel(const float *v, int64_t
     resolve_prefix(st, 4, key_a, mask, rank, lost);
     unsigned long long cnt = 0;
     unsigned int mn = 0xFFFFFFFFu;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-         i += (int64_t)gridDim.x * blockDim.x) {
-        const uint32_t key = sort_key(v[i]);
+    for_each_value(v, n, [&](float x) {
+        const uint32_t key = sort_key(x);
         if (key <= key_a)
             ++cnt;
         else
             mn = min(mn, key);
-    }
+    });
     // one pair of atomics per workgroup
     __shared__ unsigned long long s_cnt;
     __shared__ unsigned int s_min;
@@ -528,19 +554,58 @@ __device__ inline int find_mix_layer(const MixLayer *layers, int n_layers, int64
     return lo;
 }
 
+// Both mixed-mask kernels walk the pooled element numbering in groups of four: a group that lies
+// in one layer and is 16-byte aligned there moves as vectors, any other group element by element.
+struct MixGroup {
+    MixLayer L;
+    int64_t e;   // first element inside the layer
+    bool vec;
+};
+
+__device__ __forceinline__ MixGroup mix_group(const MixLayer *layers, int n_layers, int64_t total,
+                                              int64_t i)
+{
+    MixGroup g;
+    const int l = find_mix_layer(layers, n_layers, i);
+    g.L = layers[l];
+    g.e = i - g.L.begin;
+    const int64_t end = l + 1 < n_layers ? layers[l + 1].begin : total;
+    g.vec = i + 4 <= end && (((uintptr_t)(g.L.score + g.e)) & 15) == 0 &&
+            (((uintptr_t)(g.L.mask0 + g.e)) & 3) == 0 && (((uintptr_t)(g.L.out + g.e)) & 3) == 0;
+    return g;
+}
+
+__device__ __forceinline__ float mix_value(float x, uint8_t m0)
+{
+    const float sq = x * x;
+    const float nrm = sqrtf(sq) / 1.0f;
+    return nrm - (m0 ? 1.0f : 0.0f);
+}
+
 // pool[i] = ||x|| of the single element (sqrt(x*x) / 1, the reference's norm over a tile of one
 // column) minus 1 where the TW mask already keeps it (prune_algo.py:159-161)
 __global__ void __launch_bounds__(256)
     mix_values_kernel(const MixLayer *layers, int n_layers, int64_t total, float *pool)
 {
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const MixLayer L = layers[find_mix_layer(layers, n_layers, i)];
-        const int64_t e = i - L.begin;
-        const float x = L.score[e];
-        const float sq = x * x;
-        const float nrm = sqrtf(sq) / 1.0f;
-        pool[i] = nrm - (L.mask0[e] ? 1.0f : 0.0f);
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
+    for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < total; i += stride) {
+        const MixGroup g = mix_group(layers, n_layers, total, i);
+        if (g.vec) {
+            const float4 x = *reinterpret_cast<const float4 *>(g.L.score + g.e);
+            const uint32_t m = *reinterpret_cast<const uint32_t *>(g.L.mask0 + g.e);
+            float4 r;
+            r.x = mix_value(x.x, (uint8_t)(m & 255u));
+            r.y = mix_value(x.y, (uint8_t)((m >> 8) & 255u));
+            r.z = mix_value(x.z, (uint8_t)((m >> 16) & 255u));
+            r.w = mix_value(x.w, (uint8_t)(m >> 24));
+            *reinterpret_cast<float4 *>(pool + i) = r; // the pool is 256-byte aligned, i = 0 mod 4
+        } else {
+            for (int64_t j = i; j < min(i + 4, total); ++j) {
+                const MixLayer L = layers[find_mix_layer(layers, n_layers, j)];
+                const int64_t e = j - L.begin;
+                pool[j] = mix_value(L.score[e], L.mask0[e]);
+            }
+        }
     }
 }
 
@@ -551,13 +616,26 @@ __global__ void __launch_bounds__(256)
 {
     const float thr32 = st->thr32;
     const double thr64 = st->thr64;
-    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
-        const MixLayer L = layers[find_mix_layer(layers, n_layers, i)];
-        const int64_t e = i - L.begin;
-        const float v = pool[i];
-        const bool extra = f64 ? (double)v > thr64 : v > thr32;
-        L.out[e] = (L.mask0[e] || extra) ? 1 : 0;
+    auto above = [&](float v) { return f64 ? (double)v > thr64 : v > thr32; };
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x * 4;
+    for (int64_t i = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < total; i += stride) {
+        const MixGroup g = mix_group(layers, n_layers, total, i);
+        if (g.vec) {
+            const float4 v = *reinterpret_cast<const float4 *>(pool + i);
+            const uint32_t m = *reinterpret_cast<const uint32_t *>(g.L.mask0 + g.e);
+            uint32_t o = 0;
+            o |= ((m & 0x000000FFu) || above(v.x)) ? 0x00000001u : 0u;
+            o |= ((m & 0x0000FF00u) || above(v.y)) ? 0x00000100u : 0u;
+            o |= ((m & 0x00FF0000u) || above(v.z)) ? 0x00010000u : 0u;
+            o |= ((m & 0xFF000000u) || above(v.w)) ? 0x01000000u : 0u;
+            *reinterpret_cast<uint32_t *>(g.L.out + g.e) = o;
+        } else {
+            for (int64_t j = i; j < min(i + 4, total); ++j) {
+                const MixLayer L = layers[find_mix_layer(layers, n_layers, j)];
+                const int64_t e = j - L.begin;
+                L.out[e] = (L.mask0[e] || above(pool[j])) ? 1 : 0;
+            }
+        }
     }
 }
 
@@ -1079,7 +1157,7 @@ try {
         return fail(TW_ERR_ALLOC, "hipMalloc of %lld element scores failed", (long long)total);
     TW_HIP(hipMemcpyAsync(d_layers, ml.data(), sizeof(MixLayer) * n_layers, hipMemcpyHostToDevice, s));
     TW_HIP(hipStreamSynchronize(s)); // `ml` is pageable host memory
-    const unsigned grid = (unsigned)std::min<int64_t>((total + 255) / 256, 256 * 64);
+    const unsigned grid = (unsigned)std::min<int64_t>((total + 1023) / 1024, 256 * 32);
     hipLaunchKernelGGL(mix_values_kernel, dim3(grid), dim3(256), 0, s, d_layers, n_layers, total,
                        d_pool);
     TW_HIP(hipGetLastError());

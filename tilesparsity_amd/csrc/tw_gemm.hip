@@ -902,16 +902,19 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 float out_bias = 0.0f;
                 if (pt < BN)
                     out_col = u.col0 + p.kept_n[u.kn_off + (pt < u.n_cnt ? pt : 0)];
-                if (!preloaded) {
+                if (!preloaded && nsteps > 0) {
                     Idx ix[R];
 #pragma unroll
                     for (int j = 0; j < R; ++j)
                         load_idx(tc, j, ix[j]); // the padded list keeps every index load in bounds
                     load_idx(tc, R, ix_next);
+                    // Every register slot is loaded whether or not the item has that many steps
+                    // (the index list is padded, the weight step is clamped): the number of loads
+                    // in flight is then the same on every path into the slots below, and the
+                    // compiler can wait for exactly the loads a slot needs.
 #pragma unroll
                     for (int j = 0; j < R; ++j)
-                        if (j < nsteps)
-                            issue(tc, j, ix[j], a_ring[j], b_ring[j]);
+                        issue(tc, j < nsteps ? j : nsteps - 1, ix[j], a_ring[j], b_ring[j]);
                 }
                 TW_WS_PHASE(0, 256)
                 TW_WS_PHASE(1, 256)
@@ -966,12 +969,20 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                 // (the column numbers have arrived by now: the bias load flies over the last slots)
                 if (p.bias && pt < BN)
                     out_bias = p.bias[out_col];
-                for (; j0 < nsteps; j0 += R) {
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        if (j0 + r < nsteps)
-                            slot(j0 + r, r, j0 + r + R < nsteps);
-                }
+                // The last one to three slots, written out so that each knows at compile time
+                // whether it still fetches a step (a slot that decides this at run time makes the
+                // compiler wait for every load in flight before the first LDS write).
+                static_assert(R == 2, "the drain is written out for two register slots");
+                if (nsteps - j0 == 3) {
+                    slot(j0, 0, true);
+                    slot(j0 + 1, 1, false);
+                    slot(j0 + 2, 0, false);
+                } else if (nsteps - j0 == 2) {
+                    slot(j0, 0, false);
+                    slot(j0 + 1, 1, false);
+                } else if (nsteps - j0 == 1) {
+                    slot(j0, 0, false); // an item of one step
+                } // (a unit without kept rows has no step: its columns receive beta * C)
                 // last time slot: the multiplying waves work on the last step; the first loads of
                 // the next item start now and fly over the epilogue
                 const bool chain = nxt.ticket < p.n_pipe_items;
@@ -985,8 +996,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     load_idx(tn, R, ix_next);
 #pragma unroll
                     for (int j = 0; j < R; ++j)
-                        if (j < nn)
-                            issue(tn, j, ix[j], a_ring[j], b_ring[j]);
+                        issue(tn, j < nn ? j : nn - 1, ix[j], a_ring[j], b_ring[j]);
                 }
                 preloaded = chain;
                 if (pt < BN) {

@@ -27,7 +27,7 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 # HBM bytes per sparse launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
 # by what the same counter reads for a 256 MiB copy in the same run (reads x 2.0, writes x 1.0);
 # the runs and their commands are in profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md.
-MEASURED_TRAFFIC_BYTES = {"vgg16_conv4_2": (124316 + 11282) * 1024}
+MEASURED_TRAFFIC_BYTES = {"vgg16_conv4_2": (124334 + 11282) * 1024}
 
 
 def make_workload(name):

@@ -242,6 +242,33 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
                int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
                const tw_epilogue *ep, void *stream);
 
+/* Process-wide tuning switches of tw_gemm / tw_gemm_ex; value -1 restores the automatic choice.
+ * The launch configuration is otherwise picked from the plan and M.  The reference fixes its one
+ * configuration at compile time (Volta884GemmTraits<..., Shape<32,128,128>, ...>,
+ * basic_nn.cu:250-259, and MAX_BLOCK_NUM streams, :73); tests and tuning runs use these switches
+ * to cover every kernel shape.  A forced shape or piece width that cannot take the plan (a shape
+ * narrower than the plan's unit pieces, TW_SHAPE_WIDE aside operands beyond 4 GiB) is ignored.
+ *   TW_OPT_SHAPE        one of the TW_SHAPE_* kernels below
+ *   TW_OPT_WGS_PER_CU   workgroups launched per compute unit, 1..8
+ *   TW_OPT_PIECE        columns of a tile handed out as one work item: 128, 64 or 32
+ *   TW_OPT_XCD_QUEUES   1: one work queue per accelerator die, each owning whole row blocks of A
+ *                       (default); 0: the row blocks are dealt out over all queues
+ * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
+ * TWGEMM_PIECE and TWGEMM_XCD_QUEUES, read once. */
+#define TW_OPT_SHAPE 0
+#define TW_OPT_WGS_PER_CU 1
+#define TW_OPT_PIECE 2
+#define TW_OPT_XCD_QUEUES 3
+#define TW_N_OPTIONS 4
+#define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
+#define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
+#define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns */
+#define TW_SHAPE_128x64 3  /* wave-specialised, 128 x 64 */
+#define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU */
+#define TW_SHAPE_128x32 5  /* wave-specialised, 128 x 32: skinny M */
+#define TW_N_SHAPES 6
+int tw_set_option(int option, int value);
+
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument
  * meaning: A column-major M x K (lda = M), B the compacted stream weight, C
  * column-major M x N (ldc = M), all DEVICE memory of `dtype`; mask_n/mask_k host

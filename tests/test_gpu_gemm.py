@@ -422,26 +422,39 @@ def test_graph_capture_replays_bitwise(tw, oracle):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_every_kernel_shape_agrees(tw, oracle, dtype, monkeypatch):
-    """The launch picks one of five kernel shapes from the plan and M; TWGEMM_SHAPE forces each of
-    them in turn (wide tiles: 256x128, 128x128, wave-specialised 256x128; narrow tiles: 512x64,
-    256x64): all match the oracle, and each shape repeats itself bit for bit."""
+def test_every_kernel_shape_agrees(tw, oracle, dtype):
+    """The launch picks a kernel shape, the width of a unit piece and the queue layout from the
+    plan and M; tw_set_option forces each combination a plan can run with in turn: all match the
+    oracle, and each repeats itself bit for bit."""
     rng = np.random.default_rng(88)
-    for (M, K, N, G, shapes) in ((600, 320, 384, 128, (0, 1, 4)), (1100, 200, 256, 64, (2, 3))):
-        A = rng.standard_normal((M, K)).astype(np.float32)
-        B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
-        tiles = random_tiles(rng, K, N, G, k_keep=0.45, n_keep=0.85)
-        ref = reference(oracle, A, B, tiles, dtype)
-        keep = kept_columns(tiles, N)
-        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
-            for shape in shapes:
-                monkeypatch.setenv("TWGEMM_SHAPE", str(shape))
-                print("shape", shape, M, K, N, G, dtype, flush=True)
-                C1, bits1 = run_gemm(tw, oracle, plan, A, dtype, N)
-                C2, bits2 = run_gemm(tw, oracle, plan, A, dtype, N)
-                assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL[dtype], shape
-                assert np.array_equal(bits1, bits2), shape
-        monkeypatch.delenv("TWGEMM_SHAPE", raising=False)
+    W, S1, S2, S3, S4, S5 = (tw.SHAPE_WIDE, tw.SHAPE_128x128, tw.SHAPE_512x64, tw.SHAPE_128x64,
+                             tw.SHAPE_256x128, tw.SHAPE_128x32)
+    cases = (
+        (600, 320, 384, 128, ((W, -1), (S1, -1), (S4, -1), (S3, 64), (S5, 32), (S1, 64), (S4, 32))),
+        (1100, 200, 256, 64, ((S2, -1), (S3, -1), (S5, 32), (S1, -1), (S4, -1), (W, -1))),
+        (2500, 130, 96, 32, ((S5, -1), (S3, -1), (S2, -1))),
+    )
+    try:
+        for (M, K, N, G, combos) in cases:
+            A = rng.standard_normal((M, K)).astype(np.float32)
+            B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+            tiles = random_tiles(rng, K, N, G, k_keep=0.45, n_keep=0.85)
+            ref = reference(oracle, A, B, tiles, dtype)
+            keep = kept_columns(tiles, N)
+            with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+                for shape, piece in combos:
+                    for xcd in (1, 0):
+                        tw.set_option(tw.OPT_SHAPE, shape)
+                        tw.set_option(tw.OPT_PIECE, piece)
+                        tw.set_option(tw.OPT_XCD_QUEUES, xcd)
+                        print("shape", shape, "piece", piece, "xcd", xcd, M, K, N, G, dtype, flush=True)
+                        C1, bits1 = run_gemm(tw, oracle, plan, A, dtype, N)
+                        C2, bits2 = run_gemm(tw, oracle, plan, A, dtype, N)
+                        assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL[dtype], (shape, piece)
+                        assert np.array_equal(bits1, bits2), (shape, piece)
+    finally:
+        for opt in (tw.OPT_SHAPE, tw.OPT_PIECE, tw.OPT_XCD_QUEUES):
+            tw.set_option(opt, -1)
 
 
 def test_operand_beyond_four_gib(tw, oracle):

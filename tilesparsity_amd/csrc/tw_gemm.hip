@@ -26,7 +26,9 @@
 //     LDS, then scatter whole C columns (col0 + kept_n[j]) with 16-byte stores.
 #include "tw_internal.h"
 
+#include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <type_traits>
 #include <cstddef>
 #include <cstdlib>
@@ -124,6 +126,85 @@ __device__ __forceinline__ float tw_finish(float v, const float *bias, int c, in
     return tw_activate(v, act);
 }
 
+// ---------------------------------------------------------------------------------
+// Work queue (see GemmArgs): entry q of queue x names one item, or nothing past the end.
+enum ItemKind { ITEM_PIPE = 0, ITEM_NOSTEP = 1, ITEM_ZERO = 2, ITEM_END = 3 };
+
+struct Work {
+    int kind; // ItemKind
+    int u;    // column of the item matrix: piece of a unit, or n_gemm_u + tile to fill
+    int mb;   // row block
+};
+
+__device__ __forceinline__ int queue_length(const GemmArgs &p, int x)
+{
+    return p.n_own_items + (p.n_tail_items > x ? (p.n_tail_items - x + kXcd - 1) / kXcd : 0);
+}
+
+__device__ __forceinline__ Work queue_entry(const GemmArgs &p, int x, int q)
+{
+    Work w;
+    w.kind = ITEM_END;
+    w.u = 0;
+    w.mb = 0;
+    if (q < p.n_own_items) {
+        const int i = q / p.n_all_u;
+        w.u = q - i * p.n_all_u;
+        w.mb = x * p.n_own + i;
+    } else {
+        const int j = (q - p.n_own_items) * kXcd + x;
+        if (j >= p.n_tail_items)
+            return w;
+        w.u = j / p.n_tail_mblk;
+        w.mb = kXcd * p.n_own + (j - w.u * p.n_tail_mblk);
+    }
+    w.kind = w.u < p.n_pipe_u ? ITEM_PIPE : (w.u < p.n_gemm_u ? ITEM_NOSTEP : ITEM_ZERO);
+    return w;
+}
+
+// Piece `uv` of the unit table: unit uv / n_split, its columns [j * w, (j + 1) * w) with
+// w = 32 * piece_nb and j = uv % n_split.  A piece beyond the unit's columns keeps valid
+// offsets and has n_cnt == 0: it runs like any other and stores nothing.  The descriptor is
+// workgroup-uniform and ends up in scalar registers.
+__device__ __forceinline__ UnitDev load_unit(const GemmArgs &p, int uv)
+{
+    static_assert(sizeof(UnitDev) == 48, "UnitDev is read as 12 words");
+    const int ui = uv / p.n_split;
+    int32_t w[12];
+    if (p.n_arg_units) {
+        // from the kernel-argument segment: scalar loads, no global round trip
+        const auto *ka = (const __attribute__((address_space(4))) int32_t *)
+            __builtin_amdgcn_kernarg_segment_ptr();
+#pragma unroll
+        for (int i = 0; i < 12; ++i)
+            w[i] = ka[offsetof(GemmArgs, arg_units) / 4 + ui * 12 + i];
+    } else {
+        // the address is workgroup-uniform and the table is constant: scalar loads
+        const auto *gu = (const __attribute__((address_space(4))) int32_t *)(uintptr_t)(p.units + ui);
+#pragma unroll
+        for (int i = 0; i < 12; ++i)
+            w[i] = gu[i];
+    }
+#pragma unroll
+    for (int i = 0; i < 12; ++i)
+        w[i] = __builtin_amdgcn_readfirstlane(w[i]);
+    UnitDev u;
+    __builtin_memcpy(&u, w, sizeof(UnitDev));
+    if (p.n_split > 1) {
+        const int j = uv - ui * p.n_split;
+        const int bps = p.piece_nb; // 32-column blocks per piece
+        const int nb = min(max(u.nb_cnt - j * bps, 0), bps);
+        const int nc = min(max(u.n_cnt - j * bps * kMfmaN, 0), bps * kMfmaN);
+        if (nb > 0) {
+            u.nb0 += j * bps;
+            u.kn_off += j * bps * kMfmaN;
+        }
+        u.nb_cnt = nb;
+        u.n_cnt = nc;
+    }
+    return u;
+}
+
 // WM x WN waves of 64 x 64 outputs each: workgroup tile BM = 64*WM rows by BN = 64*WN
 // compact columns.  WGS is the number of workgroups meant to share a CU.
 // BK k rows are staged per main-loop step (a multiple of 16 that divides kBlockK); the loads
@@ -155,21 +236,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 
     __shared__ __align__(16) uint16_t smem[SMEM];
     __shared__ int s_tk[2];
-    // Instrumented builds only (-DTW_EXP_TIMING): workgroup 0 records cycle stamps of its steps
-    // and phases in LDS and copies them behind the ticket slots, where tw_exp_read_debug reads
-    // them.  Not part of the shipped library.
-#ifdef TW_EXP_TIMING
-    __shared__ unsigned long long s_ts[64 * 4];
-#define TW_STAMP(step, slot)                                                              \
-    if (item == 0 && tid == 0 && (step) >= 8 && (step) < 72)                              \
-        s_ts[((step)-8) * 4 + (slot)] = __builtin_readcyclecounter();
-#define TW_PHASE(k)                                                                       \
-    if (blockIdx.x == 0 && tid == 0 && n_done_items < 2)                                  \
-        s_ts[240 + n_done_items * 8 + (k)] = __builtin_readcyclecounter();
-#else
-#define TW_STAMP(step, slot)
-#define TW_PHASE(k)
-#endif
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -185,25 +251,26 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     uint16_t *const sB = smem + 2 * ASTAGE;
 
     // ---- work items ----------------------------------------------------------------
-    // A ticket names an item: tickets below n_pipe_items are GEMM items with at least one
-    // step, then come GEMM items of units that keep no K row (their kept columns receive
-    // alpha*0 + beta*C), then the zero-fill items.  The workgroup always holds the ticket
-    // of its current and its next item and has the atomic for the one after in flight, so
-    // a ticket's round trip is hidden behind a whole item.
+    // A ticket is an index into this workgroup's queue: GEMM items with at least one step,
+    // GEMM items of units that keep no K row (their kept columns receive alpha*0 + beta*C)
+    // and zero-fill items.  The workgroup always holds the ticket of its current and its next
+    // item and has the atomic for the one after in flight, so a ticket's round trip is hidden
+    // behind a whole item.
+    const int qx = blockIdx.x % kXcd;
+    const int qlen = queue_length(p, qx);
+    // (an item is told by its column of the item matrix, compared with the bounds each time)
     struct Item {
-        int ticket;
+        int col;
         int m0;
-        UnitDev u; // valid for ticket < n_gemm_items
+        UnitDev u; // col < n_gemm_u
     };
     auto make_item = [&](int ticket) {
         Item it;
-        it.ticket = ticket;
-        it.m0 = 0;
-        if (ticket < p.n_gemm_items) {
-            const int ui = ticket / p.n_mblk;
-            it.m0 = (ticket - ui * p.n_mblk) * BM;
-            it.u = p.units[ui];
-        }
+        const Work w = queue_entry(p, qx, ticket);
+        it.col = w.kind == ITEM_END ? p.n_all_u : w.u;
+        it.m0 = w.mb * BM;
+        if (it.col < p.n_gemm_u)
+            it.u = load_unit(p, it.col);
         return it;
     };
     // per-thread addressing of an item
@@ -272,13 +339,19 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     // The first item of a workgroup is its block index; later ones are claimed from the
     // shared counter (which starts at 0 for every launch) one item ahead, with the atomic of
     // the claim after that already in flight.
-    const int ticket_base = gridDim.x;
+    const int ticket_base = gridDim.x / kXcd; // workgroups per queue
     int t_pending = 0;   // thread 0: claim in flight
     bool closed = false; // thread 0: the queue is exhausted, no claim is in flight
     int t_done = -1;     // thread 0: workgroups counted as done before this one
-    if (tid == 0)
-        t_pending = atomicAdd(&p.ticket[0], 1);
-    Item cur = make_item(blockIdx.x);
+    if (tid == 0) {
+        if ((int)(blockIdx.x / kXcd) < qlen) {
+            t_pending = atomicAdd(&p.ticket[qx], 1);
+        } else { // nothing for this workgroup: it only counts itself as done
+            closed = true;
+            t_done = atomicAdd(&p.ticket[kXcd], 1);
+        }
+    }
+    Item cur = make_item(blockIdx.x / kXcd);
     Item nxt = cur;
     bool have_next = false; // nxt is known for the current item
     // Publishes the claim in flight as the next item and starts the claim after it.  A ticket
@@ -287,14 +360,14 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     // leaves) and that count's round trip is over before the item ends.
     auto claim_next = [&]() {
         if (tid == 0) {
-            const int t = closed ? p.n_items : ticket_base + t_pending;
+            const int t = closed ? qlen : ticket_base + t_pending;
             s_tk[0] = t;
             if (!closed) {
-                if (t < p.n_items) {
-                    t_pending = atomicAdd(&p.ticket[0], 1);
+                if (t < qlen) {
+                    t_pending = atomicAdd(&p.ticket[qx], 1);
                 } else {
                     closed = true;
-                    t_done = atomicAdd(&p.ticket[1], 1);
+                    t_done = atomicAdd(&p.ticket[kXcd], 1);
                 }
             }
         }
@@ -307,21 +380,16 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     bool preloaded = false; // cur's first D steps are already in flight, i_ring holds D..2D-1
 
     bool first = true;
-    int n_done_items = 0;
-    while (cur.ticket < p.n_items) {
-        const int item = cur.ticket;
-        TW_PHASE(0)
+    while (cur.col < p.n_all_u) {
         // the very first claim of a workgroup is published after the first item's loads have
         // been issued, so that its round trip overlaps with them
-        if (!first || item >= p.n_pipe_items)
+        if (!first || cur.col >= p.n_pipe_u)
             claim_next();
         first = false;
-        if (item >= p.n_gemm_items) {
+        if (cur.col >= p.n_gemm_u) {
             // ---- zero-fill item: pruned columns of one tile receive beta*C ----
-            const int z = item - p.n_gemm_items;
-            const int zt = z / p.n_mblk;
-            const int m = (z - zt * p.n_mblk) * BM + chunk * 8;
-            const TileDev t = p.tiles[zt];
+            const int m = cur.m0 + chunk * 8;
+            const TileDev t = p.tiles[cur.col - p.n_gemm_u];
             for (int j = rrow; j < t.n_pruned; j += RPP) {
                 const int c = t.col0 + p.pruned_n[t.pn_off + j];
                 uint16_t *dst = C + (int64_t)c * p.ldc + m;
@@ -418,11 +486,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                     load_idx(tc, s + 2 * D, i_ring[(r + 2 * D) % R]); // padded list: in bounds
                     issue(tc, s + D, i_ring[(r + D) % R], a_ring[(r + D) % R], b_ring[(r + D) % R]);
                 }
-                TW_STAMP(s, 0)
                 stage(s, a_ring[r], b_ring[r]);
-                TW_STAMP(s, 1)
                 __syncthreads();
-                TW_STAMP(s, 2)
 #pragma unroll
                 for (int ks = 0; ks < KS; ++ks) {
                     frags(s, ks, af, bf);
@@ -432,7 +497,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                         for (int mi = 0; mi < 2; ++mi)
                             acc[mi][ni] = E::mfma(af[mi], bf[ni], acc[mi][ni]);
                 }
-                TW_STAMP(s, 3)
             };
 
             if (!preloaded) {
@@ -447,10 +511,8 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                     }
                 }
             }
-            TW_PHASE(1)
             if (!have_next)
                 claim_next();
-            TW_PHASE(2)
             int s0 = 0;
             // steady state: every iteration issues, stages and multiplies, no conditionals
             for (; s0 + R + D <= nsteps; s0 += R) {
@@ -460,7 +522,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
             }
             // The next item's index words are fetched before the drain, so that its first row
             // loads can be issued right after this item's last step and fly over the epilogue.
-            const bool chain = nxt.ticket < p.n_pipe_items;
+            const bool chain = nxt.col < p.n_pipe_u;
             Thr tn;
             if (chain) {
                 tn = setup(nxt);
@@ -478,7 +540,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 }
             }
             __syncthreads();
-            TW_PHASE(3)
             if (chain) {
                 const int nn = nxt.u.k_pad / BK;
 #pragma unroll
@@ -489,7 +550,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 }
             }
             preloaded = chain;
-            TW_PHASE(4)
 
             // ---- epilogue --------------------------------------------------------
             const int32_t *const nlist = p.kept_n + u.kn_off;
@@ -535,7 +595,6 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
                 }
             }
             __syncthreads();
-            TW_PHASE(5)
             for (int j = rrow; j < u.n_cnt; j += RPP) {
                 const int c = u.col0 + nlist[j];
                 // rows of the staging tile are 8-byte aligned only: two 8-byte reads
@@ -550,26 +609,19 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
             }
         }
 
-        TW_PHASE(6)
         __syncthreads();
-        TW_PHASE(7)
         cur = nxt;
         have_next = false;
-        ++n_done_items;
     }
 
-#ifdef TW_EXP_TIMING
-    __syncthreads();
-    if (blockIdx.x == 0 && tid < 256)
-        reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ts[tid];
-#endif
     // the workgroup counted last re-arms the ticket slot for the next launch: every workgroup's
     // claims had returned before it was counted.  Plain stores, made visible by the end of the
     // kernel; a device-scope fence here would write back and invalidate this XCD's L2 under the
     // workgroups that still stream through it.
     if (tid == 0 && t_done == (int)gridDim.x - 1) {
-        p.ticket[0] = 0;
-        p.ticket[1] = 0;
+#pragma unroll
+        for (int i = 0; i <= kXcd; ++i)
+            p.ticket[i] = 0;
     }
 }
 
@@ -579,56 +631,47 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 #define TW_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 // ---------------------------------------------------------------------------------
-// Wave-specialised 256 x 128 kernel (8 waves, one workgroup per CU).  Waves 0-3 only multiply:
-// wave w owns rows 64w..64w+63 of the row block and all 128 compact columns (2 x 4 MFMA
-// blocks, 128 accumulator registers).  Waves 4-7 only move data: they gather the kept rows of
-// A and the packed weight global -> registers -> LDS, R steps of 64 rows in flight.  Both
-// halves meet at one barrier per step: while the multiplying waves read stage s & 1, the
-// moving waves fill stage (s + 1) & 1, so LDS traffic, vector-memory traffic and MFMA work
-// overlap instead of following each other.  One multiplying and one moving wave share a SIMD.
-// Work items, tickets, the chained first loads of the next item and the epilogue are those of
-// tw_gemm_kmajor_kernel.
-template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(const GemmArgs p)
+// Wave-specialised BM x BN kernel.  Half of the waves only multiply: multiplying wave w owns
+// rows [w * RW, (w + 1) * RW) of the row block and all BN compact columns (MI x NI MFMA blocks
+// of 32 x 32).  The other half only move data: they gather the kept rows of A and the packed
+// weight global -> registers -> LDS, R steps of 64 rows in flight.  Both halves meet at one
+// barrier per step: while the multiplying waves read stage s & 1, the moving waves fill stage
+// (s + 1) & 1, so LDS traffic, vector-memory traffic and MFMA work overlap instead of following
+// each other.  One multiplying and one moving wave share a SIMD.
+//   BM = 128: 2 + 2 waves, two or more workgroups per CU (one's start-up and epilogue hide
+//             under the other's steps: the shape for items of few steps);
+//   BM = 256: 4 + 4 waves, one workgroup per CU (half the weight traffic per row of A);
+//   BM = 512: 4 + 4 waves, each multiplying wave 128 rows (tiles of at most 64 kept columns).
+// The first loads of the next item are issued during the last step of the current one and
+// fly over its epilogue.
+template <int DT, int BM, int BN>
+__global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(const GemmArgs p)
 {
-    constexpr int NT = 512, NP = 256, BM = 256, BN = 128, BK = 64;
+    constexpr int NMW = BM == 128 ? 2 : 4;     // multiplying waves, and as many moving waves
+    constexpr int NPM = 64 * NMW;              // threads of either half
+    constexpr int NT = 2 * NPM;
+    constexpr int BK = 64;
     constexpr int KS = BK / kMfmaK, PKS = kBlockK / kMfmaK;
     constexpr int R = 2;                       // register slots = steps of loads in flight
-    constexpr int MI = 2, NI = 4;
+    constexpr int RW = BM / NMW;               // rows of a multiplying wave
+    constexpr int MI = RW / 32, NI = BN / kMfmaN;
     constexpr int CPR = BM / 8;                // 16-byte chunks per staged A row / stored C column
-    constexpr int RPP = NP / CPR;              // A rows covered by one pass of the moving waves
-    constexpr int PASSES = BK / RPP;           // A loads per moving thread and step
-    constexpr int BPASS = BN * BK / 8 / NP;    // weight loads per moving thread and step
+    constexpr int RG = 64 / CPR;               // rows a moving wave covers with one load
+    constexpr int RPW = BK / NMW;              // rows of a step per moving wave
+    constexpr int PASSES = RPW / RG;           // A loads per moving thread and step
+    constexpr int BPASS = BN * BK / 8 / NPM;   // weight loads per moving thread and step
     constexpr int PITCH = BM + TW_A_PAD;
     constexpr int ASTAGE = BK * PITCH, BSTAGE = BN * BK;
     constexpr int CPITCH = BM + 4;
     constexpr int PIPE = 2 * (ASTAGE + BSTAGE);
     constexpr int SMEM = PIPE > BN * CPITCH ? PIPE : BN * CPITCH;
     static_assert(BK == kBlockK && KS == PKS, "one packed weight step per main-loop step");
+    static_assert(CPR <= 64 && PASSES % 4 == 0 && BPASS >= 1 && BN <= NPM, "tile shape");
     using E = Elem<DT>;
 
     __shared__ __align__(16) uint16_t smem[SMEM];
     __shared__ int s_tk[2];
     __shared__ int s_cols[BN];   // output columns of the current item's unit
-    __shared__ float s_bias[BN]; // ... and their bias values (fused epilogue)
-    // Instrumented builds only (-DTW_EXP_TIMING=1: cycle stamps of workgroup 0's item number
-    // TW_EXP_ITEM; =2: start and end time of every workgroup), read back with tw_exp_read_debug.
-#ifdef TW_EXP_TIMING
-    __shared__ unsigned long long s_ws[256];
-#ifndef TW_EXP_ITEM
-#define TW_EXP_ITEM 0
-#endif
-    int ws_item = 0;
-#define ws_first (ws_item == TW_EXP_ITEM)
-#define TW_WS_STAMP(step, k, t)                                                          \
-    if (blockIdx.x == 0 && ws_first && threadIdx.x == (t) && (step) < 30)               \
-        s_ws[(step)*8 + (k)] = __builtin_readcyclecounter();
-#define TW_WS_PHASE(k, t)                                                                \
-    if (blockIdx.x == 0 && ws_first && threadIdx.x == (t))                               \
-        s_ws[240 + (k)] = __builtin_readcyclecounter();
-#else
-#define TW_WS_STAMP(step, k, t)
-#define TW_WS_PHASE(k, t)
-#endif
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -639,63 +682,55 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     uint16_t *const sA = smem;
     uint16_t *const sB = smem + 2 * ASTAGE;
 
+    // this workgroup's queue
+    const int qx = blockIdx.x % kXcd;
+    const int qi = blockIdx.x / kXcd;        // position among the queue's workgroups
+    const int qwg = gridDim.x / kXcd;        // workgroups per queue
+    const int qlen = queue_length(p, qx);
+
+    // An item is told by its column of the item matrix: below n_pipe_u a GEMM item with steps,
+    // below n_gemm_u one without, below n_all_u a tile to fill, n_all_u past the end.  (The
+    // tests below compare the column with these bounds each time, rather than a kind worked out
+    // once: with the latter the compiler threads the item loop into copies that each keep their
+    // own set of load registers.)
     struct Item {
-        int ticket;
+        int col;
         int m0, m_end; // rows [m0, m_end) of A and C, at most BM of them
-        UnitDev u;     // valid for ticket < n_gemm_items
+        UnitDev u;     // col < n_gemm_u
     };
     auto make_item = [&](int ticket) {
         Item it;
-        it.ticket = ticket;
-        it.m0 = 0;
-        it.m_end = 0;
-        if (ticket < p.n_gemm_items) {
-            const auto *ka = (const __attribute__((address_space(4))) int32_t *)
-                __builtin_amdgcn_kernarg_segment_ptr();
-            const int ui = ticket / p.n_mblk;
-            it.m0 = (ticket - ui * p.n_mblk) * BM;
-            it.m_end = it.m0 + BM < p.M ? it.m0 + BM : p.M;
-            static_assert(sizeof(UnitDev) == 48, "UnitDev is read as 12 words");
-            int32_t w[12];
-            if (p.n_arg_units) {
-                // from the kernel-argument segment: scalar loads, no global round trip
-#pragma unroll
-                for (int i = 0; i < 12; ++i)
-                    w[i] = ka[offsetof(GemmArgs, arg_units) / 4 + ui * 12 + i];
-            } else {
-                __builtin_memcpy(w, &p.units[ui], sizeof(UnitDev));
-            }
-            // the descriptor is workgroup-uniform: keep it, and all derived from it, scalar
-#pragma unroll
-            for (int i = 0; i < 12; ++i)
-                w[i] = __builtin_amdgcn_readfirstlane(w[i]);
-            __builtin_memcpy(&it.u, w, sizeof(UnitDev));
-        }
+        const Work w = queue_entry(p, qx, ticket);
+        it.col = w.kind == ITEM_END ? p.n_all_u : w.u;
+        it.m0 = w.mb * BM;
+        it.m_end = it.m0 + BM < p.M ? it.m0 + BM : p.M;
+        if (it.col < p.n_gemm_u)
+            it.u = load_unit(p, it.col);
         return it;
     };
+    auto is_end = [&](const Item &it) { return it.col >= p.n_all_u; };
+    auto has_steps = [&](const Item &it) { return it.col < p.n_pipe_u; };
+    auto is_fill = [&](const Item &it) { return it.col >= p.n_gemm_u; };
     // Both halves of the workgroup walk the same item sequence and execute the same sequence
     // of barriers; thread 0 (a multiplying wave) owns the ticket counter.
-#ifdef TW_EXP_TIMING
-    if (blockIdx.x == 0 && tid == 0) {
-        s_ws[248] = __builtin_readcyclecounter();
-        s_ws[249] = __builtin_amdgcn_s_memrealtime();
-    }
-#if TW_EXP_TIMING == 2
-    if (tid == 0 && blockIdx.x < 256)
-        reinterpret_cast<unsigned *>(p.dbg)[blockIdx.x * 2] = (unsigned)__builtin_amdgcn_s_memrealtime();
-#endif
-#endif
-    // The first two items of a workgroup are fixed (block index, block index + grid size), so
+    // The first two items of a workgroup are fixed (entries qi and qi + qwg of its queue), so
     // that no atomic's round trip sits between the start of the kernel and the first loads;
-    // the shared counter hands out the items after those.
-    const int ticket_base = 2 * gridDim.x;
-    int t_pending = 0;                     // thread 0: result of the claim in flight
-    int t_next = gridDim.x + blockIdx.x;   // thread 0: the next ticket once known, or -1
+    // the queue's counter hands out the entries after those.
+    const int ticket_base = 2 * qwg;
+    int t_pending = 0;      // thread 0: result of the claim in flight
+    int t_next = qi + qwg;  // thread 0: the next ticket once known, or -1
     bool closed = false;    // thread 0: no claim of this workgroup is in flight, none will follow
     bool announced = false; // thread 0: the workgroup has been counted as done with the counter
     int t_done = -1;        // thread 0: workgroups counted before this one (atomic's result)
-    if (tid == 0)
-        t_pending = atomicAdd(&p.ticket[0], 1);
+    if (tid == 0) {
+        if (qi < qlen) {
+            t_pending = atomicAdd(&p.ticket[qx], 1);
+        } else { // nothing for this workgroup: it only counts itself as done
+            closed = true;
+            announced = true;
+            t_done = atomicAdd(&p.ticket[kXcd], 1);
+        }
+    }
     // Picks up the claim in flight and starts the one after it, unless the queue is exhausted.
     // Called before an item's output stores are issued: memory operations complete in order, so
     // waiting for an atomic issued after them (or overwriting its register) would wait for the
@@ -703,12 +738,12 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     auto pick_up = [&]() {
         if (tid == 0 && t_next < 0) {
             if (closed) {
-                t_next = p.n_items;
+                t_next = qlen;
             } else {
                 t_next = ticket_base + t_pending;
                 asm volatile("" : "+v"(t_next)); // here, not where it is published
-                if (t_next < p.n_items)
-                    t_pending = atomicAdd(&p.ticket[0], 1);
+                if (t_next < qlen)
+                    t_pending = atomicAdd(&p.ticket[qx], 1);
                 else
                     closed = true;
             }
@@ -719,13 +754,13 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     // counts itself as done with the counter right away and the count's round trip is over long
     // before the item ends; the workgroup counted last re-arms the slot when it leaves.
     auto announce = [&]() {
-        if (t_next >= p.n_items && !announced) {
+        if (t_next >= qlen && !announced) {
             if (!closed) {
                 // the second fixed item is already past the end: the first claim is in flight
                 asm volatile("" ::"v"(t_pending));
                 closed = true;
             }
-            t_done = atomicAdd(&p.ticket[1], 1);
+            t_done = atomicAdd(&p.ticket[kXcd], 1);
             announced = true;
         }
     };
@@ -741,30 +776,16 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
     };
     auto published = [&]() { return make_item(__builtin_amdgcn_readfirstlane(s_tk[0])); };
     auto claim = [&]() { // two barriers of its own: items without steps
-        if (tid == 0) {
-            pick_up();
-            s_tk[0] = t_next;
-            announce();
-            t_next = -1;
-        }
-        TW_WS_STAMP(0, 6, 256)
+        publish();
         TW_LDS_BARRIER();
-        TW_WS_STAMP(0, 7, 256)
-        const Item it = make_item(__builtin_amdgcn_readfirstlane(s_tk[0]));
-#ifdef TW_EXP_TIMING
-        if (it.u.k_pad >= 0)
-            TW_WS_STAMP(1, 6, 256)
-#endif
+        const Item it = published();
         TW_LDS_BARRIER();
-        TW_WS_STAMP(1, 7, 256)
         return it;
     };
     // zero-fill item: pruned columns of one tile receive beta*C (all threads, no barrier)
-    auto zero_fill = [&](int item) {
-        const int z = item - p.n_gemm_items;
-        const int zt = z / p.n_mblk;
-        const int m = (z - zt * p.n_mblk) * BM + (tid % CPR) * 8;
-        const TileDev t = p.tiles[zt];
+    auto zero_fill = [&](const Item &it) {
+        const int m = it.m0 + (tid % CPR) * 8;
+        const TileDev t = p.tiles[it.col - p.n_gemm_u];
         for (int j = tid / CPR; j < t.n_pruned; j += NT / CPR) {
             const int c = t.col0 + p.pruned_n[t.pn_off + j];
             uint16_t *dst = C + (int64_t)c * p.ldc + m;
@@ -784,7 +805,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         }
     };
     // scatters the staged C tile (all threads): whole columns col0 + kept_n[j], 16-byte stores
-    // (the output columns col0 + kept_n[j] come from s_cols, filled by the moving waves)
+    // (the output columns come from s_cols, filled by the first multiplying wave)
     auto store_tile = [&](const UnitDev &u, int m0, int m_end) {
         const int m_st = m0 + (tid % CPR) * 8;
         for (int j = tid / CPR; j < u.n_cnt; j += NT / CPR) {
@@ -801,236 +822,190 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
         }
     };
 
-    if (wave >= 4) {
+    if (wave >= NMW) {
         // ================= moving waves ===================================================
-        // Thread pt moves chunk pt % 32 (8 consecutive m) of the rows 8 * (pt / 32) .. + 7 of a
-        // step: a wave covers 16 consecutive kept rows, whose indices it fetches with one
-        // scalar load.  Addresses are a uniform base plus a 32-bit byte offset per lane.
-        const int pt = tid - NP;
-        const int chunk = pt % CPR, rgrp = pt / CPR;
-        const bool upper = (lane >> 5) != 0;           // second row group of this wave
-        const int mw = wave - 4;
+        // A load of a wave covers RG kept rows (CPR lanes of 16 bytes each per row); lane
+        // (g, chunk) moves chunk `chunk` (8 consecutive m) of the rows
+        // mw * RPW + g * PASSES + 0 .. PASSES - 1 of a step.  The lane fetches the indices of its
+        // own rows (a 16-byte load per four rows, the lanes of a row group share the address)
+        // one step before the row loads that use them.  Row addresses are a uniform base plus a
+        // 32-bit byte offset per lane.
+        const int pt = tid - NPM;
+        const int chunk = lane % CPR, g = lane / CPR;
+        const int mw = wave - NMW;
+        const int row0 = mw * RPW + g * PASSES;        // this lane's first row of a step
         const uint32_t lda_b = (uint32_t)p.lda * 2u;   // bytes; K * lda * 2 < 2^32 (host check)
-        typedef int i32x16 __attribute__((ext_vector_type(16)));
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
         struct Idx {
-            int k[16];
+            i32x4 k[PASSES / 4];
         };
+        const uint32_t v_idx = (uint32_t)row0 * 4u;    // byte offset of this lane's indices in a step
+        const uint32_t v_b = (uint32_t)(pt & 255) * 16u; // ... of its 16-byte piece in a weight block
+        // every address is a workgroup-uniform base plus a 32-bit byte offset per lane
         struct Thr {
-            const int32_t *klist;   // + 16 * mw: this wave's rows of step 0
+            const char *k_base;     // the unit's kept-K list (bytes), uniform
             const char *a_base;     // A + m0 (bytes), uniform
-            const char *b_base[BPASS];
+            const char *b_base[BPASS]; // weight block of load bp in step 0, uniform
             int64_t b_pack_b;
             uint32_t v_chunk;       // byte offset of this lane's chunk inside a gathered row
             bool m_ok;
         };
         auto setup = [&](const Item &it) {
             Thr t;
-            t.klist = p.kept_k + it.u.kk_off + 16 * mw; // padded past k_pad
+            t.k_base = reinterpret_cast<const char *>(p.kept_k + it.u.kk_off); // padded past k_pad
             t.a_base = reinterpret_cast<const char *>(A + it.m0);
             t.m_ok = it.m0 + chunk * 8 < it.m_end;
             t.v_chunk = t.m_ok ? chunk * 16 : 0; // beyond the row block: re-read its first chunk
-            // weight chunk c = pt + bp * NP of a step is (nb = bp, k16 = pt / 64, lane = pt % 64);
-            // a block beyond the unit reads block 0 (its products are never stored)
+            // weight chunk c = pt + bp * NPM of a step is (nb = c / 256, k16 = (c / 64) % 4,
+            // lane = c % 64), i.e. 16-byte piece c % 256 of block nb; a block beyond the unit
+            // reads block 0 (its products are never stored)
 #pragma unroll
-            for (int bp = 0; bp < BPASS; ++bp)
-                t.b_base[bp] = reinterpret_cast<const char *>(
-                    Bp + it.u.b_off + (int64_t)(it.u.nb0 + (bp < it.u.nb_cnt ? bp : 0)) * (PKS * 64 * 8));
+            for (int bp = 0; bp < BPASS; ++bp) {
+                const int nb = (bp * NPM) / 256 < it.u.nb_cnt ? (bp * NPM) / 256 : 0;
+                t.b_base[bp] = reinterpret_cast<const char *>(Bp + it.u.b_off) +
+                               ((int64_t)(it.u.nb0 + nb) * 256 + ((bp * NPM) & 255)) * 16;
+            }
             t.b_pack_b = (int64_t)it.u.nblk * (PKS * 64 * 8 * 2);
             return t;
         };
         auto load_idx = [&](const Thr &t, int s, Idx &ix) {
-            const i32x16 v = *reinterpret_cast<const __attribute__((address_space(4))) i32x16 *>(
-                (uintptr_t)(t.klist + s * BK));
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                ix.k[i] = v[i];
-                asm volatile("" : "+s"(ix.k[i])); // keep the words scalar and the load whole
+            for (int i = 0; i < PASSES / 4; ++i)
+                ix.k[i] = *reinterpret_cast<const i32x4 *>(t.k_base + (int64_t)s * (BK * 4) + 16 * i + v_idx);
+        };
+        // (`live` is all ones, or zero for a refill that fetches nothing: row 0, chunk 0)
+        auto load_a = [&](const Thr &t, const Idx &ix, int ps, uint32_t live, uint32_t vc) {
+            const uint32_t off = ((uint32_t)ix.k[ps >> 2][ps & 3] & live) * lda_b + vc;
+            return *reinterpret_cast<const u32x4 *>(t.a_base + off);
+        };
+        auto load_b = [&](const Thr &t, int s, int bp, uint32_t vb) {
+            return *reinterpret_cast<const u32x4 *>(t.b_base[bp] + (int64_t)s * t.b_pack_b + vb);
+        };
+        // The item loop is rotated: an iteration first starts the loads of its item, then finishes
+        // the item before it (the two barriers around the staged C tile, this half's share of the
+        // stores), then runs its item's time slots.  So the first loads of an item fly over the
+        // epilogue of its predecessor, and the load registers live within one iteration only
+        // (carried around the loop, the compiler keeps them in two register sets and copies one
+        // into the other, waiting for the loads in flight).
+        Item cur = make_item(qi);
+        Item nxt = cur, prev = cur;
+        bool have_next = false, have_prev = false;
+        for (;;) {
+            u32x4 a_ring[R][PASSES];
+            u32x4 b_ring[R][BPASS];
+            Idx ix_next; // row indices of the step issued next
+            const Thr tc = setup(cur);
+            const int nsteps = has_steps(cur) ? cur.u.k_pad / BK : 0;
+            if (nsteps > 0) {
+                // First loads: weight and rows of steps 0 and 1, the index loads one step ahead,
+                // in the order the time slots keep up.  Both register slots are loaded whether or
+                // not the item has two steps (the index list is padded, the weight step is
+                // clamped), like every slot below refills its registers whether or not a step is
+                // left to fetch: the sequence of loads is then the same on every path and the
+                // compiler can wait for exactly the loads a slot needs.
+                Idx ix0, ix1;
+                load_idx(tc, 0, ix0);
+                load_idx(tc, 1, ix1);
+#pragma unroll
+                for (int bp = 0; bp < BPASS; ++bp)
+                    b_ring[0][bp] = load_b(tc, 0, bp, v_b);
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps)
+                    a_ring[0][ps] = load_a(tc, ix0, ps, 0xFFFFFFFFu, tc.v_chunk);
+                load_idx(tc, 2, ix_next);
+#pragma unroll
+                for (int bp = 0; bp < BPASS; ++bp)
+                    b_ring[1][bp] = load_b(tc, nsteps > 1 ? 1 : 0, bp, v_b);
+#pragma unroll
+                for (int ps = 0; ps < PASSES; ++ps)
+                    a_ring[1][ps] = load_a(tc, ix1, ps, 0xFFFFFFFFu, tc.v_chunk);
             }
-        };
-        auto load_a = [&](const Thr &t, const Idx &ix, int ps) {
-            uint32_t o0 = (uint32_t)ix.k[ps] * lda_b, o1 = (uint32_t)ix.k[8 + ps] * lda_b;
-            asm volatile("" : "+s"(o0), "+s"(o1)); // multiply on the scalar unit, select afterwards
-            return *reinterpret_cast<const u32x4 *>(t.a_base + ((upper ? o1 : o0) + t.v_chunk));
-        };
-        auto load_b = [&](const Thr &t, int s, int bp) {
-            return *reinterpret_cast<const u32x4 *>(t.b_base[bp] + (int64_t)s * t.b_pack_b +
-                                                    (uint32_t)(pt * 16));
-        };
-        auto issue = [&](const Thr &t, int s, const Idx &ix, u32x4(&ar)[PASSES], u32x4(&br)[BPASS]) {
-#pragma unroll
-            for (int ps = 0; ps < PASSES; ++ps)
-                ar[ps] = load_a(t, ix, ps);
-#pragma unroll
-            for (int bp = 0; bp < BPASS; ++bp)
-                br[bp] = load_b(t, s, bp);
-        };
-        u32x4 a_ring[R][PASSES];
-        u32x4 b_ring[R][BPASS];
-        Idx ix_next;            // row indices of the step issued next
-        bool preloaded = false; // cur's first R steps are in flight, ix_next is that of step R
-
-        TW_WS_PHASE(6, 256)
-        Item cur = make_item(blockIdx.x);
-        Item nxt = cur;
-        bool have_next = false;
-#ifdef TW_EXP_TIMING
-        if (cur.u.k_pad >= 0)
-            TW_WS_PHASE(7, 256)
-#endif
-        while (cur.ticket < p.n_items) {
-            const int item = cur.ticket;
-#if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
-            TW_WS_PHASE(6, 256)
-#endif
-            if (item >= p.n_pipe_items) { // no step, no pipeline barrier to ride on
+            if (have_prev) {
+                if (!is_fill(prev)) {
+                    TW_LDS_BARRIER(); // end of the last time slot
+                    TW_LDS_BARRIER(); // the C tile is staged
+                    store_tile(prev.u, prev.m0, prev.m_end);
+                }
+                TW_LDS_BARRIER(); // LDS may be reused now
+            }
+            if (is_end(cur))
+                break;
+            if (!has_steps(cur)) { // no step, no pipeline barrier to ride on
                 nxt = claim();
                 have_next = true;
             }
-#if defined(TW_EXP_TIMING) && TW_EXP_ITEM > 0
-            TW_WS_PHASE(7, 256)
-#endif
-            if (item >= p.n_gemm_items) {
-                zero_fill(item);
-            } else {
+            if (is_fill(cur)) {
+                zero_fill(cur);
+            } else if (nsteps > 0) {
                 const UnitDev &u = cur.u;
-                const int m0 = cur.m0;
-                const int nsteps = u.k_pad / BK;
-                const Thr tc = setup(cur);
-                // output columns of the unit and their bias: fetched now, handed to the other waves
-                // through LDS with the last step
-                int out_col = 0;
-                float out_bias = 0.0f;
-                if (pt < BN)
-                    out_col = u.col0 + p.kept_n[u.kn_off + (pt < u.n_cnt ? pt : 0)];
-                if (!preloaded && nsteps > 0) {
-                    Idx ix[R];
-#pragma unroll
-                    for (int j = 0; j < R; ++j)
-                        load_idx(tc, j, ix[j]); // the padded list keeps every index load in bounds
-                    load_idx(tc, R, ix_next);
-                    // Every register slot is loaded whether or not the item has that many steps
-                    // (the index list is padded, the weight step is clamped): the number of loads
-                    // in flight is then the same on every path into the slots below, and the
-                    // compiler can wait for exactly the loads a slot needs.
-#pragma unroll
-                    for (int j = 0; j < R; ++j)
-                        issue(tc, j < nsteps ? j : nsteps - 1, ix[j], a_ring[j], b_ring[j]);
-                }
-                TW_WS_PHASE(0, 256)
-                TW_WS_PHASE(1, 256)
                 // time slot j: write step j (loaded R slots ago) into stage j & 1 and reuse its
                 // registers for the loads of step j + R.  Every register is written to LDS and
                 // refilled by its next load back to back, so that the LDS queue and the
-                // vector-memory queue are fed at the same time.
-                auto slot = [&](int j, int r, bool more) {
-                    TW_WS_STAMP(j, 2, 256)
+                // vector-memory queue are fed at the same time.  When no step j + R is left, the
+                // refill reads one fixed 16-byte piece with all lanes (a single cache line per
+                // load, never used): no branch, and one copy of this code serves every slot.
+                const int k_left0 = u.k_kept - row0; // kept rows from this lane's first row on
+                auto slot = [&](int j, int r) {
                     uint16_t *const stA = sA + (j & 1) * ASTAGE;
                     uint16_t *const stB = sB + (j & 1) * BSTAGE;
-                    const bool edge = j * BK + BK > u.k_kept || m0 + BM > cur.m_end;
+                    const bool more = j + R < nsteps;
+                    const uint32_t live = more ? 0xFFFFFFFFu : 0u;
                     const Idx ix = ix_next;
-                    if (more)
-                        load_idx(tc, j + R + 1, ix_next);
-#pragma unroll
-                    for (int ps = 0; ps < PASSES; ++ps) {
-                        u32x4 v = a_ring[r][ps];
-                        if (edge) {
-                            // rows beyond K_t and chunks beyond M become zeros
-                            const uint32_t keep =
-                                (j * BK + rgrp * 8 + ps < u.k_kept && tc.m_ok) ? 0xFFFFFFFFu : 0u;
-                            v.x &= keep;
-                            v.y &= keep;
-                            v.z &= keep;
-                            v.w &= keep;
-                        }
-                        *reinterpret_cast<u32x4 *>(stA + (rgrp * 8 + ps) * PITCH + chunk * 8) = v;
-                        if (more)
-                            a_ring[r][ps] = load_a(tc, ix, ps);
-                    }
+                    load_idx(tc, j + R + 1, ix_next); // the list is padded: always in bounds
+                    const int sb = more ? j + R : 0;
+                    const uint32_t vb = v_b & live;
 #pragma unroll
                     for (int bp = 0; bp < BPASS; ++bp) {
-                        *reinterpret_cast<u32x4 *>(stB + (pt + bp * NP) * 8) = b_ring[r][bp];
-                        if (more)
-                            b_ring[r][bp] = load_b(tc, j + R, bp);
+                        *reinterpret_cast<u32x4 *>(stB + (pt + bp * NPM) * 8) = b_ring[r][bp];
+                        b_ring[r][bp] = load_b(tc, sb, bp, vb);
                     }
-                    TW_WS_STAMP(j, 4, 256)
+                    const uint32_t vc = tc.v_chunk & live;
+                    const int k_left = k_left0 - j * BK;
+#pragma unroll
+                    for (int ps = 0; ps < PASSES; ++ps) {
+                        // rows beyond K_t and chunks beyond M become zeros
+                        const uint32_t keep = (ps < k_left && tc.m_ok) ? 0xFFFFFFFFu : 0u;
+                        u32x4 v = a_ring[r][ps];
+                        v.x &= keep;
+                        v.y &= keep;
+                        v.z &= keep;
+                        v.w &= keep;
+                        *reinterpret_cast<u32x4 *>(stA + (row0 + ps) * PITCH + chunk * 8) = v;
+                        a_ring[r][ps] = load_a(tc, ix, ps, live, vc);
+                    }
                     TW_LDS_BARRIER();
-                    TW_WS_STAMP(j, 5, 256)
                     if (j == 0 && !have_next) {
                         nxt = published();
                         have_next = true;
                     }
                 };
-                int j0 = 0;
-                for (; j0 + 2 * R <= nsteps; j0 += R) {
-#pragma unroll
-                    for (int r = 0; r < R; ++r)
-                        slot(j0 + r, r, true);
+                static_assert(R == 2, "the slots alternate between two register slots");
+                for (int j = 0;;) {
+                    slot(j, 0);
+                    if (++j >= nsteps)
+                        break;
+                    slot(j, 1);
+                    if (++j >= nsteps)
+                        break;
                 }
-                // (the column numbers have arrived by now: the bias load flies over the last slots)
-                if (p.bias && pt < BN)
-                    out_bias = p.bias[out_col];
-                // The last one to three slots, written out so that each knows at compile time
-                // whether it still fetches a step (a slot that decides this at run time makes the
-                // compiler wait for every load in flight before the first LDS write).
-                static_assert(R == 2, "the drain is written out for two register slots");
-                if (nsteps - j0 == 3) {
-                    slot(j0, 0, true);
-                    slot(j0 + 1, 1, false);
-                    slot(j0 + 2, 0, false);
-                } else if (nsteps - j0 == 2) {
-                    slot(j0, 0, false);
-                    slot(j0 + 1, 1, false);
-                } else if (nsteps - j0 == 1) {
-                    slot(j0, 0, false); // an item of one step
-                } // (a unit without kept rows has no step: its columns receive beta * C)
-                // last time slot: the multiplying waves work on the last step; the first loads of
-                // the next item start now and fly over the epilogue
-                const bool chain = nxt.ticket < p.n_pipe_items;
-                if (chain) {
-                    const Thr tn = setup(nxt);
-                    const int nn = nxt.u.k_pad / BK;
-                    Idx ix[R];
-#pragma unroll
-                    for (int j = 0; j < R; ++j)
-                        load_idx(tn, j, ix[j]);
-                    load_idx(tn, R, ix_next);
-#pragma unroll
-                    for (int j = 0; j < R; ++j)
-                        issue(tn, j < nn ? j : nn - 1, ix[j], a_ring[j], b_ring[j]);
-                }
-                preloaded = chain;
-                if (pt < BN) {
-                    s_cols[pt] = out_col;
-                    s_bias[pt] = out_bias;
-                }
-                TW_WS_PHASE(2, 256)
-                TW_LDS_BARRIER(); // end of the last time slot
-                TW_WS_PHASE(3, 256)
-                TW_LDS_BARRIER(); // the C tile is staged
-                TW_WS_PHASE(4, 256)
-                store_tile(u, m0, cur.m_end);
-                TW_WS_PHASE(5, 256)
-            }
-            TW_LDS_BARRIER(); // LDS may be reused now
+            } // (a unit without kept rows has no step: its columns receive beta * C)
+            prev = cur;
+            have_prev = true;
             cur = nxt;
             have_next = false;
-#ifdef TW_EXP_TIMING
-            ++ws_item;
-#endif
         }
     } else {
         // ================= multiplying waves ==============================================
-        Item cur = make_item(blockIdx.x);
+        Item cur = make_item(qi);
         Item nxt = cur;
         bool have_next = false;
-        while (cur.ticket < p.n_items) {
-            const int item = cur.ticket;
-            if (item >= p.n_pipe_items) {
+        while (!is_end(cur)) {
+            if (!has_steps(cur)) {
                 nxt = claim();
                 have_next = true;
             }
-            if (item >= p.n_gemm_items) {
-                zero_fill(item);
+            if (is_fill(cur)) {
+                zero_fill(cur);
             } else {
                 const UnitDev &u = cur.u;
                 const int m0 = cur.m0;
@@ -1043,7 +1018,20 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #pragma unroll
                         for (int r = 0; r < 16; ++r)
                             acc[mi][ni][r] = 0.0f;
-                const bool w_active = m0 + wave * 64 < cur.m_end;
+                const bool w_active = m0 + wave * RW < cur.m_end;
+                // output columns of this lane's compact columns and their bias: fetched now, used
+                // in the epilogue (the wait for the first staged step covers their round trips)
+                const int32_t *const nlist = p.kept_n + u.kn_off;
+                int out_col[NI];
+                float out_bias[NI];
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni) {
+                    const int j = ni * 32 + (lane & 31);
+                    out_col[ni] = u.col0 + nlist[j < u.n_cnt ? j : 0];
+                }
+#pragma unroll
+                for (int ni = 0; ni < NI; ++ni)
+                    out_bias[ni] = p.bias ? p.bias[out_col[ni]] : 0.0f;
                 auto frags = [&](int s, int ks, u32x4(&af)[MI], u32x4(&bf)[NI]) {
                     const uint16_t *const stA = sA + (s & 1) * ASTAGE;
                     const uint16_t *const stB = sB + (s & 1) * BSTAGE;
@@ -1053,7 +1041,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                         // row L/4, columns 4*(L%4)..+3 and receives column L of the 4 rows.
                         const int L = lane & 15;
                         const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
-                        const int col = wave * 64 + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
+                        const int col = wave * RW + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
                         const uint16_t *q = stA + row * PITCH + col;
                         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
                         s16x4 hi =
@@ -1076,7 +1064,6 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                     have_next = true;
                 }
                 for (int s = 0; s < nsteps; ++s) {
-                    TW_WS_STAMP(s, 0, 0)
                     if (w_active) {
                         u32x4 af[2][MI], bf[2][NI];
                         frags(s, 0, af[0], bf[0]);
@@ -1091,12 +1078,10 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                                     acc[mi][ni] = E::mfma(af[ks & 1][mi], bf[ks & 1][ni], acc[mi][ni]);
                         }
                     }
-                    TW_WS_STAMP(s, 1, 0)
                     TW_LDS_BARRIER();
                 }
 
                 // epilogue: alpha/beta in fp32, round, hand the tile over through LDS
-                const int32_t *const nlist = p.kept_n + u.kn_off;
                 float scale = p.alpha;
                 const bool fused = (p.bias || p.act) && p.beta == 0.0f;
                 if (p.beta != 0.0f) {
@@ -1105,34 +1090,34 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni) {
                         const int j = ni * 32 + (lane & 31);
-                        const int col = j < u.n_cnt ? u.col0 + nlist[j] : 0;
+                        const int col = out_col[ni];
                         const int64_t coff = (int64_t)col * p.ldc;
 #pragma unroll
                         for (int mi = 0; mi < MI; ++mi)
 #pragma unroll
                             for (int r = 0; r < 16; ++r) {
-                                const int m = m0 + wave * 64 + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
+                                const int m = m0 + wave * RW + mi * 32 + (lane >> 5) * 4 + (r >> 2) * 8 + (r & 3);
                                 float old = 0.0f;
                                 if (p.beta != 0.0f && j < u.n_cnt && m < cur.m_end)
                                     old = E::from_bits(C[coff + m]);
-                                acc[mi][ni][r] =
-                                    tw_finish(p.alpha * acc[mi][ni][r] + p.beta * old, p.bias, col, p.act);
+                                acc[mi][ni][r] = tw_activate(
+                                    p.alpha * acc[mi][ni][r] + p.beta * old + out_bias[ni], p.act);
                             }
                     }
                     scale = 1.0f;
                 }
                 if (fused) {
-                    // bias (handed over through LDS by the moving waves) and activation in fp32,
-                    // one rounding; the activation is a compile-time constant of each copy
+                    // bias and activation in fp32, one rounding; the activation is a compile-time
+                    // constant of each copy
                     auto stage_fused = [&](auto act_tag) {
                         constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
                         for (int ni = 0; ni < NI; ++ni) {
                             const int j = ni * 32 + (lane & 31);
-                            const float bj = p.bias ? s_bias[j] : 0.0f;
+                            const float bj = out_bias[ni];
 #pragma unroll
                             for (int mi = 0; mi < MI; ++mi) {
-                                const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
+                                const int mloc = wave * RW + mi * 32 + (lane >> 5) * 4;
 #pragma unroll
                                 for (int r4 = 0; r4 < 4; ++r4) {
                                     float v[4];
@@ -1167,7 +1152,7 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                         const int j = ni * 32 + (lane & 31); // compact column inside the unit
 #pragma unroll
                         for (int mi = 0; mi < MI; ++mi) {
-                            const int mloc = wave * 64 + mi * 32 + (lane >> 5) * 4;
+                            const int mloc = wave * RW + mi * 32 + (lane >> 5) * 4;
 #pragma unroll
                             for (int r4 = 0; r4 < 4; ++r4) {
                                 u32x2 pk;
@@ -1180,6 +1165,11 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
                         }
                     }
                 }
+                if (wave == 0 && lane < 32) {
+#pragma unroll
+                    for (int ni = 0; ni < NI; ++ni)
+                        s_cols[ni * 32 + lane] = out_col[ni];
+                }
                 pick_up();
                 if (tid == 0 && announced)
                     asm volatile("" : "+v"(t_done)); // the count has returned: read it before the stores
@@ -1189,31 +1179,15 @@ template <int DT> __global__ void __launch_bounds__(512, 2) tw_gemm_ws_kernel(co
             TW_LDS_BARRIER(); // LDS may be reused now
             cur = nxt;
             have_next = false;
-#ifdef TW_EXP_TIMING
-            ++ws_item;
-#endif
         }
-#ifdef TW_EXP_TIMING
-        if (blockIdx.x == 0 && tid == 0) {
-            s_ws[250] = __builtin_readcyclecounter();
-            s_ws[251] = __builtin_amdgcn_s_memrealtime();
-        }
-        __builtin_amdgcn_s_waitcnt(0);
-#if TW_EXP_TIMING == 2
-        if (tid == 0 && blockIdx.x < 256)
-            reinterpret_cast<unsigned *>(p.dbg)[blockIdx.x * 2 + 1] = (unsigned)__builtin_amdgcn_s_memrealtime();
-#else
-        if (blockIdx.x == 0 && tid < 256)
-            reinterpret_cast<unsigned long long *>(p.dbg)[tid] = s_ws[tid];
-#endif
-#endif
         // the workgroup counted last re-arms the ticket slot for the next launch: every
         // workgroup's claims had returned before it was counted.  Plain stores, made visible by
         // the end of the kernel; a device-scope fence here would write back and invalidate this
         // XCD's L2 under the workgroups that still stream through it.
         if (tid == 0 && t_done == (int)gridDim.x - 1) {
-            p.ticket[0] = 0;
-            p.ticket[1] = 0;
+#pragma unroll
+            for (int i = 0; i <= kXcd; ++i)
+                p.ticket[i] = 0;
         }
     }
 }
@@ -1240,10 +1214,11 @@ __global__ void __launch_bounds__(256, 2) tw_gemm_generic_kernel(const GemmArgs 
     const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
     uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
     const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
+    // one workgroup per item, unit after unit (the queues are not used here: n_split == 1)
     const int item = blockIdx.x;
 
-    if (item >= p.n_gemm_items) { // zero-fill item: pruned columns receive beta*C
-        const int z = item - p.n_gemm_items;
+    if (item >= p.n_gemm_u * p.n_mblk) { // zero-fill item: pruned columns receive beta*C
+        const int z = item - p.n_gemm_u * p.n_mblk;
         const int zt = z / p.n_mblk;
         const int m0 = (z - zt * p.n_mblk) * BM;
         const TileDev t = p.tiles[zt];
@@ -1375,40 +1350,151 @@ __global__ void insert_row_kernel(uint16_t *matrix, const uint16_t *matrix_2, in
 // outputs above this size are written through to memory: the size of one XCD's L2
 constexpr int64_t kStoreThroughBytes = 4 << 20;
 
-static int env_int(const char *name, int dflt)
-{
-    const char *v = getenv(name);
-    return v && *v ? atoi(v) : dflt;
-}
-
-// Tile shapes: 0: 256 x 128 (8 waves of 64 x 64, one workgroup per CU), 1: 128 x 128 (4 waves,
-// two per CU), 2: 512 x 64, 3: 256 x 64 (the two shapes for tiles of at most 64 kept columns),
-// 4: 256 x 128 wave-specialised (the default for wider tiles; shape 0 remains for operands the
-// 32-bit offsets of shape 4 cannot address).
+// Kernel shapes: rows of a work item, widest unit piece taken, workgroups meant to share a CU.
+// SHAPE_WIDE is tw_gemm_kmajor_kernel (64-bit addressing, for operands the 32-bit row offsets of
+// the wave-specialised kernel cannot reach); all others are tw_gemm_ws_kernel<BM, BN>.
 struct Shape {
-    int bm, wgs_per_cu;
+    int bm, bn, wgs_per_cu;
 };
-static const Shape kShapes[5] = {{256, 1}, {128, 2}, {512, 1}, {256, 2}, {256, 1}};
+static const Shape kShapes[TW_N_SHAPES] = {
+    {256, 128, 1}, // TW_SHAPE_WIDE
+    {128, 128, 2}, // TW_SHAPE_128x128
+    {512, 64, 1},  // TW_SHAPE_512x64
+    {128, 64, 2},  // TW_SHAPE_128x64
+    {256, 128, 1}, // TW_SHAPE_256x128
+    {128, 32, 2},  // TW_SHAPE_128x32
+};
 
 template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int grid, hipStream_t s)
 {
     switch (shape) {
-    case 0:
+    case TW_SHAPE_WIDE:
         hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 2, 64, 2, 1>), dim3(grid), dim3(512), 0, s, a);
         break;
-    case 1:
-        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 2, 2, 32, 3, 2>), dim3(grid), dim3(256), 0, s, a);
+    case TW_SHAPE_128x128:
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 128>), dim3(grid), dim3(256), 0, s, a);
         break;
-    case 2:
-        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 8, 1, 32, 2, 1>), dim3(grid), dim3(512), 0, s, a);
+    case TW_SHAPE_512x64:
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 512, 64>), dim3(grid), dim3(512), 0, s, a);
         break;
-    case 3:
-        hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 1, 32, 2, 2>), dim3(grid), dim3(256), 0, s, a);
+    case TW_SHAPE_128x64:
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 64>), dim3(grid), dim3(256), 0, s, a);
         break;
-    default: // 4: wave-specialised 256 x 128
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT>), dim3(grid), dim3(512), 0, s, a);
+    case TW_SHAPE_128x32:
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 32>), dim3(grid), dim3(256), 0, s, a);
+        break;
+    default: // TW_SHAPE_256x128
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128>), dim3(grid), dim3(512), 0, s, a);
         break;
     }
+}
+
+// Process-wide tuning switches (tw_set_option); -1 = automatic.  The environment variables
+// TWGEMM_SHAPE, TWGEMM_WGS_PER_CU, TWGEMM_PIECE and TWGEMM_XCD_QUEUES give their initial values
+// and are read once.
+static std::atomic<int> g_opt[TW_N_OPTIONS];
+static std::once_flag g_opt_once;
+static const char *const kOptEnv[TW_N_OPTIONS] = {"TWGEMM_SHAPE", "TWGEMM_WGS_PER_CU", "TWGEMM_PIECE",
+                                                  "TWGEMM_XCD_QUEUES"};
+
+static bool option_in_range(int option, int value)
+{
+    if (value == -1)
+        return true;
+    switch (option) {
+    case TW_OPT_SHAPE:
+        return value >= 0 && value < TW_N_SHAPES;
+    case TW_OPT_WGS_PER_CU:
+        return value >= 1 && value <= 8;
+    case TW_OPT_PIECE:
+        return value == 32 || value == 64 || value == 128;
+    case TW_OPT_XCD_QUEUES:
+        return value == 0 || value == 1;
+    }
+    return false;
+}
+
+static void init_options()
+{
+    std::call_once(g_opt_once, [] {
+        for (int o = 0; o < TW_N_OPTIONS; ++o) {
+            const char *v = getenv(kOptEnv[o]);
+            const int x = v && *v ? atoi(v) : -1;
+            g_opt[o].store(option_in_range(o, x) ? x : -1, std::memory_order_relaxed);
+        }
+    });
+}
+
+static int option(int o)
+{
+    init_options();
+    return g_opt[o].load(std::memory_order_relaxed);
+}
+
+static int round_up32(int v) { return (v + 31) / 32 * 32; }
+
+// What a launch runs with: kernel shape, columns of a unit piece, workgroups per CU.
+struct Choice {
+    int shape, piece, per_cu;
+    bool xcd;
+};
+
+// Picks the shape from the plan and M.  Wide tiles with many rows run 256-row items (half the
+// weight traffic per row of A).  Items of few steps run 128-row items with two workgroups per CU,
+// so that one's start-up and epilogue hide under the other's steps.  Launches with too few items
+// for the chip (skinny M) hand a unit out in pieces of 64 or 32 columns.
+static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
+{
+    Choice c;
+    const int width = std::max(32, round_up32(plan->max_unit_n)); // 32, 64, 96 or 128
+    const int cu = plan->cu_count;
+    const bool ws_ok = (uint64_t)plan->K * (uint64_t)lda * 2u < (1ull << 32);
+    const int64_t units = std::max(1, plan->n_pipe_units);
+    auto items = [&](int bm, int piece) {
+        return units * ((width + piece - 1) / piece) * ((M + bm - 1) / bm);
+    };
+    c.xcd = option(TW_OPT_XCD_QUEUES) != 0;
+    c.piece = 128;
+    if (!ws_ok) {
+        c.shape = TW_SHAPE_WIDE;
+    } else if (width > 64) {
+        if (items(128, 128) * 2 < cu) { // skinny: split the units until half the chip has work
+            c.piece = items(128, 64) * 2 >= cu ? 64 : 32;
+            c.shape = c.piece == 64 ? TW_SHAPE_128x64 : TW_SHAPE_128x32;
+        } else if (items(256, 128) * 4 < 3 * cu || plan->mean_steps <= 8) {
+            c.shape = TW_SHAPE_128x128;
+        } else {
+            c.shape = TW_SHAPE_256x128;
+        }
+    } else if (width > 32) {
+        c.piece = 64;
+        if (items(512, 64) * 5 >= 3 * cu) {
+            c.shape = TW_SHAPE_512x64;
+        } else if (items(128, 64) * 2 >= cu) {
+            c.shape = TW_SHAPE_128x64;
+        } else {
+            c.piece = 32;
+            c.shape = TW_SHAPE_128x32;
+        }
+    } else {
+        c.piece = 32;
+        c.shape = TW_SHAPE_128x32;
+    }
+    // forced choices, where they fit the plan: a shape takes pieces up to its width
+    const int f_piece = option(TW_OPT_PIECE), f_shape = option(TW_OPT_SHAPE);
+    if (f_shape >= 0 && (f_shape != TW_SHAPE_WIDE ? ws_ok : true)) {
+        const int piece = f_piece > 0 ? f_piece : std::min(128, kShapes[f_shape].bn);
+        if (std::min(piece, width) <= kShapes[f_shape].bn) {
+            c.shape = f_shape;
+            c.piece = piece;
+        }
+    } else if (f_piece > 0 && std::min(f_piece, width) <= kShapes[c.shape].bn) {
+        c.piece = f_piece;
+    }
+    if (c.shape == TW_SHAPE_WIDE)
+        c.piece = 128;
+    c.per_cu = option(TW_OPT_WGS_PER_CU) > 0 ? option(TW_OPT_WGS_PER_CU) : kShapes[c.shape].wgs_per_cu;
+    return c;
 }
 
 } // namespace tw
@@ -1417,6 +1503,17 @@ using namespace tw;
 
 extern "C" {
 
+int tw_set_option(int option_id, int value)
+{
+    if (option_id < 0 || option_id >= TW_N_OPTIONS)
+        return fail(TW_ERR_LAYOUT, "option %d: unknown", option_id);
+    if (!option_in_range(option_id, value))
+        return fail(TW_ERR_LAYOUT, "option %d: value %d is out of range", option_id, value);
+    init_options();
+    g_opt[option_id].store(value, std::memory_order_relaxed);
+    return TW_OK;
+}
+
 int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
             int64_t ldc, int M, float alpha, float beta, int pruned_cols, void *stream)
 {
@@ -1424,10 +1521,14 @@ int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void 
                       stream);
 }
 
-int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
-               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
-               void *stream)
+namespace {
+
+// argument checks shared by the launching entry points; TW_OK with *run == false: nothing to do
+int check_gemm_args(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
+                    int c_layout, int64_t ldc, int M, int pruned_cols, const tw_epilogue *ep,
+                    bool *run)
 {
+    *run = false;
     if (!plan)
         return fail(TW_ERR_NULL, "plan is NULL");
     if (ep && (ep->activation < TW_ACT_NONE || ep->activation > TW_ACT_TANH))
@@ -1453,76 +1554,19 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
                     (long long)lda, (long long)ldc);
     if (((uintptr_t)A & 15) || ((uintptr_t)C & 15))
         return fail(TW_ERR_ALIGNMENT, "A and C must be 16-byte aligned");
-    {
-        // the plan's tables and packed weight live on the device it was built on
-        int dev = -1;
-        TW_HIP(hipGetDevice(&dev));
-        if (dev != plan->device)
-            return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d",
-                        plan->device, dev);
-    }
-    if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR) {
-        // layout-generic path (element strides), 128-row blocks, one workgroup per item
-        GemmArgs a;
-        a.units = plan->d_units;
-        a.tiles = plan->d_tiles;
-        a.kept_k = plan->d_kept_k_pad;
-        a.kept_n = plan->d_kept_n;
-        a.pruned_n = plan->d_pruned_n;
-        a.Bp = plan->d_Bp;
-        a.A = A;
-        a.C = C;
-        a.lda = lda;
-        a.ldc = ldc;
-        a.M = M;
-        a.n_mblk = (M + 127) / 128;
-        a.n_gemm_items = plan->n_units * a.n_mblk;
-        a.n_pipe_items = plan->n_pipe_units * a.n_mblk;
-        a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
-        a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
-        a.alpha = alpha;
-        a.beta = beta;
-        a.ticket = nullptr;
-        a.dbg = nullptr;
-        a.n_arg_units = 0;
-        a.bias = ep ? ep->bias : nullptr;
-        a.act = ep ? ep->activation : TW_ACT_NONE;
-        a.store_through = 0;
-        if (a.n_items == 0)
-            return TW_OK;
-        const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
-        const int64_t sa_k = a_layout == TW_LAYOUT_KMAJOR ? lda : 1;
-        const int64_t sc_m = c_layout == TW_LAYOUT_KMAJOR ? 1 : ldc;
-        const int64_t sc_n = c_layout == TW_LAYOUT_KMAJOR ? ldc : 1;
-        if (plan->dtype == TW_F16)
-            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_F16>), dim3(a.n_items), dim3(256), 0,
-                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
-        else
-            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_BF16>), dim3(a.n_items), dim3(256), 0,
-                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
-        TW_HIP(hipGetLastError());
-        return TW_OK;
-    }
+    // the plan's tables and packed weight live on the device it was built on
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev != plan->device)
+        return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d",
+                    plan->device, dev);
+    *run = true;
+    return TW_OK;
+}
 
-    // Shape choice: the large tile halves the weight traffic per row of A, but needs enough
-    // work items to fill the chip; otherwise the small tile with two workgroups per CU.
-    const bool narrow = plan->max_unit_n <= 64;
-    // the wave-specialised kernel addresses A with 32-bit byte offsets
-    const bool ws_ok = (uint64_t)plan->K * (uint64_t)lda * 2u < (1ull << 32);
-    int shape = narrow ? 2 : (ws_ok ? 4 : 0);
-    {
-        const int forced = env_int("TWGEMM_SHAPE", -1);
-        const int64_t big_items =
-            (int64_t)plan->n_units * ((M + kShapes[shape].bm - 1) / kShapes[shape].bm);
-        if (forced >= 0 && forced < 5 && (forced == 2 || forced == 3) == narrow && (forced != 4 || ws_ok))
-            shape = forced;
-        else if (big_items * 5 < 3 * (int64_t)plan->cu_count && (narrow || M <= 128))
-            shape = narrow ? 3 : 1; // too few large items to occupy the chip (for wide tiles the
-                                    // wave-specialised kernel still wins unless a 128-row block
-                                    // holds all of M)
-    }
-    const int BM = kShapes[shape].bm;
-    GemmArgs a;
+void fill_common(GemmArgs &a, const tw_plan *plan, const void *A, int64_t lda, void *C, int64_t ldc,
+                 int M, float alpha, float beta, const tw_epilogue *ep)
+{
     a.units = plan->d_units;
     a.tiles = plan->d_tiles;
     a.kept_k = plan->d_kept_k_pad;
@@ -1534,44 +1578,104 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
     a.lda = lda;
     a.ldc = ldc;
     a.M = M;
-    a.n_mblk = (M + BM - 1) / BM;
-    a.n_gemm_items = plan->n_units * a.n_mblk;
-    a.n_pipe_items = plan->n_pipe_units * a.n_mblk;
-    const int per_cu = env_int("TWGEMM_WGS_PER_CU", kShapes[shape].wgs_per_cu);
-    a.n_zero_tiles = pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0;
-    a.n_items = a.n_gemm_items + a.n_zero_tiles * a.n_mblk;
     a.alpha = alpha;
     a.beta = beta;
     a.bias = ep ? ep->bias : nullptr;
     a.act = ep ? ep->activation : TW_ACT_NONE;
-    // an output larger than one L2 is written through (see store_chunk)
-    a.store_through = (int64_t)M * plan->N * 2 > kStoreThroughBytes;
-    if (a.n_items == 0)
+    a.store_through = 0;
+    a.ticket = nullptr;
+    a.n_arg_units = 0;
+}
+
+// item matrix and queues of a launch with `bm`-row items and unit pieces of `piece` columns
+void fill_queues(GemmArgs &a, const tw_plan *plan, int M, int bm, int piece, int pruned_cols, bool xcd)
+{
+    const int width = std::max(32, round_up32(plan->max_unit_n));
+    a.n_split = (std::min(width, 128) + piece - 1) / piece;
+    a.piece_nb = piece / kMfmaN;
+    a.n_mblk = (M + bm - 1) / bm;
+    a.n_pipe_u = plan->n_pipe_units * a.n_split;
+    a.n_gemm_u = plan->n_units * a.n_split;
+    a.n_all_u = a.n_gemm_u + (pruned_cols == TW_PRUNED_ZERO ? plan->n_zero_tiles : 0);
+    a.n_own = xcd ? a.n_mblk / kXcd : 0;
+    a.n_own_items = a.n_own * a.n_all_u;
+    a.n_tail_mblk = a.n_mblk - kXcd * a.n_own;
+    a.n_tail_items = a.n_tail_mblk * a.n_all_u;
+}
+
+// launches the K-major kernels with the counters at `ticket` (kTicketInts zeros)
+int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *ticket, hipStream_t s)
+{
+    if (a.n_all_u == 0)
         return TW_OK;
-    const unsigned slot =
-        __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kTicketSlots;
-    a.ticket = plan->d_tickets + 2 * slot;
-    a.dbg = plan->d_tickets + 2 * kTicketSlots;
+    a.ticket = ticket;
     a.n_arg_units = plan->n_units <= kMaxArgUnits ? plan->n_units : 0;
     for (int i = 0; i < a.n_arg_units; ++i)
         a.arg_units[i] = plan->h_units[i];
-
-    const int grid = (int)std::min<int64_t>(a.n_items, (int64_t)plan->cu_count * per_cu);
-    hipStream_t s = (hipStream_t)stream;
+    // queue 0 is the longest: one workgroup per entry, up to the chip's share of a queue
+    const int64_t qlen0 = (int64_t)a.n_own_items + (a.n_tail_items + kXcd - 1) / kXcd;
+    const int64_t per_queue = std::max<int64_t>(1, (int64_t)plan->cu_count * c.per_cu / kXcd);
+    const int grid = (int)(kXcd * std::min(qlen0, per_queue));
     if (plan->dtype == TW_F16)
-        launch_kmajor<TW_F16>(shape, a, grid, s);
+        launch_kmajor<TW_F16>(c.shape, a, grid, s);
     else
-        launch_kmajor<TW_BF16>(shape, a, grid, s);
+        launch_kmajor<TW_BF16>(c.shape, a, grid, s);
     TW_HIP(hipGetLastError());
     return TW_OK;
 }
 
-#ifdef TW_EXP_TIMING
-int tw_exp_read_debug(const tw_plan *plan, void *host, int nbytes)
+} // namespace
+
+int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
+               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
+               void *stream)
 {
-    return hipMemcpy(host, plan->d_tickets + 2 * kTicketSlots, nbytes, hipMemcpyDeviceToHost);
+    bool run = false;
+    const int st = check_gemm_args(plan, A, a_layout, lda, C, c_layout, ldc, M, pruned_cols, ep, &run);
+    if (st != TW_OK || !run)
+        return st;
+    GemmArgs a;
+    fill_common(a, plan, A, lda, C, ldc, M, alpha, beta, ep);
+    if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR) {
+        // layout-generic path (element strides), 128-row blocks, one workgroup per item
+        fill_queues(a, plan, M, 128, 128, pruned_cols, false);
+        const int64_t n_items = (int64_t)a.n_all_u * a.n_mblk;
+        if (n_items == 0)
+            return TW_OK;
+        const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
+        const int64_t sa_k = a_layout == TW_LAYOUT_KMAJOR ? lda : 1;
+        const int64_t sc_m = c_layout == TW_LAYOUT_KMAJOR ? 1 : ldc;
+        const int64_t sc_n = c_layout == TW_LAYOUT_KMAJOR ? ldc : 1;
+        if (plan->dtype == TW_F16)
+            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_F16>), dim3((unsigned)n_items), dim3(256), 0,
+                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
+        else
+            hipLaunchKernelGGL((tw_gemm_generic_kernel<TW_BF16>), dim3((unsigned)n_items), dim3(256), 0,
+                               (hipStream_t)stream, a, sa_m, sa_k, sc_m, sc_n);
+        TW_HIP(hipGetLastError());
+        return TW_OK;
+    }
+
+    const Choice c = choose_shape(plan, M, lda);
+    fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
+    // an output larger than one L2 is written through (see store_chunk)
+    a.store_through = (int64_t)M * plan->N * 2 > kStoreThroughBytes;
+    // Ticket slot of this launch.  A launch recorded into a HIP graph keeps its slot for every
+    // replay, so recorded launches draw from a range of their own that eager launches never use.
+    hipStream_t s = (hipStream_t)stream;
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
+        (void)hipGetLastError();
+        cap = hipStreamCaptureStatusNone;
+    }
+    unsigned slot;
+    if (cap == hipStreamCaptureStatusActive)
+        slot = kEagerSlots + __atomic_fetch_add(&plan->next_capture_slot, 1u, __ATOMIC_RELAXED) %
+                                 (unsigned)(kTicketSlots - kEagerSlots);
+    else
+        slot = __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kEagerSlots;
+    return launch_gemm(plan, a, c, plan->d_tickets + kTicketInts * slot, s);
 }
-#endif
 
 int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A, const void *B,
                       float beta, void *C, int block_num, const int32_t *N_cal,

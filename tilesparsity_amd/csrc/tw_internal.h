@@ -21,6 +21,7 @@ constexpr int kMfmaK = 16;    // k extent of one v_mfma_f32_32x32x16
 constexpr int kBlockK = 64;   // k rows per packed weight step; K_t is padded to this
 constexpr int kMaxUnitN = 128; // compact columns handled by one work item
 constexpr int kTicketSlots = 256;
+constexpr int kEagerSlots = 192;  // slots of eager launches; the rest serve launches recorded in graphs
 constexpr int kMaxArgUnits = 32;
 
 // One schedulable piece of a tile: at most kMaxUnitN compact columns.
@@ -47,6 +48,16 @@ struct TileDev {
     int32_t pad_;
 };
 
+// The work of one launch is a matrix of items: `n_all_u` columns (pieces of units that have kept
+// K rows first, heaviest first; then pieces of units without; then, with TW_PRUNED_ZERO, the tiles
+// whose pruned columns are filled) by `n_mblk` blocks of BM rows.  It is handed out through
+// kXcd queues, one per accelerator die: workgroup b runs on die b % kXcd and draws from that
+// die's queue only, so the workgroups that share an L2 work on the same rows of A.  Queue x owns
+// the row blocks [x * n_own, (x + 1) * n_own) (all their items, row block after row block) and
+// every kXcd-th item of the remaining `n_tail_mblk` row blocks (unit after unit).
+constexpr int kXcd = 8;
+constexpr int kTicketInts = 16; // per slot: [0, kXcd) next index of each queue, [kXcd] workgroups done
+
 struct GemmArgs {
     const UnitDev *units;   // sorted by k_kept descending
     const TileDev *tiles;
@@ -59,16 +70,20 @@ struct GemmArgs {
     int64_t lda, ldc;
     int32_t M;
     int32_t n_mblk;       // ceil(M / BM)
-    int32_t n_gemm_items; // n_units * n_mblk
-    int32_t n_pipe_items; // items of units with at least one kept K row (they come first)
-    int32_t n_items;      // + n_zero_tiles * n_mblk when zero-filling
-    int32_t n_zero_tiles; // tiles with pruned columns (first entries of `tiles`)
+    int32_t n_split;      // a unit is handed out as n_split pieces of 32 * piece_nb compact columns
+    int32_t piece_nb;
+    int32_t n_pipe_u;     // pieces of units with at least one kept K row
+    int32_t n_gemm_u;     // + pieces of units without (their columns receive beta * C)
+    int32_t n_all_u;      // + tiles with pruned columns to fill
+    int32_t n_own;        // row blocks owned by each queue
+    int32_t n_own_items;  // n_own * n_all_u
+    int32_t n_tail_mblk;  // n_mblk - kXcd * n_own
+    int32_t n_tail_items; // n_tail_mblk * n_all_u
     float alpha, beta;
     const float *bias;    // fp32 [N] added to every written column before the activation, or null
     int32_t act;          // TW_ACT_*
     int32_t store_through; // output stores write through to memory (large outputs) or stay in L2
-    int32_t *ticket;      // [0] next item, [1] finished workgroups
-    void *dbg;            // 2 KiB scratch after the ticket slots (instrumented builds only)
+    int32_t *ticket;      // kTicketInts counters, zero between launches
     // Copy of `units` inside the kernel arguments for plans of at most kMaxArgUnits units
     // (n_arg_units == 0 otherwise): a workgroup then reads its first unit through the scalar
     // cache instead of waiting for a global load before it can fetch anything else.
@@ -95,7 +110,7 @@ struct tw_plan {
     tw::UnitDev *d_units = nullptr;
     tw::TileDev *d_tiles = nullptr;
     void *d_Bp = nullptr;
-    int32_t *d_tickets = nullptr; // kTicketSlots pairs
+    int32_t *d_tickets = nullptr; // kTicketSlots slots of kTicketInts counters
     // Ownership: every pointer above points into one of these two allocations.  d_lists holds the
     // four index arrays when the pre-pass compacted them on the device (else they sit in d_slab);
     // d_slab holds the unit / tile tables, the pruned-column and padded kept-K lists, the packing
@@ -103,7 +118,8 @@ struct tw_plan {
     void *d_lists = nullptr;
     void *d_slab = nullptr;
     void *d_pack_tiles = nullptr; // tw::PackTile[n_tiles] for packing from a dense weight
-    mutable unsigned next_slot = 0;
+    mutable unsigned next_slot = 0, next_capture_slot = 0;
+    int mean_steps = 0; // mean number of 64-row steps of the units that have any
     int cu_count = 0;
 };
 

@@ -589,8 +589,12 @@ int finalize_plan_geometry(tw_plan *p)
     p->n_units = (int)units.size();
     p->h_units = units;
     p->n_pipe_units = 0;
-    for (const UnitDev &u : units)
+    int64_t steps = 0;
+    for (const UnitDev &u : units) {
         p->n_pipe_units += u.k_pad > 0;
+        steps += u.k_pad / kBlockK;
+    }
+    p->mean_steps = p->n_pipe_units ? (int)(steps / p->n_pipe_units) : 0;
     p->n_zero_tiles = (int)ztiles.size();
 
     // One device allocation for everything the plan owns besides lists that were compacted on
@@ -630,7 +634,7 @@ int finalize_plan_geometry(tw_plan *p)
         o_rn = put(rel_n.data(), rel_n.size() * sizeof(int32_t));
     }
     const size_t o_tickets = (stage.size() + 255) / 256 * 256;
-    const size_t ticket_bytes = sizeof(int32_t) * 2 * kTicketSlots + 2048;
+    const size_t ticket_bytes = sizeof(int32_t) * kTicketInts * kTicketSlots;
     const size_t o_bp = (o_tickets + ticket_bytes + 1023) / 1024 * 1024;
     const size_t bp_bytes = (size_t)std::max<int64_t>(p->packed_elems, 8) * 2;
     char *slab = nullptr;

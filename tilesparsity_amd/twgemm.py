@@ -24,6 +24,8 @@ F16, BF16 = 0, 1
 KMAJOR, ROWMAJOR = 0, 1
 PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
+OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES = 0, 1, 2, 3
+SHAPE_WIDE, SHAPE_128x128, SHAPE_512x64, SHAPE_128x64, SHAPE_256x128, SHAPE_128x32 = range(6)
 
 
 class Epilogue(ctypes.Structure):
@@ -47,7 +49,7 @@ EXPORTED_SYMBOLS = (
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
-    "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask",
+    "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option",
 )
 
 
@@ -142,6 +144,7 @@ def lib():
                                  ctypes.POINTER(ctypes.c_double), vp]),
         "tw_lstm_gates": (c_int, [c_int, c_int, c_int, vp, c_i64, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
         "tw_plan_from_device_mask": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, vp, vp, c_int, pp]),
+        "tw_set_option": (c_int, [c_int, c_int]),
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
@@ -157,6 +160,11 @@ def lib():
 def _check(status):
     if status != OK:
         raise TwError(status, lib().tw_last_error().decode())
+
+
+def set_option(option, value):
+    """tw_set_option: process-wide tuning switch of the GEMM launches (OPT_*), -1 = automatic."""
+    _check(lib().tw_set_option(int(option), int(value)))
 
 
 def _i32(a):

@@ -252,7 +252,8 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
  *   TW_OPT_WGS_PER_CU   workgroups launched per compute unit, 1..8
  *   TW_OPT_PIECE        columns of a tile handed out as one work item: 128, 64 or 32
  *   TW_OPT_XCD_QUEUES   1: one work queue per accelerator die, each owning whole row blocks of A
- *                       (default); 0: the row blocks are dealt out over all queues
+ *                       (the workgroups of a die then share those rows in their L2);
+ *                       0 (default): the work items are dealt out over the dies in turn
  * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
  * TWGEMM_PIECE and TWGEMM_XCD_QUEUES, read once. */
 #define TW_OPT_SHAPE 0

@@ -625,6 +625,18 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     }
 }
 
+// Scheduling hints for NMM MFMAs of one 16-row k step: each MFMA is followed by its share of
+// the NRD LDS reads that fetch the operands of the next k step (none after the last step).
+template <int NRD, int NMM, int I, bool READS> __device__ __forceinline__ void sched_mfma_with_reads()
+{
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0); // one MFMA
+    constexpr int n = NRD * (I + 1) / NMM - NRD * I / NMM;
+    if constexpr (READS && n > 0)
+        __builtin_amdgcn_sched_group_barrier(0x100, n, 0); // n LDS reads
+    if constexpr (I + 1 < NMM)
+        sched_mfma_with_reads<NRD, NMM, I + 1, READS>();
+}
+
 // Workgroup barrier for hand-overs through LDS only: waits for this wave's LDS operations, not
 // for its global loads, stores or atomics in flight (which __syncthreads() would do for stores
 // and atomics), so prefetched loads, the item's output stores and the ticket atomic keep flying.
@@ -644,7 +656,7 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
 //   BM = 512: 4 + 4 waves, each multiplying wave 128 rows (tiles of at most 64 kept columns).
 // The first loads of the next item are issued during the last step of the current one and
 // fly over its epilogue.
-template <int DT, int BM, int BN>
+template <int DT, int BM, int BN, int R>
 __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(const GemmArgs p)
 {
     constexpr int NMW = BM == 128 ? 2 : 4;     // multiplying waves, and as many moving waves
@@ -652,7 +664,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
     constexpr int NT = 2 * NPM;
     constexpr int BK = 64;
     constexpr int KS = BK / kMfmaK, PKS = kBlockK / kMfmaK;
-    constexpr int R = 2;                       // register slots = steps of loads in flight
+    // (R register slots = steps of loads in flight per moving wave)
     constexpr int RW = BM / NMW;               // rows of a multiplying wave
     constexpr int MI = RW / 32, NI = BN / kMfmaN;
     constexpr int CPR = BM / 8;                // 16-byte chunks per staged A row / stored C column
@@ -828,7 +840,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         // (g, chunk) moves chunk `chunk` (8 consecutive m) of the rows
         // mw * RPW + g * PASSES + 0 .. PASSES - 1 of a step.  The lane fetches the indices of its
         // own rows (a 16-byte load per four rows, the lanes of a row group share the address)
-        // one step before the row loads that use them.  Row addresses are a uniform base plus a
+        // R steps before the row loads that use them.  Row addresses are a uniform base plus a
         // 32-bit byte offset per lane.
         const int pt = tid - NPM;
         const int chunk = lane % CPR, g = lane / CPR;
@@ -893,32 +905,30 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         for (;;) {
             u32x4 a_ring[R][PASSES];
             u32x4 b_ring[R][BPASS];
-            Idx ix_next; // row indices of the step issued next
+            Idx ix_ring[R]; // row indices of the steps whose loads the next R slots issue
             const Thr tc = setup(cur);
             const int nsteps = has_steps(cur) ? cur.u.k_pad / BK : 0;
             if (nsteps > 0) {
-                // First loads: weight and rows of steps 0 and 1, the index loads one step ahead,
-                // in the order the time slots keep up.  Both register slots are loaded whether or
-                // not the item has two steps (the index list is padded, the weight step is
+                // First loads: weight and rows of steps 0 .. R - 1, the index loads R steps ahead,
+                // in the order the time slots keep up.  All register slots are loaded whether or
+                // not the item has that many steps (the index list is padded, the weight step is
                 // clamped), like every slot below refills its registers whether or not a step is
                 // left to fetch: the sequence of loads is then the same on every path and the
                 // compiler can wait for exactly the loads a slot needs.
-                Idx ix0, ix1;
-                load_idx(tc, 0, ix0);
-                load_idx(tc, 1, ix1);
+                Idx ix[R];
 #pragma unroll
-                for (int bp = 0; bp < BPASS; ++bp)
-                    b_ring[0][bp] = load_b(tc, 0, bp, v_b);
+                for (int r = 0; r < R; ++r)
+                    load_idx(tc, r, ix[r]);
 #pragma unroll
-                for (int ps = 0; ps < PASSES; ++ps)
-                    a_ring[0][ps] = load_a(tc, ix0, ps, 0xFFFFFFFFu, tc.v_chunk);
-                load_idx(tc, 2, ix_next);
+                for (int r = 0; r < R; ++r) {
+                    load_idx(tc, R + r, ix_ring[r]);
 #pragma unroll
-                for (int bp = 0; bp < BPASS; ++bp)
-                    b_ring[1][bp] = load_b(tc, nsteps > 1 ? 1 : 0, bp, v_b);
+                    for (int bp = 0; bp < BPASS; ++bp)
+                        b_ring[r][bp] = load_b(tc, r < nsteps ? r : nsteps - 1, bp, v_b);
 #pragma unroll
-                for (int ps = 0; ps < PASSES; ++ps)
-                    a_ring[1][ps] = load_a(tc, ix1, ps, 0xFFFFFFFFu, tc.v_chunk);
+                    for (int ps = 0; ps < PASSES; ++ps)
+                        a_ring[r][ps] = load_a(tc, ix[r], ps, 0xFFFFFFFFu, tc.v_chunk);
+                }
             }
             if (have_prev) {
                 if (!is_fill(prev)) {
@@ -950,8 +960,10 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                     uint16_t *const stB = sB + (j & 1) * BSTAGE;
                     const bool more = j + R < nsteps;
                     const uint32_t live = more ? 0xFFFFFFFFu : 0u;
-                    const Idx ix = ix_next;
-                    load_idx(tc, j + R + 1, ix_next); // the list is padded: always in bounds
+                    // the indices of step j + R were fetched R slots ago; those of step j + 2 R
+                    // are fetched now (the list is padded: always in bounds)
+                    const Idx ix = ix_ring[r];
+                    load_idx(tc, j + 2 * R, ix_ring[r]);
                     const int sb = more ? j + R : 0;
                     const uint32_t vb = v_b & live;
 #pragma unroll
@@ -979,14 +991,14 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                         have_next = true;
                     }
                 };
-                static_assert(R == 2, "the slots alternate between two register slots");
-                for (int j = 0;;) {
-                    slot(j, 0);
-                    if (++j >= nsteps)
-                        break;
-                    slot(j, 1);
-                    if (++j >= nsteps)
-                        break;
+                for (int j = 0; j < nsteps;) {
+#pragma unroll
+                    for (int r = 0; r < R; ++r) {
+                        if (j < nsteps) {
+                            slot(j, r);
+                            ++j;
+                        }
+                    }
                 }
             } // (a unit without kept rows has no step: its columns receive beta * C)
             prev = cur;
@@ -1077,6 +1089,17 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                                 for (int mi = 0; mi < MI; ++mi)
                                     acc[mi][ni] = E::mfma(af[ks & 1][mi], bf[ks & 1][ni], acc[mi][ni]);
                         }
+                        // Instruction order of the step, pinned: the operands of the first 16 k
+                        // rows, then every MFMA of 16 k rows followed by its share of the LDS reads
+                        // for the next 16.  (Left alone, the scheduler reads one operand at a time
+                        // into the same registers and waits for each before the two MFMAs that
+                        // use it: the LDS latency then shows 16 times per step.)
+                        constexpr int NRD = 2 * MI + NI, NMM = MI * NI;
+                        __builtin_amdgcn_sched_group_barrier(0x100, NRD, 0);
+#pragma unroll
+                        for (int ks = 0; ks + 1 < KS; ++ks)
+                            sched_mfma_with_reads<NRD, NMM, 0, true>();
+                        sched_mfma_with_reads<NRD, NMM, 0, false>();
                     }
                     TW_LDS_BARRIER();
                 }
@@ -1365,6 +1388,25 @@ static const Shape kShapes[TW_N_SHAPES] = {
     {128, 32, 2},  // TW_SHAPE_128x32
 };
 
+// Steps of loads a moving wave keeps in flight, per shape (bounded by its 256 registers: a step
+// takes 4 * (A loads + weight loads per thread) of them).  Measured on the benchmark shapes: two
+// steps in flight are as fast as three or four, or faster.
+#ifndef TW_R_256x128
+#define TW_R_256x128 2
+#endif
+#ifndef TW_R_128x128
+#define TW_R_128x128 2
+#endif
+#ifndef TW_R_512x64
+#define TW_R_512x64 2
+#endif
+#ifndef TW_R_128x64
+#define TW_R_128x64 2
+#endif
+#ifndef TW_R_128x32
+#define TW_R_128x32 2
+#endif
+
 template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int grid, hipStream_t s)
 {
     switch (shape) {
@@ -1372,19 +1414,19 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
         hipLaunchKernelGGL((tw_gemm_kmajor_kernel<DT, 4, 2, 64, 2, 1>), dim3(grid), dim3(512), 0, s, a);
         break;
     case TW_SHAPE_128x128:
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 128>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 128, TW_R_128x128>), dim3(grid), dim3(256), 0, s, a);
         break;
     case TW_SHAPE_512x64:
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 512, 64>), dim3(grid), dim3(512), 0, s, a);
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 512, 64, TW_R_512x64>), dim3(grid), dim3(512), 0, s, a);
         break;
     case TW_SHAPE_128x64:
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 64>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 64, TW_R_128x64>), dim3(grid), dim3(256), 0, s, a);
         break;
     case TW_SHAPE_128x32:
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 32>), dim3(grid), dim3(256), 0, s, a);
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 32, TW_R_128x32>), dim3(grid), dim3(256), 0, s, a);
         break;
     default: // TW_SHAPE_256x128
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128>), dim3(grid), dim3(512), 0, s, a);
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128, TW_R_256x128>), dim3(grid), dim3(512), 0, s, a);
         break;
     }
 }
@@ -1439,10 +1481,13 @@ struct Choice {
     bool xcd;
 };
 
-// Picks the shape from the plan and M.  Wide tiles with many rows run 256-row items (half the
-// weight traffic per row of A).  Items of few steps run 128-row items with two workgroups per CU,
-// so that one's start-up and epilogue hide under the other's steps.  Launches with too few items
-// for the chip (skinny M) hand a unit out in pieces of 64 or 32 columns.
+// Picks the shape from the plan and M.  Wide tiles run 256-row items (half the weight traffic
+// per row of A), or 128-row items with two workgroups per CU when 256-row items would leave a
+// quarter of the chip without work.  Launches with too few items for the chip (skinny M) hand a
+// unit out in pieces of 64 or 32 columns.  One queue per die is an option, not the default: the
+// workgroups of a die then share the rows of A in their L2 (measured on the 0 %-sparse plan of
+// the headline shape: a third of the reads from memory), but no benchmark shape ran faster for
+// it and the stress shape, whose 512-row block of A fills an L2, ran 13 % slower.
 static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
 {
     Choice c;
@@ -1453,7 +1498,7 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
     auto items = [&](int bm, int piece) {
         return units * ((width + piece - 1) / piece) * ((M + bm - 1) / bm);
     };
-    c.xcd = option(TW_OPT_XCD_QUEUES) != 0;
+    c.xcd = option(TW_OPT_XCD_QUEUES) == 1;
     c.piece = 128;
     if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
@@ -1461,7 +1506,7 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
         if (items(128, 128) * 2 < cu) { // skinny: split the units until half the chip has work
             c.piece = items(128, 64) * 2 >= cu ? 64 : 32;
             c.shape = c.piece == 64 ? TW_SHAPE_128x64 : TW_SHAPE_128x32;
-        } else if (items(256, 128) * 4 < 3 * cu || plan->mean_steps <= 8) {
+        } else if (items(256, 128) * 4 < 3 * cu) {
             c.shape = TW_SHAPE_128x128;
         } else {
             c.shape = TW_SHAPE_256x128;

@@ -544,8 +544,8 @@ int finalize_plan_geometry(tw_plan *p)
         const int32_t kkp_off = (int32_t)kept_k_pad.size();
         kept_k_pad.insert(kept_k_pad.end(), p->kept_k_idx.begin() + p->kept_k_ptr[t],
                           p->kept_k_idx.begin() + p->kept_k_ptr[t + 1]);
-        // padding past k_pad: the kernel prefetches the index list up to six 64-row steps ahead
-        kept_k_pad.resize(kkp_off + p->k_pad[t] + 6 * kBlockK, 0);
+        // padding past k_pad: the kernel prefetches the index list up to eight 64-row steps ahead
+        kept_k_pad.resize(kkp_off + p->k_pad[t] + 8 * kBlockK, 0);
         p->b_off[t] = off;
         off += (int64_t)p->k_pad[t] * p->n_pad[t];
         off = (off + 511) / 512 * 512; // keep every tile 1 KiB aligned

@@ -242,6 +242,23 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
                int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
                const tw_epilogue *ep, void *stream);
 
+/* tw_gemm_ex for callers that cannot allocate device memory: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.
+ * It has no counterpart in the reference (Stream_Gemm_NN creates and destroys 32 streams per call,
+ * basic_nn.cu:396-406,440-443).  Same arguments and results as tw_gemm_ex, bit for bit; the only
+ * scratch memory the kernels use besides the inputs and outputs - the work-queue counters of the
+ * launch - lives in a 256-byte array inside the library's device image, one copy per GPU, held
+ * until the process ends.  The call allocates and frees nothing: it clears the counters with a
+ * small kernel on `stream`, then launches the GEMM on `stream`.
+ *   Limit: a launch of more than 2^31 - 1 work items (tile pieces x row blocks of 128 .. 512 rows)
+ *   is refused with TW_ERR_SHAPE, as it is by tw_gemm_ex; devices 0..63.
+ *   Every call on one GPU shares that GPU's counters: calls that overlap on one GPU (two streams,
+ *   two host threads, a graph replay next to an eager call) race and give wrong results.
+ *   Serialise them, or use tw_gemm_ex, whose plans carry 256 counter slots of their own. */
+int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
+                   int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
+                   const tw_epilogue *ep, void *stream);
+
 /* Process-wide tuning switches of tw_gemm / tw_gemm_ex; value -1 restores the automatic choice.
  * The launch configuration is otherwise picked from the plan and M.  The reference fixes its one
  * configuration at compile time (Volta884GemmTraits<..., Shape<32,128,128>, ...>,

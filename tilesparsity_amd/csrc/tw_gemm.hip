@@ -1546,6 +1546,12 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
 
 using namespace tw;
 
+// Launch-time scratch of tw_gemm_static: the work-queue counters of one launch.  One copy per
+// GPU, held until the process ends; every tw_gemm_static call on a GPU uses it.
+constexpr int kStaticScratchInts = 64; // 256 bytes, of which kTicketInts counters are used
+static_assert(kStaticScratchInts >= kTicketInts, "the counters of a launch fit the static scratch");
+static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
 extern "C" {
 
 int tw_set_option(int option_id, int value)
@@ -1632,6 +1638,9 @@ void fill_common(GemmArgs &a, const tw_plan *plan, const void *A, int64_t lda, v
     a.n_arg_units = 0;
 }
 
+// work items of a launch are counted in 32-bit integers
+constexpr int64_t kMaxItems = 0x7fffffff;
+
 // item matrix and queues of a launch with `bm`-row items and unit pieces of `piece` columns
 void fill_queues(GemmArgs &a, const tw_plan *plan, int M, int bm, int piece, int pruned_cols, bool xcd)
 {
@@ -1669,11 +1678,38 @@ int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *tick
     return TW_OK;
 }
 
-} // namespace
+__global__ void clear_counters_kernel(int32_t *counters)
+{
+    if (threadIdx.x < kTicketInts)
+        counters[threadIdx.x] = 0;
+}
 
-int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
-               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
-               void *stream)
+// Device address of `scratch` on the current device, looked up once per device (the array's name
+// is only a host-side stand-in; every GPU holds its own copy at its own address).
+int static_scratch(int32_t **out)
+{
+    constexpr int kMaxDevices = 64;
+    static std::mutex mu;
+    static int32_t *ptr[kMaxDevices] = {};
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(TW_ERR_DEVICE, "device %d: tw_gemm_static serves devices 0..%d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptr[dev]) {
+        void *p = nullptr;
+        TW_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        ptr[dev] = static_cast<int32_t *>(p);
+    }
+    *out = ptr[dev];
+    return TW_OK;
+}
+
+// tw_gemm_ex and tw_gemm_static: the latter brings the counters (`static_ticket`), cleared on the
+// stream before the launch; the former takes a ticket slot of the plan.
+int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
+              int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
+              void *stream, bool use_static)
 {
     bool run = false;
     const int st = check_gemm_args(plan, A, a_layout, lda, C, c_layout, ldc, M, pruned_cols, ep, &run);
@@ -1687,6 +1723,9 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
         const int64_t n_items = (int64_t)a.n_all_u * a.n_mblk;
         if (n_items == 0)
             return TW_OK;
+        if (n_items > kMaxItems)
+            return fail(TW_ERR_SHAPE, "%lld work items (M=%d): a launch takes at most %lld",
+                        (long long)n_items, M, (long long)kMaxItems);
         const int64_t sa_m = a_layout == TW_LAYOUT_KMAJOR ? 1 : lda;
         const int64_t sa_k = a_layout == TW_LAYOUT_KMAJOR ? lda : 1;
         const int64_t sc_m = c_layout == TW_LAYOUT_KMAJOR ? 1 : ldc;
@@ -1703,11 +1742,27 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
 
     const Choice c = choose_shape(plan, M, lda);
     fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
+    if ((int64_t)a.n_all_u * a.n_mblk > kMaxItems)
+        return fail(TW_ERR_SHAPE, "%lld work items (M=%d): a launch takes at most %lld",
+                    (long long)a.n_all_u * a.n_mblk, M, (long long)kMaxItems);
     // an output larger than one L2 is written through (see store_chunk)
     a.store_through = (int64_t)M * plan->N * 2 > kStoreThroughBytes;
     // Ticket slot of this launch.  A launch recorded into a HIP graph keeps its slot for every
     // replay, so recorded launches draw from a range of their own that eager launches never use.
     hipStream_t s = (hipStream_t)stream;
+    if (use_static) {
+        // the counters must start at zero: cleared with a kernel (a launch can then be recorded
+        // into a graph), whatever the last call on this GPU left in them
+        int32_t *counters = nullptr;
+        const int sst = static_scratch(&counters);
+        if (sst != TW_OK)
+            return sst;
+        if (a.n_all_u == 0)
+            return TW_OK;
+        hipLaunchKernelGGL(clear_counters_kernel, dim3(1), dim3(64), 0, s, counters);
+        TW_HIP(hipGetLastError());
+        return launch_gemm(plan, a, c, counters, s);
+    }
     hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
     if (hipStreamIsCapturing(s, &cap) != hipSuccess) {
         (void)hipGetLastError();
@@ -1720,6 +1775,24 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
     else
         slot = __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kEagerSlots;
     return launch_gemm(plan, a, c, plan->d_tickets + kTicketInts * slot, s);
+}
+
+} // namespace
+
+int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
+               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
+               void *stream)
+{
+    return gemm_impl(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep, stream,
+                     false);
+}
+
+int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
+                   int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
+                   const tw_epilogue *ep, void *stream)
+{
+    return gemm_impl(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep, stream,
+                     true);
 }
 
 int tw_stream_gemm_nn(int M, int N, int K, int dtype, float alpha, const void *A, const void *B,

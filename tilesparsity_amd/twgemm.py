@@ -49,7 +49,7 @@ EXPORTED_SYMBOLS = (
     "tw_tiles_every_g_columns", "tw_tiles_every_g_kept_columns",
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
-    "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option",
+    "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
 )
 
 
@@ -122,6 +122,8 @@ def lib():
         "tw_gemm": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int, vp]),
         "tw_gemm_ex": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int,
                                ctypes.POINTER(Epilogue), vp]),
+        "tw_gemm_static": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int,
+                                   ctypes.POINTER(Epilogue), vp]),
         "tw_stream_gemm_nn": (c_int, [c_int, c_int, c_int, c_int, c_f, vp, vp, c_f, vp, c_int,
                                       i32p, i32p, pp, pp, i64p, i64p, vp]),
         "tw_cast_f32": (c_int, [vp, vp, c_i64, c_int, vp]),
@@ -403,20 +405,23 @@ class Plan:
     # -- the GEMM
     def gemm(self, A_ptr, C_ptr, M, lda=None, ldc=None, alpha=1.0, beta=0.0,
              a_layout=KMAJOR, c_layout=KMAJOR, pruned_cols=PRUNED_UNTOUCHED, stream=0,
-             bias_ptr=None, activation=ACT_NONE):
+             bias_ptr=None, activation=ACT_NONE, static=False):
         """C = act(alpha * A (B (.) mask) + beta * C + bias) on device pointers; asynchronous.
-        bias_ptr: device fp32 [N] or None; activation: ACT_NONE / ACT_RELU / ACT_GELU / ACT_TANH."""
+        bias_ptr: device fp32 [N] or None; activation: ACT_NONE / ACT_RELU / ACT_GELU / ACT_TANH.
+        static=True goes through tw_gemm_static (work-queue counters in the library's own device
+        array; calls that overlap on one GPU race)."""
         if lda is None:
             lda = M if a_layout == KMAJOR else self.K
         if ldc is None:
             ldc = M if c_layout == KMAJOR else self.N
-        if bias_ptr is None and activation == ACT_NONE:
+        if bias_ptr is None and activation == ACT_NONE and not static:
             _check(lib().tw_gemm(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
                                  ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
                                  pruned_cols, ctypes.c_void_p(int(stream or 0))))
             return
         ep = Epilogue(ctypes.c_void_p(int(bias_ptr or 0)), int(activation))
-        _check(lib().tw_gemm_ex(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
+        fn = lib().tw_gemm_static if static else lib().tw_gemm_ex
+        _check(fn(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
                                 ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
                                 pruned_cols, ctypes.byref(ep), ctypes.c_void_p(int(stream or 0))))
 

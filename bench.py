@@ -47,27 +47,81 @@ def make_workload(name):
     return table[name]()
 
 
-def time_plan(plan, bufs, M, steps, warmup, torch):
-    """Average seconds per launch over `steps` back-to-back launches, timed with events on
-    the stream the kernel runs on; buffers rotate so that A and C come from HBM."""
+def time_steps(launch, steps, warmup, torch):
+    """Average seconds per step over exactly `steps` back-to-back calls of launch(i), timed with
+    events on the stream the kernels run on, after `warmup` untimed calls."""
     stream = torch.cuda.current_stream()
-    s = stream.cuda_stream
-    n = len(bufs)
     for i in range(warmup):
-        a, c = bufs[i % n]
-        plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+        launch(i)
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record(stream)
     for i in range(steps):
-        a, c = bufs[i % n]
-        plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+        launch(i)
     stop.record(stream)
     torch.cuda.synchronize()
     return start.elapsed_time(stop) * 1e-3 / steps
 
 
-def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20):
+def time_plan(plan, bufs, M, steps, warmup, torch):
+    """Seconds per launch of a plan; buffers rotate so that A and C come from HBM."""
+    s = torch.cuda.current_stream().cuda_stream
+    n = len(bufs)
+
+    def launch(i):
+        a, c = bufs[i % n]
+        plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+    return time_steps(launch, steps, warmup, torch)
+
+
+def time_plan_graph(plan, bufs, M, steps, warmup, torch):
+    """The same with the `steps` launches recorded once into a HIP graph and the graph replayed:
+    for launches of a few microseconds, which the host cannot issue as fast as the GPU runs them
+    (the NMT recurrence: 50 time steps back to back with fixed weights)."""
+    n = len(bufs)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            for i in range(steps):
+                a, c = bufs[i % n]
+                plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    for _ in range(max(1, warmup // max(1, steps) + 1)):
+        graph.replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(stream)
+    graph.replay()          # exactly `steps` launches
+    stop.record(stream)
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
+def roofline_of(M, K, N, tiles, t, traffic=None):
+    """Roofline block of one launch that took t seconds: the binding roof is the larger of the
+    ideal HBM time (algorithmic bytes at 8 TB/s) and the ideal MFMA time (kept flops at the dense
+    16-bit peak)."""
+    from tilesparsity_amd import workloads as W
+    by, fk = W.algorithmic_bytes(M, K, N, tiles), W.flops_kept(M, tiles)
+    if by / (HBM_PEAK_GBS * 1e9) >= fk / (MFMA_PEAK_TFLOPS * 1e12):
+        ach = by / t / 1e9
+        return {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": ach / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes": by}
+    ach = fk / t / 1e12
+    return {"bound": "mfma", "achieved": ach, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+            "frac": ach / MFMA_PEAK_TFLOPS, "traffic": traffic, "algorithmic_flops": fk}
+
+
+def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, graph=False):
+    """Times the TW plan (`steps` launches after `warmup`: the headline figure), then `repeats`
+    more rounds of the same length each for the TW plan, for the 0 %-sparse plan of the same
+    kernel and for the library's dense GEMM (torch.matmul, i.e. hipBLASLt / rocBLAS) on the same
+    operands, layout and rotating buffers; the ratios are taken between the medians."""
     from tilesparsity_amd import twgemm as tw
     from tilesparsity_amd import workloads as W
     M, K, N, G, dtype, tiles = wl["M"], wl["K"], wl["N"], wl["G"], wl["dtype"], wl["tiles"]
@@ -81,22 +135,36 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20):
             for i in range(n_sets)]
     sparse = tw.Plan.create(K, N, dtype, tiles, B)
     dense = tw.Plan.dense(K, N, G, dtype, B)
-    t_sparse = time_plan(sparse, bufs, M, steps, warmup, torch)
-    t_dense = time_plan(dense, bufs, M, max(3, steps // 4), max(2, warmup // 4), torch)
+    timer = time_plan_graph if graph else time_plan
+    t_sparse = timer(sparse, bufs, M, steps, warmup, torch)
+    reps_sparse = [timer(sparse, bufs, M, steps, 2, torch) for _ in range(repeats)]
+    reps_dense = [timer(dense, bufs, M, steps, 2, torch) for _ in range(repeats)]
     sparse.destroy()
     dense.destroy()
+    # the library's dense GEMM in the same layout: C^T [N, M] = W^T [N, K] . A^T [K, M]
+    Wt = torch.from_numpy(np.ascontiguousarray(B.T)).cuda().to(tdt)
+
+    def lib_launch(i):
+        a, c = bufs[i % n_sets]
+        torch.matmul(Wt, a, out=c)
+    reps_lib = [time_steps(lib_launch, steps, 2, torch) for _ in range(repeats)]
+    t_sp, t_de, t_lib = (float(np.median(x)) for x in (reps_sparse, reps_dense, reps_lib))
     fk, fd = W.flops_kept(M, tiles), W.flops_dense(M, K, N)
     by = W.algorithmic_bytes(M, K, N, tiles)
     res = dict(
         workload=wl["name"], M=M, K=K, N=N, G=G, dtype=dtype, seed=wl["seed"], n_tiles=len(tiles),
-        us_sparse=t_sparse * 1e6, us_dense=t_dense * 1e6,
+        us_sparse=t_sparse * 1e6, us_sparse_median=t_sp * 1e6, us_dense=t_de * 1e6,
+        us_dense_library=t_lib * 1e6, timed_with="hip graph replay" if graph else "stream launches",
+        repeats=repeats,
         effective_tflops=fd / t_sparse / 1e12, actual_tflops=fk / t_sparse / 1e12,
-        dense_tflops=fd / t_dense / 1e12, speedup_vs_dense=t_dense / t_sparse,
+        dense_tflops=fd / t_de / 1e12, dense_library_tflops=fd / t_lib / 1e12,
+        speedup_vs_dense=t_de / t_sp, speedup_vs_dense_library=t_lib / t_sp,
         mfma_util_kept=fk / t_sparse / 1e12 / MFMA_PEAK_TFLOPS,
-        mfma_util_dense_run=fd / t_dense / 1e12 / MFMA_PEAK_TFLOPS,
+        mfma_util_dense_run=fd / t_de / 1e12 / MFMA_PEAK_TFLOPS,
         algorithmic_bytes=by, hbm_gbs=by / t_sparse / 1e9, rotating_buffer_sets=n_sets,
-        kept_flops=fk, dense_flops=fd)
-    del bufs, At
+        kept_flops=fk, dense_flops=fd,
+        roofline=roofline_of(M, K, N, tiles, t_sparse))
+    del bufs, At, Wt
     torch.cuda.empty_cache()
     return res, (A, B)
 
@@ -318,6 +386,8 @@ def main():
 
     wl = make_workload(args.workload)
     res, (A, B) = run_workload(wl, args.steps, args.warmup, torch)
+    roof = dict(res["roofline"])
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
     out = {
         "metric": "effective TFLOP/s (dense flops / time) at 75% TW sparsity, G=128",
         "value": res["effective_tflops"], "unit": "TFLOP/s", "n_gpus": 1,
@@ -327,28 +397,39 @@ def main():
         "config": {"workload": "%s M=%d K=%d N=%d G=%d, %d tiles, seed %d" % (
             wl["name"], wl["M"], wl["K"], wl["N"], wl["G"], len(wl["tiles"]), wl["seed"])},
         "speedup_vs_dense_plan": res["speedup_vs_dense"],
+        "speedup_vs_dense_library": res["speedup_vs_dense_library"],
         "actual_tflops": res["actual_tflops"], "dense_plan_tflops": res["dense_tflops"],
+        "dense_library_tflops": res["dense_library_tflops"],
         "mfma_utilisation_kept_flops": res["mfma_util_kept"],
         "mfma_utilisation_dense_run": res["mfma_util_dense_run"],
-        "us_sparse": res["us_sparse"], "us_dense": res["us_dense"],
-        "roofline": {"bound": "hbm", "achieved": res["hbm_gbs"], "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": res["hbm_gbs"] / HBM_PEAK_GBS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "algorithmic_bytes": res["algorithmic_bytes"]},
+        "us_sparse": res["us_sparse"], "us_sparse_median": res["us_sparse_median"],
+        "us_dense": res["us_dense"], "us_dense_library": res["us_dense_library"],
+        "repeats_for_medians": res["repeats"],
+        "roofline": roof,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, A, B)
     del A, B
+    # the other shapes the target names: BERT-base FFN (small K per tile) and the NMT gate GEMM
+    # (skinny M; its 50 time steps are recorded into a graph and replayed), each with the
+    # roofline of its own launch; --all adds the remaining configurations
+    names = ["bert_base_ffn", "nmt_lstm_gates"]
     if args.all:
-        others = {}
-        for name in ("bert_base_ffn", "nmt_lstm_gates", "bert_large_ffn1_50", "bert_large_ffn1_75",
-                     "bert_large_ffn1_90", "bert_large_ffn2_50", "bert_large_ffn2_75",
-                     "bert_large_ffn2_90", "imbalance_stress"):
-            r, _ = run_workload(make_workload(name), args.steps, args.warmup, torch)
-            others[name] = {k: r[k] for k in ("us_sparse", "us_dense", "effective_tflops",
-                                              "actual_tflops", "dense_tflops", "speedup_vs_dense",
-                                              "mfma_util_kept", "hbm_gbs", "dtype")}
-            print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
+        names += ["bert_large_ffn1_50", "bert_large_ffn1_75", "bert_large_ffn1_90",
+                  "bert_large_ffn2_50", "bert_large_ffn2_75", "bert_large_ffn2_90", "imbalance_stress"]
+    if args.workload != "vgg16_conv4_2":
+        names = []
+    others = {}
+    for name in names:
+        nmt = name == "nmt_lstm_gates"
+        r, _ = run_workload(make_workload(name), 50 if nmt else args.steps, args.warmup, torch,
+                            repeats=3, graph=nmt)
+        others[name] = {k: r[k] for k in ("us_sparse", "us_sparse_median", "us_dense",
+                                          "us_dense_library", "effective_tflops", "actual_tflops",
+                                          "speedup_vs_dense", "speedup_vs_dense_library",
+                                          "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "roofline")}
+        print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
+    if others:
         out["other_workloads"] = others
     print(json.dumps(out), flush=True)
     return 0

@@ -284,7 +284,8 @@ int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_SHAPE_128x64 3  /* wave-specialised, 128 x 64 */
 #define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU */
 #define TW_SHAPE_128x32 5  /* wave-specialised, 128 x 32: skinny M */
-#define TW_N_SHAPES 6
+#define TW_SHAPE_256x64 6  /* wave-specialised, 256 x 64 */
+#define TW_N_SHAPES 7
 int tw_set_option(int option, int value);
 
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument

@@ -34,7 +34,9 @@ by tests/golden/make_prune_vectors.py from Pruning/VGG/prune_algo.py under the N
 image (2.2.6).  The reference's published environment used an older NumPy whose percentile
 interpolates in float64 for every input; the two can differ only when a norm ties with the
 threshold to the last bit.  granularity_pruning has no vectors from the reference (MyHook.py
-imports TensorFlow, which this image lacks): parity unpinned beyond its property tests.
+imports TensorFlow, which this image lacks); it is pinned by a brute-force check on small inputs
+(norms by plain sums, the percentile from the two order statistics by hand, kept rows = those
+strictly above it) and by its one-tile case, which must keep the rows tiled_wise_1d keeps.
 """
 import numpy as np
 

@@ -1386,6 +1386,7 @@ static const Shape kShapes[TW_N_SHAPES] = {
     {128, 64, 2},  // TW_SHAPE_128x64
     {256, 128, 1}, // TW_SHAPE_256x128
     {128, 32, 2},  // TW_SHAPE_128x32
+    {256, 64, 1},  // TW_SHAPE_256x64
 };
 
 // Steps of loads a moving wave keeps in flight, per shape (bounded by its 256 registers: a step
@@ -1402,6 +1403,9 @@ static const Shape kShapes[TW_N_SHAPES] = {
 #endif
 #ifndef TW_R_128x64
 #define TW_R_128x64 2
+#endif
+#ifndef TW_R_256x64
+#define TW_R_256x64 3
 #endif
 #ifndef TW_R_128x32
 #define TW_R_128x32 2
@@ -1424,6 +1428,9 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
         break;
     case TW_SHAPE_128x32:
         hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 32, TW_R_128x32>), dim3(grid), dim3(256), 0, s, a);
+        break;
+    case TW_SHAPE_256x64:
+        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 64, TW_R_256x64>), dim3(grid), dim3(512), 0, s, a);
         break;
     default: // TW_SHAPE_256x128
         hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128, TW_R_256x128>), dim3(grid), dim3(512), 0, s, a);
@@ -1515,6 +1522,8 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
         c.piece = 64;
         if (items(512, 64) * 5 >= 3 * cu) {
             c.shape = TW_SHAPE_512x64;
+        } else if (items(256, 64) * 5 >= 3 * cu) {
+            c.shape = TW_SHAPE_256x64;
         } else if (items(128, 64) * 2 >= cu) {
             c.shape = TW_SHAPE_128x64;
         } else {

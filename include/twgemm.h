@@ -158,12 +158,13 @@ int tw_plan_from_mask_cover(int K, int N, int dtype, int n_tiles, const int32_t 
 /* The same pre-pass on DEVICE operands: mask (K x N bytes) and B (fp32, row-major) are device
  * memory, e.g. the masks tw_prune_* leave on the device and a weight that already lives there, so
  * nothing but the tile table, the list lengths and the lists' host copies crosses the host
- * boundary.  cover != 0 as tw_plan_from_mask_cover, else as tw_plan_from_mask_tiles.  The call
- * works on the default stream and returns when the plan is complete; work that writes mask or B
- * on a stream that does not synchronise with the default stream must have finished before. */
+ * boundary.  cover != 0 as tw_plan_from_mask_cover, else as tw_plan_from_mask_tiles.  Every
+ * kernel and copy of the build runs on `stream` (a hipStream_t, NULL = the default stream), after
+ * whatever produced mask and B on that stream; the call waits for that stream and returns when
+ * the plan is complete. */
 int tw_plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                              const int32_t *tile_width, const uint8_t *mask, const float *B,
-                             int cover, tw_plan **out);
+                             int cover, void *stream, tw_plan **out);
 
 /* Build a plan from one layer of the reference's exported pruned model (exportPrunedModel,
  * Pruning/BERT/utils/MyHook.py:54-89): mask_i / mask_o are the relative offsets

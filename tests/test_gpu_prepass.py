@@ -110,6 +110,21 @@ def test_delete_insert_row_kernels(tw):
     expect = np.zeros_like(src)
     expect[kept] = src[kept]
     assert np.array_equal(from_device_bits(d_back), expect)
+    # more rows than one grid dimension holds (the reference's kernels take any row count)
+    rows, cols, n_keep = 70000, 9, 66000
+    src = rng.integers(0, 65536, (rows, cols)).astype(np.uint16)
+    kept = np.sort(rng.choice(rows, n_keep, replace=False)).astype(np.int32)
+    rel = torch.from_numpy(kept - np.arange(n_keep, dtype=np.int32)).cuda()
+    d_src = to_device_bits(src, (rows, cols))
+    d_out = torch.zeros((n_keep, cols), dtype=torch.int16, device="cuda")
+    tw.delete_row(d_src.data_ptr(), d_out.data_ptr(), n_keep, cols, rel.data_ptr())
+    d_back = torch.zeros((rows, cols), dtype=torch.int16, device="cuda")
+    tw.insert_row(d_back.data_ptr(), d_out.data_ptr(), n_keep, cols, rel.data_ptr())
+    torch.cuda.synchronize()
+    assert np.array_equal(from_device_bits(d_out), src[kept])
+    expect = np.zeros_like(src)
+    expect[kept] = src[kept]
+    assert np.array_equal(from_device_bits(d_back), expect)
 
 
 def test_device_operands_give_the_same_plan(tw, oracle):
@@ -146,6 +161,16 @@ def test_device_operands_give_the_same_plan(tw, oracle):
             (td, bd), (th, bh) = pd.export(), ph.export()
             assert np.array_equal(bd, bh)
             assert np.array_equal(bd, oracle.cast_bits(oracle.stream_weight(np.where(m != 0, W, np.float32(0)), po.cover_tiles_from_mask(m, table)), "bf16"))
+        # on a stream of the caller: the mask is produced on that stream right before the build
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            dm2 = torch.zeros_like(dm)
+            dm2.copy_(dm)
+            with tw.Plan.from_device_mask(K, N, dm2.data_ptr(), table, "bf16", dW.data_ptr(), cover=True,
+                                          stream=side.cuda_stream) as ps:
+                _, bs = ps.export()
+        assert np.array_equal(bs, bd)
     with pytest.raises(tw.TwError):
         tw.Plan.from_device_mask(8, 8, 0, [(0, 8)], "f16", 0)
 

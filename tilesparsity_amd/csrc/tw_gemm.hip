@@ -1345,29 +1345,30 @@ __global__ void __launch_bounds__(256, 2) tw_gemm_generic_kernel(const GemmArgs 
 
 __global__ void cast_f32_kernel(const float *src, uint16_t *dst, int64_t n, int dtype)
 {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= n) // strict bound; the reference's `idx > n` writes one element too many
-        return;
-    dst[i] = dtype == TW_BF16 ? (uint16_t)Elem<TW_BF16>::to_bits(src[i])
-                              : (uint16_t)Elem<TW_F16>::to_bits(src[i]);
+    // strict bound (the reference's `idx > n` writes one element too many); grid-stride, so any n
+    // fits a launch
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+         i += (int64_t)gridDim.x * blockDim.x)
+        dst[i] = dtype == TW_BF16 ? (uint16_t)Elem<TW_BF16>::to_bits(src[i])
+                                  : (uint16_t)Elem<TW_F16>::to_bits(src[i]);
 }
 
 __global__ void delete_row_kernel(const uint16_t *matrix, uint16_t *matrix_2, int rows, int columns,
                                   const int32_t *mask)
 {
     const int j = blockIdx.x * blockDim.x + threadIdx.x;
-    const int i = blockIdx.y;
-    if (i < rows && j < columns)
-        matrix_2[(int64_t)i * columns + j] = matrix[(int64_t)(i + mask[i]) * columns + j];
+    if (j < columns)
+        for (int i = blockIdx.y; i < rows; i += gridDim.y) // any row count fits a launch
+            matrix_2[(int64_t)i * columns + j] = matrix[(int64_t)(i + mask[i]) * columns + j];
 }
 
 __global__ void insert_row_kernel(uint16_t *matrix, const uint16_t *matrix_2, int rows, int columns,
                                   const int32_t *mask)
 {
     const int j = blockIdx.x * blockDim.x + threadIdx.x;
-    const int i = blockIdx.y;
-    if (i < rows && j < columns)
-        matrix[(int64_t)(i + mask[i]) * columns + j] = matrix_2[(int64_t)i * columns + j];
+    if (j < columns)
+        for (int i = blockIdx.y; i < rows; i += gridDim.y)
+            matrix[(int64_t)(i + mask[i]) * columns + j] = matrix_2[(int64_t)i * columns + j];
 }
 
 // outputs above this size are written through to memory: the size of one XCD's L2
@@ -1839,7 +1840,7 @@ int tw_cast_f32(const float *src, void *dst, int64_t n, int dtype, void *stream)
         return TW_OK;
     if (!src || !dst)
         return fail(TW_ERR_NULL, "src or dst is NULL");
-    hipLaunchKernelGGL(cast_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+    hipLaunchKernelGGL(cast_f32_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 1 << 20)), dim3(256), 0,
                        (hipStream_t)stream, src, (uint16_t *)dst, n, dtype);
     TW_HIP(hipGetLastError());
     return TW_OK;
@@ -1854,7 +1855,7 @@ int tw_delete_row(const void *matrix, void *matrix_2, int rows, int columns, con
         return TW_OK;
     if (!matrix || !matrix_2 || !mask)
         return fail(TW_ERR_NULL, "matrix, matrix_2 or mask is NULL");
-    hipLaunchKernelGGL(delete_row_kernel, dim3((columns + 255) / 256, rows), dim3(256), 0,
+    hipLaunchKernelGGL(delete_row_kernel, dim3((columns + 255) / 256, std::min(rows, 65535)), dim3(256), 0,
                        (hipStream_t)stream, (const uint16_t *)matrix, (uint16_t *)matrix_2, rows,
                        columns, mask);
     TW_HIP(hipGetLastError());
@@ -1870,7 +1871,7 @@ int tw_insert_row(void *matrix, const void *matrix_2, int rows, int columns, con
         return TW_OK;
     if (!matrix || !matrix_2 || !mask)
         return fail(TW_ERR_NULL, "matrix, matrix_2 or mask is NULL");
-    hipLaunchKernelGGL(insert_row_kernel, dim3((columns + 255) / 256, rows), dim3(256), 0,
+    hipLaunchKernelGGL(insert_row_kernel, dim3((columns + 255) / 256, std::min(rows, 65535)), dim3(256), 0,
                        (hipStream_t)stream, (uint16_t *)matrix, (const uint16_t *)matrix_2, rows,
                        columns, mask);
     TW_HIP(hipGetLastError());

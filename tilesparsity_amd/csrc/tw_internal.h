@@ -152,8 +152,9 @@ int validate_lists(int K, int N, int n_tiles, const int32_t *tile_col0, const in
                    const int32_t *kept_n_ptr, const int32_t *kept_n_idx);
 
 // fills the host-side geometry (k_pad, n_pad, b_off, packed_elems) of a plan whose
-// lists are set, uploads lists/units/tiles and allocates the packed weight (zeroed).
-int finalize_plan_geometry(tw_plan *p);
+// lists are set, uploads lists/units/tiles and allocates the packed weight (zeroed); the copies
+// run on `s`, which is waited for.
+int finalize_plan_geometry(tw_plan *p, hipStream_t s);
 
 // device pack: packed weight from a row-major fp32 [K,N] device buffer
 int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s, const uint8_t *d_mask = nullptr);

@@ -519,7 +519,41 @@ template <typename T> static int upload(T **dst, const std::vector<T> &src)
     return TW_OK;
 }
 
-int finalize_plan_geometry(tw_plan *p)
+static void free_plan(tw_plan *p);
+
+// Owners of what a builder holds until it succeeds: whatever path leaves the builder (an error
+// return, an exception on its way to the status conversion), the device buffer and the
+// half-built plan are released.
+struct DeviceBuffer {
+    void *ptr = nullptr;
+    DeviceBuffer() = default;
+    DeviceBuffer(const DeviceBuffer &) = delete;
+    DeviceBuffer &operator=(const DeviceBuffer &) = delete;
+    ~DeviceBuffer()
+    {
+        if (ptr)
+            (void)hipFree(ptr);
+    }
+};
+struct PlanOwner {
+    tw_plan *p = nullptr;
+    PlanOwner() = default;
+    PlanOwner(const PlanOwner &) = delete;
+    PlanOwner &operator=(const PlanOwner &) = delete;
+    ~PlanOwner()
+    {
+        if (p)
+            free_plan(p);
+    }
+    tw_plan *release()
+    {
+        tw_plan *r = p;
+        p = nullptr;
+        return r;
+    }
+};
+
+int finalize_plan_geometry(tw_plan *p, hipStream_t s)
 {
     const int nt = p->n_tiles;
     p->k_pad.assign(nt, 0);
@@ -641,12 +675,12 @@ int finalize_plan_geometry(tw_plan *p)
     if (hipMalloc((void **)&slab, o_bp + bp_bytes) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the plan failed", o_bp + bp_bytes);
     p->d_slab = slab;
-    TW_HIP(hipMemcpy(slab, stage.data(), stage.size(), hipMemcpyHostToDevice));
-    // asynchronous: the packing kernel follows on the same (default) stream and the builders wait
-    // for it; a plan with nothing to pack waits here
-    TW_HIP(hipMemsetAsync(slab + o_tickets, 0, o_bp + bp_bytes - o_tickets, nullptr));
-    if (p->packed_elems == 0)
-        TW_HIP(hipStreamSynchronize(nullptr));
+    TW_HIP(hipMemcpyAsync(slab, stage.data(), stage.size(), hipMemcpyHostToDevice, s));
+    // the packing kernel follows on the same stream and the builders wait for it; a plan with
+    // nothing to pack waits here (the staged tables are host memory of this call: wait either way
+    // before they go out of scope)
+    TW_HIP(hipMemsetAsync(slab + o_tickets, 0, o_bp + bp_bytes - o_tickets, s));
+    TW_HIP(hipStreamSynchronize(s));
     p->d_units = reinterpret_cast<UnitDev *>(slab + o_units);
     p->d_tiles = reinterpret_cast<TileDev *>(slab + o_tiles);
     p->d_pruned_n = reinterpret_cast<int32_t *>(slab + o_pruned);
@@ -705,13 +739,14 @@ int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStre
     int st = upload(&d_pt, pt);
     if (st)
         return st;
+    DeviceBuffer pt_owner;
+    pt_owner.ptr = d_pt;
     dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
     hipLaunchKernelGGL(pack_stream_kernel, grid, dim3(256), 0, s, d_pt, (const uint16_t *)d_Bs,
                        p->K, (uint16_t *)p->d_Bp);
     hipError_t e = hipGetLastError();
     if (e == hipSuccess)
         e = hipStreamSynchronize(s);
-    hipFree(d_pt);
     if (e != hipSuccess)
         return fail(TW_ERR_DEVICE, "stream-weight packing kernel failed: %s", hipGetErrorString(e));
     return TW_OK;
@@ -727,13 +762,14 @@ int unpack_to_stream(const tw_plan *p, uint16_t *d_Bs, hipStream_t s)
         int st = upload(&d_pt, pt);
         if (st)
             return st;
+        DeviceBuffer pt_owner;
+        pt_owner.ptr = d_pt;
         dim3 grid((unsigned)((mg + 255) / 256), (unsigned)p->n_tiles);
         hipLaunchKernelGGL(unpack_stream_kernel, grid, dim3(256), 0, s, d_pt,
                            (const uint16_t *)p->d_Bp, p->K, d_Bs);
         hipError_t e = hipGetLastError();
         if (e == hipSuccess)
             e = hipStreamSynchronize(s);
-        hipFree(d_pt);
         if (e != hipSuccess)
             return fail(TW_ERR_DEVICE, "unpack kernel failed: %s", hipGetErrorString(e));
     }
@@ -762,15 +798,13 @@ static int pack_host_weight(tw_plan *p, const float *B)
 {
     if (p->packed_elems == 0)
         return TW_OK;
-    float *d_B = nullptr;
+    DeviceBuffer d_B;
     size_t bytes = (size_t)p->K * p->N * sizeof(float);
-    if (hipMalloc((void **)&d_B, bytes) != hipSuccess)
+    if (hipMalloc(&d_B.ptr, bytes) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the weight upload failed", bytes);
-    hipError_t e = hipMemcpy(d_B, B, bytes, hipMemcpyHostToDevice);
-    int st = e == hipSuccess ? pack_from_dense(p, d_B, nullptr)
-                             : fail(TW_ERR_DEVICE, "weight upload failed: %s", hipGetErrorString(e));
-    hipFree(d_B);
-    return st;
+    hipError_t e = hipMemcpy(d_B.ptr, B, bytes, hipMemcpyHostToDevice);
+    return e == hipSuccess ? pack_from_dense(p, static_cast<const float *>(d_B.ptr), nullptr)
+                           : fail(TW_ERR_DEVICE, "weight upload failed: %s", hipGetErrorString(e));
 }
 
 } // namespace tw
@@ -796,7 +830,8 @@ try {
         return st;
     if (!B)
         return fail(TW_ERR_NULL, "B is NULL");
-    tw_plan *p = new (std::nothrow) tw_plan;
+    PlanOwner owner;
+    tw_plan *p = owner.p = new (std::nothrow) tw_plan;
     if (!p)
         return fail(TW_ERR_ALLOC, "out of host memory");
     p->K = K;
@@ -809,11 +844,9 @@ try {
     p->kept_n_ptr.assign(kept_n_ptr, kept_n_ptr + n_tiles + 1);
     p->kept_k_idx.assign(kept_k_idx, kept_k_idx + kept_k_ptr[n_tiles]);
     p->kept_n_idx.assign(kept_n_idx, kept_n_idx + kept_n_ptr[n_tiles]);
-    if ((st = finalize_plan_geometry(p)) || (st = pack_host_weight(p, B))) {
-        free_plan(p);
+    if ((st = finalize_plan_geometry(p, nullptr)) || (st = pack_host_weight(p, B)))
         return st;
-    }
-    *out = p;
+    *out = owner.release();
     return TW_OK;
 }
 TW_CATCH_TO_STATUS
@@ -867,7 +900,7 @@ TW_CATCH_TO_STATUS
 // device memory.  Temporaries (flags, counters, the tile table) share one allocation.
 static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                                  const int32_t *tile_width, const uint8_t *d_mask, const float *d_B,
-                                 bool cover, tw_plan **out)
+                                 bool cover, hipStream_t s, tw_plan **out)
 {
     if (!out)
         return fail(TW_ERR_NULL, "out is NULL");
@@ -911,28 +944,21 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     const size_t o_counts = o_mismatch + up(sizeof(unsigned long long));
     const size_t o_tcol0 = o_counts + up(sizeof(int32_t) * n_seg);
     const size_t ws_bytes = o_tcol0 + up(sizeof(int32_t) * (nt + 1));
-    char *ws = nullptr;
-    tw_plan *p = nullptr;
-    auto cleanup = [&]() { hipFree(ws); };
-#define TW_TRY(call)                                                                       \
-    do {                                                                                   \
-        hipError_t e_ = (call);                                                            \
-        if (e_ != hipSuccess) {                                                            \
-            cleanup();                                                                     \
-            free_plan(p);                                                                  \
-            return fail(TW_ERR_DEVICE, "%s failed: %s", #call, hipGetErrorString(e_));     \
-        }                                                                                  \
-    } while (0)
-
-    TW_TRY(hipMalloc((void **)&ws, ws_bytes));
+    // the workspace and the half-built plan are released on every way out of this function;
+    // every kernel and copy runs on the caller's stream, which this function waits for
+    DeviceBuffer ws_owner;
+    PlanOwner owner;
+#define TW_TRY(call) TW_HIP(call)
+    TW_TRY(hipMalloc(&ws_owner.ptr, ws_bytes));
+    char *const ws = static_cast<char *>(ws_owner.ptr);
     uint8_t *d_rowflag = reinterpret_cast<uint8_t *>(ws + o_rowflag);
     uint8_t *d_colflag = reinterpret_cast<uint8_t *>(ws + o_colflag);
     unsigned long long *d_mismatch = reinterpret_cast<unsigned long long *>(ws + o_mismatch);
     int32_t *d_seg_counts = reinterpret_cast<int32_t *>(ws + o_counts);
     int32_t *d_tcol0 = reinterpret_cast<int32_t *>(ws + o_tcol0);
-    TW_TRY(hipMemcpy(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice));
+    TW_TRY(hipMemcpyAsync(d_tcol0, tcol0.data(), sizeof(int32_t) * (nt + 1), hipMemcpyHostToDevice, s));
     // row flags, column flags and the mismatch counter start at zero (adjacent in the workspace)
-    TW_TRY(hipMemsetAsync(ws, 0, o_counts, nullptr));
+    TW_TRY(hipMemsetAsync(ws, 0, o_counts, s));
 
     const dim3 seg_grid((unsigned)nt, (unsigned)(n_seg_k + n_seg_n));
     {
@@ -941,32 +967,30 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
         const int nchunk = (N + 15) / 16;
         const int cw = nchunk > 32 ? 64 : (nchunk > 16 ? 32 : 16);
         const dim3 grid((unsigned)((nchunk + cw - 1) / cw), (unsigned)((K + 63) / 64));
-        hipLaunchKernelGGL(mask_flags_kernel, grid, dim3(256), 0, nullptr, d_mask, K, N, d_tcol0, nt,
+        hipLaunchKernelGGL(mask_flags_kernel, grid, dim3(256), 0, s, d_mask, K, N, d_tcol0, nt,
                            cw, d_rowflag, d_colflag);
-        hipLaunchKernelGGL(validate_tw_kernel, grid, dim3(256), 0, nullptr, d_mask, K, N, d_tcol0, nt,
+        hipLaunchKernelGGL(validate_tw_kernel, grid, dim3(256), 0, s, d_mask, K, N, d_tcol0, nt,
                            cw, d_rowflag, d_colflag, d_mismatch);
-        hipLaunchKernelGGL(count_flags_kernel, seg_grid, dim3(256), 0, nullptr, d_rowflag, d_colflag,
+        hipLaunchKernelGGL(count_flags_kernel, seg_grid, dim3(256), 0, s, d_rowflag, d_colflag,
                            K, d_tcol0, nt, n_seg_k, n_seg_n, d_seg_counts);
         TW_TRY(hipGetLastError());
     }
     // the mismatch counter and the segment counts come back with one copy (they are adjacent)
     std::vector<char> back(o_tcol0 - o_mismatch);
-    TW_TRY(hipMemcpy(back.data(), ws + o_mismatch, back.size(), hipMemcpyDeviceToHost));
+    TW_TRY(hipMemcpyAsync(back.data(), ws + o_mismatch, back.size(), hipMemcpyDeviceToHost, s));
+    TW_TRY(hipStreamSynchronize(s));
     unsigned long long mismatch = 0;
     std::memcpy(&mismatch, back.data(), sizeof(mismatch));
     const int32_t *seg_counts = reinterpret_cast<const int32_t *>(back.data() + (o_counts - o_mismatch));
     if (mismatch != 0 && !cover) {
-        cleanup();
         return fail(TW_ERR_NOT_TW,
                     "%llu mask elements differ from (row kept) & (column kept) of their tile",
                     mismatch);
     }
 
-    p = new (std::nothrow) tw_plan;
-    if (!p) {
-        cleanup();
+    tw_plan *const p = owner.p = new (std::nothrow) tw_plan;
+    if (!p)
         return fail(TW_ERR_ALLOC, "out of host memory");
-    }
     p->K = K;
     p->N = N;
     p->dtype = dtype;
@@ -998,7 +1022,7 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     p->d_kept_n = reinterpret_cast<int32_t *>(lists + l_kn);
     p->d_rel_k = reinterpret_cast<int32_t *>(lists + l_rk);
     p->d_rel_n = reinterpret_cast<int32_t *>(lists + l_rn);
-    hipLaunchKernelGGL(compact_lists_kernel, seg_grid, dim3(256), 0, nullptr, d_rowflag, d_colflag, K,
+    hipLaunchKernelGGL(compact_lists_kernel, seg_grid, dim3(256), 0, s, d_rowflag, d_colflag, K,
                        d_tcol0, nt, n_seg_k, n_seg_n, d_seg_counts, p->d_kept_k, p->d_rel_k,
                        p->d_kept_n, p->d_rel_n);
     TW_TRY(hipGetLastError());
@@ -1006,27 +1030,25 @@ static int plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int
     p->kept_n_idx.resize(p->kept_n_ptr[nt]);
     {
         std::vector<char> both(l_kn + sizeof(int32_t) * sn);
-        TW_TRY(hipMemcpy(both.data(), lists, both.size(), hipMemcpyDeviceToHost));
+        TW_TRY(hipMemcpyAsync(both.data(), lists, both.size(), hipMemcpyDeviceToHost, s));
+        TW_TRY(hipStreamSynchronize(s));
         if (!p->kept_k_idx.empty())
             std::memcpy(p->kept_k_idx.data(), both.data(), sizeof(int32_t) * p->kept_k_idx.size());
         if (!p->kept_n_idx.empty())
             std::memcpy(p->kept_n_idx.data(), both.data() + l_kn, sizeof(int32_t) * p->kept_n_idx.size());
     }
-    cleanup();
 #undef TW_TRY
     st = validate_lists(K, N, nt, p->tile_col0.data(), p->tile_width.data(), p->kept_k_ptr.data(),
                         p->kept_k_idx.data(), p->kept_n_ptr.data(), p->kept_n_idx.data());
     if (!st)
-        st = finalize_plan_geometry(p);
+        st = finalize_plan_geometry(p, s);
     // rows and columns of a covering tile are the union of its elements: the elements the mask
     // drops inside that cover are stored as zeros
     if (!st && p->packed_elems > 0)
-        st = pack_from_dense(p, d_B, nullptr, cover && mismatch != 0 ? d_mask : nullptr);
-    if (st) {
-        free_plan(p);
+        st = pack_from_dense(p, d_B, s, cover && mismatch != 0 ? d_mask : nullptr);
+    if (st)
         return st;
-    }
-    *out = p;
+    *out = owner.release();
     return TW_OK;
 }
 
@@ -1045,28 +1067,27 @@ static int plan_from_mask_impl(int K, int N, int dtype, int n_tiles, const int32
     if (!mask || !B || !tile_col0 || !tile_width)
         return fail(TW_ERR_NULL, "mask, B or the tile table is NULL");
     const size_t b_bytes = (size_t)K * N * sizeof(float), m_bytes = (size_t)K * N;
-    char *buf = nullptr;
-    if (hipMalloc((void **)&buf, b_bytes + m_bytes) != hipSuccess)
+    DeviceBuffer upload_buf;
+    if (hipMalloc(&upload_buf.ptr, b_bytes + m_bytes) != hipSuccess)
         return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes for the mask and weight upload failed",
                     b_bytes + m_bytes);
+    char *const buf = static_cast<char *>(upload_buf.ptr);
     hipError_t e = hipMemcpy(buf, B, b_bytes, hipMemcpyHostToDevice);
     if (e == hipSuccess)
         e = hipMemcpy(buf + b_bytes, mask, m_bytes, hipMemcpyHostToDevice);
-    int st = e == hipSuccess
-                 ? plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width,
-                                         reinterpret_cast<const uint8_t *>(buf + b_bytes),
-                                         reinterpret_cast<const float *>(buf), cover, out)
-                 : fail(TW_ERR_DEVICE, "mask / weight upload failed: %s", hipGetErrorString(e));
-    hipFree(buf);
-    return st;
+    return e == hipSuccess
+               ? plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width,
+                                       reinterpret_cast<const uint8_t *>(buf + b_bytes),
+                                       reinterpret_cast<const float *>(buf), cover, nullptr, out)
+               : fail(TW_ERR_DEVICE, "mask / weight upload failed: %s", hipGetErrorString(e));
 }
 
 int tw_plan_from_device_mask(int K, int N, int dtype, int n_tiles, const int32_t *tile_col0,
                              const int32_t *tile_width, const uint8_t *mask, const float *B,
-                             int cover, tw_plan **out)
+                             int cover, void *stream, tw_plan **out)
 try {
     return plan_from_device_mask(K, N, dtype, n_tiles, tile_col0, tile_width, mask, B, cover != 0,
-                                 out);
+                                 (hipStream_t)stream, out);
 }
 TW_CATCH_TO_STATUS
 
@@ -1176,7 +1197,8 @@ try {
                         ni.data());
     if (st)
         return st;
-    tw_plan *p = new (std::nothrow) tw_plan;
+    PlanOwner owner;
+    tw_plan *p = owner.p = new (std::nothrow) tw_plan;
     if (!p)
         return fail(TW_ERR_ALLOC, "out of host memory");
     p->K = K;
@@ -1189,11 +1211,10 @@ try {
     p->kept_n_ptr = np;
     p->kept_k_idx = ki;
     p->kept_n_idx = ni;
-    if ((st = finalize_plan_geometry(p)) || (st = pack_from_stream(p, B_stream, off_B, nullptr))) {
-        free_plan(p);
+    if ((st = finalize_plan_geometry(p, nullptr)) ||
+        (st = pack_from_stream(p, B_stream, off_B, nullptr)))
         return st;
-    }
-    *out = p;
+    *out = owner.release();
     return TW_OK;
 }
 TW_CATCH_TO_STATUS
@@ -1250,17 +1271,13 @@ try {
     if (mask_n_rel && sn)
         TW_HIP(hipMemcpy(mask_n_rel, p->d_rel_n, sizeof(int32_t) * sn, hipMemcpyDeviceToHost));
     if (B_stream) {
-        uint16_t *d_Bs = nullptr;
+        DeviceBuffer d_Bs;
         const size_t bytes = (size_t)p->K * p->N * 2;
-        if (hipMalloc((void **)&d_Bs, bytes) != hipSuccess)
+        if (hipMalloc(&d_Bs.ptr, bytes) != hipSuccess)
             return fail(TW_ERR_ALLOC, "hipMalloc of %zu bytes failed", bytes);
-        int st = unpack_to_stream(p, d_Bs, nullptr);
-        hipError_t e = hipSuccess;
-        if (!st)
-            e = hipMemcpy(B_stream, d_Bs, bytes, hipMemcpyDeviceToHost);
-        hipFree(d_Bs);
-        if (st)
+        if (int st = unpack_to_stream(p, static_cast<uint16_t *>(d_Bs.ptr), nullptr))
             return st;
+        const hipError_t e = hipMemcpy(B_stream, d_Bs.ptr, bytes, hipMemcpyDeviceToHost);
         if (e != hipSuccess)
             return fail(TW_ERR_DEVICE, "read-back failed: %s", hipGetErrorString(e));
     }

@@ -654,7 +654,10 @@ int g_ws_device = -1; // the device the buffer lives on; calls on another device
 
 class Arena {
 public:
-    Arena() : lock_(g_ws_mutex)
+    // `s`: the stream the call queues its kernels on; the buffer is not handed to the next call
+    // before that stream has run dry, whichever way the call ends (an error return after kernels
+    // were queued included).
+    explicit Arena(hipStream_t s) : lock_(g_ws_mutex), stream_(s)
     {
         if (hipGetDevice(&device_) != hipSuccess)
             device_ = -2;
@@ -664,6 +667,7 @@ public:
     }
     ~Arena()
     {
+        (void)hipStreamSynchronize(stream_);
         for (void *p : extras_)
             hipFree(p);
         if (usable_ && need_ > g_ws_size) { // grow for the next call
@@ -694,6 +698,7 @@ public:
 
 private:
     std::lock_guard<std::mutex> lock_;
+    hipStream_t stream_;
     int device_ = -1;
     bool usable_ = false;
     size_t off_ = 0, need_ = 0;
@@ -924,7 +929,7 @@ try {
         return fail(TW_ERR_TILE_TABLE, "tiles cover %d columns, N=%d", c, N);
     tcol0[n_tiles] = N;
     hipStream_t s = (hipStream_t)stream;
-    Arena ar;
+    Arena ar(s);
     int32_t *d_tab = ar.alloc_n<int32_t>(n_tiles + 1);
     PruneLayer *d_table = ar.alloc_n<PruneLayer>(1);
     if (!d_tab || !d_table)
@@ -960,7 +965,7 @@ try {
     if (!scores || !norms)
         return fail(TW_ERR_NULL, "a pointer is NULL");
     hipStream_t s = (hipStream_t)stream;
-    Arena ar;
+    Arena ar(s);
     ColLayer *d_cl = ar.alloc_n<ColLayer>(1);
     if (!d_cl)
         return fail(TW_ERR_ALLOC, "hipMalloc of the layer table failed");
@@ -982,7 +987,7 @@ try {
     if (q_type != TW_Q_F32 && q_type != TW_Q_F64)
         return fail(TW_ERR_LAYOUT, "q_type=%d: unknown", q_type);
     Threshold t;
-    Arena ar;
+    Arena ar((hipStream_t)stream);
     int st = percentile_linear(ar, values, n, q, q_type, (hipStream_t)stream, &t);
     if (!st)
         st = read_threshold(t, (hipStream_t)stream, result);
@@ -1006,7 +1011,7 @@ try {
         lt[l].tcol0.push_back(N[l]);
     }
     Threshold thr;
-    Arena ar;
+    Arena ar((hipStream_t)stream);
     st = rows_stage(ar, n_layers, K, N, scores, lt, {}, sparsity, q_type, masks, &thr,
                     (hipStream_t)stream);
     double value = 0.0;
@@ -1034,7 +1039,7 @@ try {
     for (int c = 0; c <= N; c += granularity)
         lt[0].tcol0.push_back(c);
     Threshold thr;
-    Arena ar;
+    Arena ar((hipStream_t)stream);
     st = rows_stage(ar, 1, &K, &N, sc, lt, {}, sparsity, q_type, mk, &thr, (hipStream_t)stream,
                     kNormNotDivided | kPerTileThreshold);
     double value = 0.0;
@@ -1070,7 +1075,7 @@ try {
         coff[l] = total_n;
         total_n += N[l];
     }
-    Arena ar;
+    Arena ar((hipStream_t)stream);
     float *d_cnorm = ar.alloc_n<float>(total_n);
     uint8_t *d_ckeep = ar.alloc_n<uint8_t>(total_n);
     ColLayer *d_cl = ar.alloc_n<ColLayer>(n_layers);
@@ -1150,7 +1155,7 @@ try {
         ml[l].begin = total;
         total += (int64_t)K[l] * N[l];
     }
-    Arena ar;
+    Arena ar(s);
     float *d_pool = ar.alloc_n<float>(total);
     MixLayer *d_layers = ar.alloc_n<MixLayer>(n_layers);
     if (!d_pool || !d_layers)

@@ -145,7 +145,7 @@ def lib():
         "tw_prune_mix": (c_int, [c_int, i32p, i32p, pp, pp, ctypes.c_double, c_int, pp,
                                  ctypes.POINTER(ctypes.c_double), vp]),
         "tw_lstm_gates": (c_int, [c_int, c_int, c_int, vp, c_i64, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
-        "tw_plan_from_device_mask": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, vp, vp, c_int, pp]),
+        "tw_plan_from_device_mask": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, vp, vp, c_int, vp, pp]),
         "tw_set_option": (c_int, [c_int, c_int]),
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
@@ -326,9 +326,9 @@ class Plan:
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod
-    def from_device_mask(cls, K, N, mask_ptr, tile_table, dtype, B_ptr, cover=False):
+    def from_device_mask(cls, K, N, mask_ptr, tile_table, dtype, B_ptr, cover=False, stream=0):
         """As from_mask_tiles, with the mask (K x N bytes) and the fp32 weight in device memory
-        (raw pointers): nothing is uploaded."""
+        (raw pointers): nothing is uploaded.  The build runs on `stream` and waits for it."""
         col0 = _i32([t[0] for t in tile_table])
         width = _i32([t[1] for t in tile_table])
         h = ctypes.c_void_p()
@@ -336,7 +336,7 @@ class Plan:
                                               _ptr(col0, ctypes.c_int32), _ptr(width, ctypes.c_int32),
                                               ctypes.c_void_p(int(mask_ptr or 0)),
                                               ctypes.c_void_p(int(B_ptr or 0)), 1 if cover else 0,
-                                              ctypes.byref(h)))
+                                              ctypes.c_void_p(int(stream or 0)), ctypes.byref(h)))
         return cls(h.value, K, N, dtype_code(dtype))
 
     @classmethod

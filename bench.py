@@ -24,10 +24,16 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 
-# HBM bytes per sparse launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled
-# by what the same counter reads for a 256 MiB copy in the same run (reads x 2.0, writes x 1.0);
-# the runs and their commands are in profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md.
-MEASURED_TRAFFIC_BYTES = {"vgg16_conv4_2": (124334 + 11282) * 1024}
+# HBM bytes per sparse launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+# dispatch), each scaled by what the same counter reads for a 256 MiB copy in the same run
+# (reads x 2.0, writes x 1.0); the runs and their commands are in profiles/tw_gemm_ws_kernel__*.md,
+# one file per workload.  Keyed by the workload's own name.
+MEASURED_TRAFFIC_BYTES = {
+    "vgg16_conv4_2_im2col": (2 * 62061 + 11410) * 1024,
+    "bert_base_ffn_in": (2 * 8076 + 24592) * 1024,
+    "nmt_lstm_gates": (2 * 4427 + 1032) * 1024,
+    "imbalance_stress": (2 * 908806 + 212608) * 1024,
+}
 
 
 def make_workload(name):
@@ -163,7 +169,7 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
         mfma_util_dense_run=fd / t_de / 1e12 / MFMA_PEAK_TFLOPS,
         algorithmic_bytes=by, hbm_gbs=by / t_sparse / 1e9, rotating_buffer_sets=n_sets,
         kept_flops=fk, dense_flops=fd,
-        roofline=roofline_of(M, K, N, tiles, t_sparse))
+        roofline=roofline_of(M, K, N, tiles, t_sparse, MEASURED_TRAFFIC_BYTES.get(wl["name"])))
     del bufs, At, Wt
     torch.cuda.empty_cache()
     return res, (A, B)
@@ -387,7 +393,6 @@ def main():
     wl = make_workload(args.workload)
     res, (A, B) = run_workload(wl, args.steps, args.warmup, torch)
     roof = dict(res["roofline"])
-    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
     out = {
         "metric": "effective TFLOP/s (dense flops / time) at 75% TW sparsity, G=128",
         "value": res["effective_tflops"], "unit": "TFLOP/s", "n_gpus": 1,

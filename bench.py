@@ -108,6 +108,53 @@ def time_plan_graph(plan, bufs, M, steps, warmup, torch):
     return start.elapsed_time(stop) * 1e-3 / steps
 
 
+def time_nmt_recurrence(wl, steps, torch):
+    """One NMT time step is the masked gate GEMM (bias in its epilogue) followed by the LSTM gate
+    arithmetic, which writes h_t into the rows of the next step's A (A_t = [x_t ; h_{t-1}],
+    K-major).  `steps` time steps are recorded into a HIP graph and replayed; returns seconds per
+    step for the pair and for the gate kernel alone."""
+    from tilesparsity_amd import twgemm as tw
+    M, K, N, dtype = wl["M"], wl["K"], wl["N"], wl["dtype"]
+    H = N // 4
+    A, B = wl["values"]()
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    At = [torch.from_numpy(A).cuda().to(tdt).t().contiguous() for _ in range(2)]
+    gates = torch.zeros((N, M), dtype=tdt, device="cuda")
+    cell = torch.zeros((H, M), dtype=torch.float32, device="cuda")
+    bias = torch.zeros((N,), dtype=torch.float32, device="cuda")
+    plan = tw.Plan.create(K, N, dtype, wl["tiles"], B)
+    out = []
+    for with_gemm in (True, False):
+        side = torch.cuda.Stream()
+        graph = torch.cuda.CUDAGraph()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(graph, stream=side):
+                s = torch.cuda.current_stream().cuda_stream
+                for i in range(steps):
+                    a, a_next = At[i % 2], At[(i + 1) % 2]
+                    if with_gemm:
+                        plan.gemm(a.data_ptr(), gates.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
+                                  stream=s, bias_ptr=bias.data_ptr())
+                    tw.lstm_gates(M, H, dtype, gates.data_ptr(), M, 1.0, cell.data_ptr(), M,
+                                  cell.data_ptr(), M, a_next.data_ptr() + (K - H) * M * 2, M, s)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        stream = torch.cuda.current_stream()
+        ts = []
+        for _ in range(6):
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+            graph.replay()
+            stop.record(stream)
+            torch.cuda.synchronize()
+            ts.append(start.elapsed_time(stop) * 1e-3 / steps)
+        out.append(float(np.median(ts[1:])))
+        del graph
+    plan.destroy()
+    return out[0], out[1]
+
+
 def roofline_of(M, K, N, tiles, t, traffic=None):
     """Roofline block of one launch that took t seconds: the binding roof is the larger of the
     ideal HBM time (algorithmic bytes at 8 TB/s) and the ideal MFMA time (kept flops at the dense
@@ -433,6 +480,10 @@ def main():
                                           "us_dense_library", "effective_tflops", "actual_tflops",
                                           "speedup_vs_dense", "speedup_vs_dense_library",
                                           "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "roofline")}
+        if nmt:
+            t_step, t_gates = time_nmt_recurrence(make_workload(name), 50, torch)
+            others[name]["us_step_gemm_and_gates"] = t_step * 1e6
+            others[name]["us_gates_alone"] = t_gates * 1e6
         print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
     if others:
         out["other_workloads"] = others

@@ -108,6 +108,30 @@ def time_plan_graph(plan, bufs, M, steps, warmup, torch):
     return start.elapsed_time(stop) * 1e-3 / steps
 
 
+def time_row_major(wl, steps, warmup, torch):
+    """The operands of the reference's Python operator: x[M,K] and the result [M,N] row-major,
+    pruned columns filled.  Seconds per launch through tw_gemm_staged (K-major copies in a
+    workspace around the K-major kernel) and through the layout-generic kernel."""
+    from tilesparsity_amd import twgemm as tw
+    M, K, N, dtype = wl["M"], wl["K"], wl["N"], wl["dtype"]
+    A, B = wl["values"]()
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    Ar = torch.from_numpy(A).cuda().to(tdt).contiguous()
+    Cr = torch.zeros((M, N), dtype=tdt, device="cuda")
+    plan = tw.Plan.create(K, N, dtype, wl["tiles"], B)
+    nbytes = plan.staged_workspace(M, tw.ROWMAJOR, tw.ROWMAJOR)
+    ws = torch.empty((nbytes,), dtype=torch.uint8, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    kw = dict(lda=K, ldc=N, a_layout=tw.ROWMAJOR, c_layout=tw.ROWMAJOR, pruned_cols=tw.PRUNED_ZERO,
+              stream=s)
+    t_staged = time_steps(lambda i: plan.gemm(Ar.data_ptr(), Cr.data_ptr(), M, workspace_ptr=ws.data_ptr(),
+                                              workspace_bytes=nbytes, **kw), steps, warmup, torch)
+    t_generic = time_steps(lambda i: plan.gemm(Ar.data_ptr(), Cr.data_ptr(), M, **kw),
+                           max(5, steps // 4), 2, torch)
+    plan.destroy()
+    return t_staged, t_generic
+
+
 def time_nmt_recurrence(wl, steps, torch):
     """One NMT time step is the masked gate GEMM (bias in its epilogue) followed by the LSTM gate
     arithmetic, which writes h_t into the rows of the next step's A (A_t = [x_t ; h_{t-1}],
@@ -480,6 +504,10 @@ def main():
                                           "us_dense_library", "effective_tflops", "actual_tflops",
                                           "speedup_vs_dense", "speedup_vs_dense_library",
                                           "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "roofline")}
+        if name == "bert_base_ffn":
+            t_staged, t_generic = time_row_major(make_workload(name), args.steps, args.warmup, torch)
+            others[name]["us_row_major_staged"] = t_staged * 1e6
+            others[name]["us_row_major_generic_kernel"] = t_generic * 1e6
         if nmt:
             t_step, t_gates = time_nmt_recurrence(make_workload(name), 50, torch)
             others[name]["us_step_gemm_and_gates"] = t_step * 1e6

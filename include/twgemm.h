@@ -260,6 +260,23 @@ int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda
                    int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
                    const tw_epilogue *ep, void *stream);
 
+/* tw_gemm_ex for row-major operands at the speed of the K-major kernels.  The reference's Python
+ * operator multiplies a row-major x[M,K] into a row-major result (mask_dense,
+ * Pruning/BERT/utils/modeling.py:992-1007); tw_gemm_ex takes such operands through a
+ * layout-generic kernel that gathers 2-byte elements.  Here a row-major A is first turned into
+ * its K-major copy and a row-major C is produced K-major and turned back, both in `workspace`
+ * (device memory, 16-byte aligned, at least tw_gemm_staged_workspace(plan, M, a_layout, c_layout)
+ * bytes: 2 * round_up(M, 64) * (K for a row-major A + N for a row-major C)); one more pass over
+ * each staged operand at the memory rate.  C's old values go through the workspace as well
+ * whenever the K-major kernel would leave some of them in place (beta != 0, untouched pruned
+ * columns, columns no tile covers).  Same arguments, results and errors as tw_gemm_ex; TW_ERR_BUFFER
+ * for a workspace that is missing or too small.  Allocates nothing; with both layouts K-major it is
+ * tw_gemm_ex.  Calls that share a workspace must not overlap. */
+int64_t tw_gemm_staged_workspace(const tw_plan *plan, int M, int a_layout, int c_layout);
+int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
+                   int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
+                   const tw_epilogue *ep, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Process-wide tuning switches of tw_gemm / tw_gemm_ex; value -1 restores the automatic choice.
  * The launch configuration is otherwise picked from the plan and M.  The reference fixes its one
  * configuration at compile time (Volta884GemmTraits<..., Shape<32,128,128>, ...>,

@@ -124,10 +124,13 @@ def test_gemm_alpha_beta_and_zero_mode(tw, oracle, dtype):
         assert oracle.rel_error(C, full) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("staged", [False, True])
 @pytest.mark.parametrize("a_layout,c_layout", [(1, 1), (1, 0), (0, 1)])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-def test_gemm_row_major_layouts(tw, oracle, a_layout, c_layout, dtype):
-    """Row-major A[M,K] (lda >= K) and/or C[M,N] (ldc >= N) through the layout-generic path."""
+def test_gemm_row_major_layouts(tw, oracle, a_layout, c_layout, dtype, staged):
+    """Row-major A[M,K] (lda >= K) and/or C[M,N] (ldc >= N): through the layout-generic kernel, and
+    staged through K-major copies in a caller's workspace (tw_gemm_staged).  Ragged sizes: M, K
+    and N are no multiples of 8, the leading dimensions leave padding that must stay untouched."""
     import torch
     rng = np.random.default_rng(31 + 2 * a_layout + c_layout)
     M, K, N, G = 203, 150, 330, 128
@@ -156,9 +159,36 @@ def test_gemm_row_major_layouts(tw, oracle, a_layout, c_layout, dtype):
             Ch[:, :M] = Cb.T
         dA, dC = to_device_bits(Ah, Ah.shape), to_device_bits(Ch, Ch.shape)
         with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            kw = {}
+            if staged:
+                nbytes = plan.staged_workspace(M, a_layout, c_layout)
+                assert nbytes == 2 * round_up(M, 64) * (K * (a_layout == tw.ROWMAJOR) +
+                                                        N * (c_layout == tw.ROWMAJOR))
+                ws = torch.full((nbytes // 2 + 64,), 0x7bcd, dtype=torch.int16, device="cuda")
+                kw = dict(workspace_ptr=ws.data_ptr(), workspace_bytes=nbytes)
+                with pytest.raises(tw.TwError) as e:
+                    plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, a_layout=a_layout,
+                              c_layout=c_layout, workspace_ptr=ws.data_ptr(), workspace_bytes=nbytes - 2)
+                assert e.value.status == tw.ERR_BUFFER
             plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
-                      a_layout=a_layout, c_layout=c_layout, pruned_cols=pruned)
+                      a_layout=a_layout, c_layout=c_layout, pruned_cols=pruned, **kw)
             torch.cuda.synchronize()
+            if staged:
+                assert torch.all(ws[nbytes // 2:] == 0x7bcd)   # nothing beyond the stated size
+                # the staged path is the K-major kernel on transposed copies: bit for bit what
+                # that kernel gives on K-major operands
+                Ak = np.zeros((K, round_up(M, 8)), np.uint16)
+                Ak[:, :M] = Ab.T
+                Ck = np.full((N, round_up(M, 8)), SENTINEL, np.uint16)
+                Ck[:, :M] = Cb.T
+                dAk, dCk = to_device_bits(Ak, Ak.shape), to_device_bits(Ck, Ck.shape)
+                plan.gemm(dAk.data_ptr(), dCk.data_ptr(), M, lda=round_up(M, 8), ldc=round_up(M, 8),
+                          alpha=alpha, beta=beta, pruned_cols=pruned)
+                torch.cuda.synchronize()
+                want = from_device_bits(dCk)[:, :M].T
+                have = from_device_bits(dC)
+                have = have[:, :N] if c_layout == tw.ROWMAJOR else have[:, :M].T
+                assert np.array_equal(np.ascontiguousarray(have), np.ascontiguousarray(want))
         out = from_device_bits(dC)
         got = out[:, :N] if c_layout == tw.ROWMAJOR else out[:, :M].T
         pad = out[:, N:] if c_layout == tw.ROWMAJOR else out[:, M:]

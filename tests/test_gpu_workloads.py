@@ -58,6 +58,43 @@ def test_config1_bert_base_ffn(tw, oracle):
     check_workload(tw, oracle, W.bert_base_ffn())
 
 
+def test_config1_row_major_operands_staged(tw, oracle):
+    """Config 1 with the operands of the reference's Python operator: x[M,K] and the result
+    [M,N] row-major, bias in the epilogue, pruned columns receive the bias (mask_dense,
+    Pruning/BERT/utils/modeling.py:992-1007).  Through tw_gemm_staged at full size: sampled rows
+    against the oracle, and the whole result bit for bit against the K-major launch."""
+    import torch
+    from tilesparsity_amd import workloads as W
+    wl = W.bert_base_ffn()
+    M, K, N, dtype, tiles = wl["M"], wl["K"], wl["N"], wl["dtype"], wl["tiles"]
+    A, B = wl["values"]()
+    rng = np.random.default_rng(wl["seed"])
+    bias = rng.standard_normal(N).astype(np.float32)
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    Ar = torch.from_numpy(A).cuda().to(tdt).contiguous()
+    At = Ar.t().contiguous()
+    dbias = torch.from_numpy(bias).cuda()
+    Cr = torch.full((M, N), 0x1234, dtype=torch.int16, device="cuda")
+    Ck = torch.full((N, M), 0x1234, dtype=torch.int16, device="cuda")
+    s = torch.cuda.current_stream().cuda_stream
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        nbytes = plan.staged_workspace(M, tw.ROWMAJOR, tw.ROWMAJOR)
+        ws = torch.empty((nbytes,), dtype=torch.uint8, device="cuda")
+        plan.gemm(Ar.data_ptr(), Cr.data_ptr(), M, lda=K, ldc=N, a_layout=tw.ROWMAJOR,
+                  c_layout=tw.ROWMAJOR, pruned_cols=tw.PRUNED_ZERO, bias_ptr=dbias.data_ptr(),
+                  stream=s, workspace_ptr=ws.data_ptr(), workspace_bytes=nbytes)
+        plan.gemm(At.data_ptr(), Ck.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
+                  bias_ptr=dbias.data_ptr(), stream=s)
+        torch.cuda.synchronize()
+    assert torch.equal(Cr, Ck.t())
+    rows = np.sort(rng.choice(M, size=96, replace=False))
+    got = oracle.bits_to_f32(from_device_bits(Cr[torch.from_numpy(rows).cuda()].contiguous()), dtype)
+    mask = oracle.plan_mask(K, N, tiles)
+    ref = oracle.mask_dense(oracle.quantize(A[rows], dtype), oracle.quantize(B, dtype), mask,
+                            bias.astype(np.float64))
+    assert oracle.rel_error(got.reshape(rows.size, N), ref) <= TOL[dtype]
+
+
 def test_config2_vgg16_conv4_2(tw, oracle):
     from tilesparsity_amd import workloads as W
     check_workload(tw, oracle, W.vgg16_conv4_2())

@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_tile_row_norms", "tw_prune_col_norms", "tw_percentile_linear", "tw_gemm_ex",
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
+    "tw_gemm_staged", "tw_gemm_staged_workspace",
 )
 
 
@@ -124,6 +125,9 @@ def lib():
                                ctypes.POINTER(Epilogue), vp]),
         "tw_gemm_static": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int,
                                    ctypes.POINTER(Epilogue), vp]),
+        "tw_gemm_staged": (c_int, [vp, vp, c_int, c_i64, vp, c_int, c_i64, c_int, c_f, c_f, c_int,
+                                   ctypes.POINTER(Epilogue), vp, c_i64, vp]),
+        "tw_gemm_staged_workspace": (c_i64, [vp, c_int, c_int, c_int]),
         "tw_stream_gemm_nn": (c_int, [c_int, c_int, c_int, c_int, c_f, vp, vp, c_f, vp, c_int,
                                       i32p, i32p, pp, pp, i64p, i64p, vp]),
         "tw_cast_f32": (c_int, [vp, vp, c_i64, c_int, vp]),
@@ -403,17 +407,32 @@ class Plan:
         return tiles, Bs
 
     # -- the GEMM
+    def staged_workspace(self, M, a_layout, c_layout):
+        """Bytes of workspace `gemm(..., workspace_ptr=...)` needs for these layouts."""
+        return int(lib().tw_gemm_staged_workspace(self._h, M, a_layout, c_layout))
+
     def gemm(self, A_ptr, C_ptr, M, lda=None, ldc=None, alpha=1.0, beta=0.0,
              a_layout=KMAJOR, c_layout=KMAJOR, pruned_cols=PRUNED_UNTOUCHED, stream=0,
-             bias_ptr=None, activation=ACT_NONE, static=False):
+             bias_ptr=None, activation=ACT_NONE, static=False, workspace_ptr=None,
+             workspace_bytes=0):
         """C = act(alpha * A (B (.) mask) + beta * C + bias) on device pointers; asynchronous.
         bias_ptr: device fp32 [N] or None; activation: ACT_NONE / ACT_RELU / ACT_GELU / ACT_TANH.
         static=True goes through tw_gemm_static (work-queue counters in the library's own device
-        array; calls that overlap on one GPU race)."""
+        array; calls that overlap on one GPU race).  With a workspace (device memory of
+        staged_workspace(...) bytes) row-major operands go through tw_gemm_staged: K-major copies
+        in the workspace around the K-major kernel, instead of the layout-generic kernel."""
         if lda is None:
             lda = M if a_layout == KMAJOR else self.K
         if ldc is None:
             ldc = M if c_layout == KMAJOR else self.N
+        if workspace_ptr is not None:
+            ep = Epilogue(ctypes.c_void_p(int(bias_ptr or 0)), int(activation))
+            _check(lib().tw_gemm_staged(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
+                                        ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,
+                                        pruned_cols, ctypes.byref(ep),
+                                        ctypes.c_void_p(int(workspace_ptr or 0)), int(workspace_bytes),
+                                        ctypes.c_void_p(int(stream or 0))))
+            return
         if bias_ptr is None and activation == ACT_NONE and not static:
             _check(lib().tw_gemm(self._h, ctypes.c_void_p(int(A_ptr or 0)), a_layout, lda,
                                  ctypes.c_void_p(int(C_ptr or 0)), c_layout, ldc, M, alpha, beta,

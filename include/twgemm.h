@@ -303,7 +303,9 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU */
 #define TW_SHAPE_128x32 5  /* wave-specialised, 128 x 32: skinny M */
 #define TW_SHAPE_256x64 6  /* wave-specialised, 256 x 64 */
-#define TW_N_SHAPES 7
+#define TW_SHAPE_AS64 7    /* A-stationary, 64 rows of all K in LDS: K up to 1136, beta == 0 */
+#define TW_SHAPE_AS32 8    /* A-stationary, 32 rows: K up to 2272, beta == 0 */
+#define TW_N_SHAPES 9
 int tw_set_option(int option, int value);
 
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument

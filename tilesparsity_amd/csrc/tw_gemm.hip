@@ -1216,6 +1216,263 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
 }
 
 // ---------------------------------------------------------------------------------
+// A-stationary kernel for a short K: a workgroup keeps a panel of A - every row k, BMS rows m -
+// in LDS for its whole life and walks over its share of the plan with it.  The streaming kernels
+// above pay a start-up chain (unit -> indices -> rows) and an epilogue per item, and with a
+// short K an item is little else (BERT-base: three steps); here A is read once per workgroup
+// with plain contiguous loads, the gather of a tile's kept rows happens inside LDS (a transposed
+// read takes a row address per lane), the packed weight goes from memory straight into the MFMA
+// operand registers of the one wave that uses it, and the waves never meet again after the
+// panel is loaded: each wave takes blocks of 32 compact columns, multiplies BMS x 32, turns its
+// product through its own piece of LDS and stores it.
+//   panel: row k at k * 2 * BMS bytes; for BMS = 64 the two 64-byte halves of a row are swapped
+//          in rows with bit 1 set, so that the four rows a transposed read touches (consecutive
+//          kept rows are mostly a few rows apart) tend to fall into different bank groups
+//   work:  block b of the plan (unit, 32-column block) belongs to group b % n_groups; workgroup
+//          (row block, group); wave w takes every eighth block of the group
+//   loads: a block is cut into segments of kAsSegSteps steps (16 groups of 16 k rows: per lane
+//          a 16-byte weight fragment and a word with its two row numbers each).  A wave computes one segment out
+//          of one register set while the loads of the next segment - of this block or the next -
+//          fill the other.  Every segment issues the loads of all its 16 groups (steps past the
+//          block's end fetch its last step again), so the number of loads in flight behind a
+//          segment is the same on every path and the wait for it is an exact count.
+// Takes beta == 0 only (C is not read), K-major operands, 32-bit row offsets.
+constexpr int kAsWaves = 8, kAsSegSteps = 4;
+
+template <int DT, int BMS>
+__global__ void __launch_bounds__(64 * kAsWaves, 1)
+    tw_gemm_as_kernel(const GemmArgs p, const int32_t *__restrict__ blocks, int n_blocks, int n_groups,
+                      int n_mblk, int k_rows)
+{
+    constexpr int NT = 64 * kAsWaves;
+    constexpr int ROWB = BMS * 2; // bytes of a panel row
+    constexpr int CH = BMS / 8;   // 16-byte chunks of a panel row
+    constexpr int MI = BMS / 32;
+    constexpr int CP = 32 + 4;    // pitch of a wave's C stage: [32 columns][CP] elements, 32 rows at a time
+    constexpr int DS = kAsSegSteps, GS = DS * 4;
+    using E = Elem<DT>;
+    extern __shared__ __align__(16) unsigned char as_smem[];
+    unsigned char *const panel = as_smem;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int mblk = blockIdx.x % n_mblk, group = blockIdx.x / n_mblk;
+    const int m0 = mblk * BMS;
+    const int m_end = m0 + BMS < p.M ? m0 + BMS : p.M;
+    const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
+    uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
+    const unsigned char *const Bp = reinterpret_cast<const unsigned char *>(p.Bp);
+    uint16_t *const cst = reinterpret_cast<uint16_t *>(as_smem + (size_t)k_rows * ROWB) + wave * 32 * CP;
+
+    // ---- the panel: 16-byte chunks, sixteen loads in flight per thread (the first segment's
+    // loads of this wave are already on their way, see below)
+    auto load_panel = [&]() {
+        const int total = k_rows * CH;
+        const uint32_t lda_b = (uint32_t)p.lda * 2u;
+        const char *const a0 = reinterpret_cast<const char *>(A + m0);
+        constexpr int PL = 16;
+        for (int base = tid; base < total; base += NT * PL) {
+            u32x4 v[PL];
+#pragma unroll
+            for (int q = 0; q < PL; ++q) {
+                const int idx = base + q * NT;
+                const int row = idx / CH, ch = idx % CH;
+                v[q] = u32x4{0u, 0u, 0u, 0u};
+                if (idx < total && m0 + ch * 8 < p.M)
+                    v[q] = *reinterpret_cast<const u32x4 *>(a0 + (uint32_t)row * lda_b + ch * 16);
+            }
+#pragma unroll
+            for (int q = 0; q < PL; ++q) {
+                const int idx = base + q * NT;
+                const int row = idx / CH, ch = idx % CH;
+                const int chs = BMS == 64 ? ch ^ (((row >> 1) & 1) << 2) : ch;
+                if (idx < total)
+                    *reinterpret_cast<u32x4 *>(panel + row * ROWB + chs * 16) = v[q];
+            }
+        }
+    };
+
+    // ---- this wave's blocks, segment by segment
+    const int L = lane & 15;
+    const int pair_e = (lane >> 5) * 4 + (L >> 2);            // this lane's word of a group's row pairs
+    const int lane_b = ((lane >> 4) & 1) * 32 + (L & 3) * 8;  // its byte offset inside a 64-byte half row
+    const int j = lane & 31;                                  // its compact column inside a block
+
+    struct Cursor {    // one segment of one block; wave-uniform
+        int b;         // block index in the plan's list, n_blocks or more: past the end
+        int seg;       // segment of the block
+        int nsteps;    // steps of the block
+        int nb;        // 32-column block inside the unit
+        int code_after; // list entry of the wave's block after this one, fetched a block ahead
+        UnitDev u;
+    };
+    const int b_stride = n_groups * kAsWaves;
+    auto open_block = [&](int b, int code) {
+        Cursor c;
+        c.b = b;
+        c.seg = 0;
+        c.nsteps = 0;
+        c.nb = 0;
+        c.code_after = 0;
+        if (b < n_blocks) {
+            c.code_after = blocks[b + b_stride < n_blocks ? b + b_stride : b];
+            c.u = load_unit(p, code >> 2);
+            c.nb = code & 3;
+            c.nsteps = c.u.k_pad / kBlockK;
+        }
+        return c;
+    };
+    auto valid = [&](const Cursor &c) { return c.b < n_blocks; };
+    auto last_segment = [&](const Cursor &c) { return (c.seg + 1) * DS >= c.nsteps; };
+    auto advance = [&](const Cursor &c) {
+        if (!last_segment(c)) {
+            Cursor n = c;
+            n.seg = c.seg + 1;
+            return n;
+        }
+        return open_block(c.b + b_stride, __builtin_amdgcn_readfirstlane(c.code_after));
+    };
+    struct Seg {
+        u32x4 bq[GS];
+        u32x4 rows[DS]; // per step: the two rows this lane addresses in each of its four groups, 16 bits each
+        int out_n;      // this lane's compact column of the block as a column of the tile
+    };
+    // all loads of a segment (a block without steps has only its column numbers)
+    auto issue = [&](const Cursor &c, Seg &g) {
+        g.out_n = p.kept_n[c.u.kn_off + c.nb * 32 + (j < c.u.n_cnt - c.nb * 32 ? j : 0)];
+        if (c.nsteps == 0)
+            return;
+        const uint32_t *const klist = p.kept_pairs + (c.u.kk_off >> 1) + pair_e * 4;
+        const unsigned char *const bsrc = Bp + c.u.b_off * 2 + (int64_t)(c.u.nb0 + c.nb) * 4096 + lane * 16;
+        const int64_t step_b = (int64_t)c.u.nblk * 4096;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            const int s = c.seg * DS + ds < c.nsteps ? c.seg * DS + ds : c.nsteps - 1;
+            g.rows[ds] = *reinterpret_cast<const u32x4 *>(klist + s * (kBlockK / 2));
+#pragma unroll
+            for (int k16 = 0; k16 < 4; ++k16)
+                g.bq[ds * 4 + k16] = *reinterpret_cast<const u32x4 *>(bsrc + s * step_b + k16 * 1024);
+        }
+    };
+    f32x16 acc[MI];
+    auto clear = [&]() {
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[mi][r] = 0.0f;
+    };
+    float out_bias = 0.0f; // bias of this lane's column of the block being computed
+    int out_col = 0;
+    auto compute = [&](const Cursor &c, const Seg &g) {
+        const int steps = min(DS, c.nsteps - c.seg * DS);
+        if (last_segment(c)) { // the column numbers have landed with the segment: the bias follows
+            out_col = c.u.col0 + g.out_n;
+            out_bias = p.bias ? p.bias[out_col] : 0.0f;
+        }
+        TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))panel + lane_b;
+#pragma unroll
+        for (int ds = 0; ds < DS; ++ds) {
+            if (ds < steps) {
+#pragma unroll
+                for (int k16 = 0; k16 < 4; ++k16) {
+                    const uint32_t r_lo = g.rows[ds][k16] & 0xFFFFu, r_hi = g.rows[ds][k16] >> 16;
+                    // row r at r * ROWB; for BMS = 64 its halves are swapped when bit 1 of r is set
+                    const uint32_t o_lo = r_lo * ROWB + (BMS == 64 ? (r_lo & 2u) << 5 : 0u);
+                    const uint32_t o_hi = r_hi * ROWB + (BMS == 64 ? (r_hi & 2u) << 5 : 0u);
+#pragma unroll
+                    for (int mi = 0; mi < MI; ++mi) {
+                        TW_LDS(unsigned char) qlo = lds_lane + (o_lo ^ (uint32_t)(mi * 64));
+                        TW_LDS(unsigned char) qhi = lds_lane + (o_hi ^ (uint32_t)(mi * 64));
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))qlo);
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))qhi);
+                        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                        acc[mi] = E::mfma(u32x4{l2.x, l2.y, h2.x, h2.y}, g.bq[ds * 4 + k16], acc[mi]);
+                    }
+                }
+            }
+        }
+    };
+    // after a block's last segment: alpha, bias, activation, one rounding; 32 rows at a time
+    // through this wave's stage; 16-byte stores
+    auto finish = [&](const Cursor &c) {
+        if (!last_segment(c))
+            return;
+        const int cnt = min(32, c.u.n_cnt - c.nb * 32);
+#pragma unroll
+        for (int mi = 0; mi < MI; ++mi) {
+            const int mloc = (lane >> 5) * 4;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                uint32_t h[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    h[e] = E::to_bits(tw_activate(p.alpha * acc[mi][r4 * 4 + e] + out_bias, p.act));
+                u32x2 pk;
+                pk.x = h[0] | (h[1] << 16);
+                pk.y = h[2] | (h[3] << 16);
+                *reinterpret_cast<u32x2 *>(cst + j * CP + mloc + r4 * 8) = pk;
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int q = 0; q < 2; ++q) { // 32 columns x 4 chunks of 8 rows
+                const int idx = lane + q * 64;
+                const int jj = idx >> 2, ch = idx & 3;
+                const int col = __shfl(out_col, jj);
+                const u32x2 lo = *reinterpret_cast<const u32x2 *>(cst + jj * CP + ch * 8);
+                const u32x2 hi = *reinterpret_cast<const u32x2 *>(cst + jj * CP + ch * 8 + 4);
+                const int m = m0 + mi * 32 + ch * 8;
+                if (jj < cnt)
+                    store_chunk(C + (int64_t)col * p.ldc + m, u32x4{lo.x, lo.y, hi.x, hi.y}, m, m_end,
+                                p.store_through != 0);
+            }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the stage is free again
+        }
+        clear();
+    };
+
+    clear();
+    Seg g0, g1;
+    const int b_first = group + n_groups * wave;
+    Cursor cur = open_block(b_first, b_first < n_blocks ? __builtin_amdgcn_readfirstlane(blocks[b_first]) : 0);
+    if (valid(cur))
+        issue(cur, g0); // weight and row numbers do not wait for the panel
+    load_panel();
+    __syncthreads();
+    if (valid(cur)) {
+        for (;;) {
+            Cursor nxt = advance(cur);
+            if (valid(nxt))
+                issue(nxt, g1);
+            compute(cur, g0);
+            finish(cur);
+            if (!valid(nxt))
+                break;
+            cur = advance(nxt);
+            if (valid(cur))
+                issue(cur, g0);
+            compute(nxt, g1);
+            finish(nxt);
+            if (!valid(cur))
+                break;
+        }
+    }
+
+    // ---- TW_PRUNED_ZERO: the pruned columns of this group's tiles receive act(bias)
+    for (int z = p.n_gemm_u + group; z < p.n_all_u; z += n_groups) {
+        const TileDev t = p.tiles[z - p.n_gemm_u];
+        for (int i = tid; i < t.n_pruned * CH; i += NT) {
+            const int jz = i / CH, ch = i % CH;
+            const int c = t.col0 + p.pruned_n[t.pn_off + jz];
+            const uint32_t hb = E::to_bits(tw_finish(0.0f, p.bias, c, p.act));
+            const uint32_t w = hb | (hb << 16);
+            store_chunk(C + (int64_t)c * p.ldc + m0 + ch * 8, u32x4{w, w, w, w}, m0 + ch * 8, m_end,
+                        p.store_through != 0);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
 // Layout-generic kernel: any combination of K-major / row-major A and C through element
 // strides.  One workgroup (4 waves, 128 x 128 tile, 32-row steps) per work item in queue
 // order, single-buffered.  Gathered A elements are fetched one by one with the lanes running
@@ -1388,7 +1645,14 @@ static const Shape kShapes[TW_N_SHAPES] = {
     {256, 128, 1}, // TW_SHAPE_256x128
     {128, 32, 2},  // TW_SHAPE_128x32
     {256, 64, 1},  // TW_SHAPE_256x64
+    {64, 128, 1},  // TW_SHAPE_AS64
+    {32, 128, 1},  // TW_SHAPE_AS32
 };
+
+// LDS of the A-stationary kernel: the panel (all K rows, BMS rows m) and a C stage per wave
+constexpr int kLdsBytes = 160 * 1024;
+static int64_t as_lds_bytes(int K, int bms) { return (int64_t)K * bms * 2 + kAsWaves * 32 * 36 * 2; }
+static bool is_as_shape(int shape) { return shape == TW_SHAPE_AS64 || shape == TW_SHAPE_AS32; }
 
 // Steps of loads a moving wave keeps in flight, per shape (bounded by its 256 registers: a step
 // takes 4 * (A loads + weight loads per thread) of them).  Measured on the benchmark shapes: two
@@ -1496,7 +1760,7 @@ struct Choice {
 // workgroups of a die then share the rows of A in their L2 (measured on the 0 %-sparse plan of
 // the headline shape: a third of the reads from memory), but no benchmark shape ran faster for
 // it and the stress shape, whose 512-row block of A fills an L2, ran 13 % slower.
-static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
+static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c)
 {
     Choice c;
     const int width = std::max(32, round_up32(plan->max_unit_n)); // 32, 64, 96 or 128
@@ -1508,6 +1772,14 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
     };
     c.xcd = option(TW_OPT_XCD_QUEUES) == 1;
     c.piece = 128;
+    // The A-stationary kernel (K short enough for a panel of A in LDS, C not read) is never the
+    // automatic choice: measured against the streaming shapes it gains 3 % on BERT-base (17.7
+    // against 18.3 us) and loses on the NMT gates (9.5 against 9.2) and on BERT-large FFN1
+    // (43 - 62 against 38 - 55 us at 50 - 90 % sparsity).
+    auto as_ok = [&](int shape) {
+        return ws_ok && !reads_c && plan->n_blocks > 0 && plan->d_kept_pairs &&
+               as_lds_bytes(plan->K, kShapes[shape].bm) <= kLdsBytes;
+    };
     if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
     } else if (width > 64) {
@@ -1537,7 +1809,10 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
     }
     // forced choices, where they fit the plan: a shape takes pieces up to its width
     const int f_piece = option(TW_OPT_PIECE), f_shape = option(TW_OPT_SHAPE);
-    if (f_shape >= 0 && (f_shape != TW_SHAPE_WIDE ? ws_ok : true)) {
+    if (f_shape >= 0 && is_as_shape(f_shape)) {
+        if (as_ok(f_shape))
+            c.shape = f_shape;
+    } else if (f_shape >= 0 && (f_shape != TW_SHAPE_WIDE ? ws_ok : true)) {
         const int piece = f_piece > 0 ? f_piece : std::min(128, kShapes[f_shape].bn);
         if (std::min(piece, width) <= kShapes[f_shape].bn) {
             c.shape = f_shape;
@@ -1546,10 +1821,36 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda)
     } else if (f_piece > 0 && std::min(f_piece, width) <= kShapes[c.shape].bn) {
         c.piece = f_piece;
     }
-    if (c.shape == TW_SHAPE_WIDE)
+    if (c.shape == TW_SHAPE_WIDE || is_as_shape(c.shape))
         c.piece = 128;
     c.per_cu = option(TW_OPT_WGS_PER_CU) > 0 ? option(TW_OPT_WGS_PER_CU) : kShapes[c.shape].wgs_per_cu;
     return c;
+}
+
+// the A-stationary kernel: one workgroup per (row block, group of blocks); no work queue
+template <int DT, int BMS> static int launch_as(const tw_plan *plan, const GemmArgs &a, int M, hipStream_t s)
+{
+    static std::once_flag once;
+    static hipError_t attr_err = hipSuccess;
+    std::call_once(once, [] {
+        attr_err = hipFuncSetAttribute((const void *)tw_gemm_as_kernel<DT, BMS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
+    });
+    if (attr_err != hipSuccess)
+        return fail(TW_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(attr_err));
+    const int n_mblk = (M + BMS - 1) / BMS;
+    // as many groups as keep every compute unit at one workgroup, each wave with a block or more
+    const int per_wg = kAsWaves;
+    int n_groups = std::max(1, plan->cu_count / n_mblk);
+    n_groups = std::min(n_groups, std::max(1, (plan->n_blocks + per_wg - 1) / per_wg));
+    if ((int64_t)n_mblk * n_groups > (int64_t)0x7fffffff)
+        return fail(TW_ERR_SHAPE, "%lld workgroups (M=%d): a launch takes at most %lld",
+                    (long long)n_mblk * n_groups, M, (long long)(int64_t)0x7fffffff);
+    hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS>), dim3((unsigned)(n_mblk * n_groups)),
+                       dim3(64 * kAsWaves), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
+                       n_mblk, plan->K);
+    TW_HIP(hipGetLastError());
+    return TW_OK;
 }
 
 } // namespace tw
@@ -1631,6 +1932,7 @@ void fill_common(GemmArgs &a, const tw_plan *plan, const void *A, int64_t lda, v
     a.units = plan->d_units;
     a.tiles = plan->d_tiles;
     a.kept_k = plan->d_kept_k_pad;
+    a.kept_pairs = plan->d_kept_pairs;
     a.kept_n = plan->d_kept_n;
     a.pruned_n = plan->d_pruned_n;
     a.Bp = plan->d_Bp;
@@ -1676,6 +1978,13 @@ int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *tick
     a.n_arg_units = plan->n_units <= kMaxArgUnits ? plan->n_units : 0;
     for (int i = 0; i < a.n_arg_units; ++i)
         a.arg_units[i] = plan->h_units[i];
+    if (is_as_shape(c.shape)) {
+        if (plan->dtype == TW_F16)
+            return c.shape == TW_SHAPE_AS64 ? launch_as<TW_F16, 64>(plan, a, a.M, s)
+                                            : launch_as<TW_F16, 32>(plan, a, a.M, s);
+        return c.shape == TW_SHAPE_AS64 ? launch_as<TW_BF16, 64>(plan, a, a.M, s)
+                                        : launch_as<TW_BF16, 32>(plan, a, a.M, s);
+    }
     // queue 0 is the longest: one workgroup per entry, up to the chip's share of a queue
     const int64_t qlen0 = (int64_t)a.n_own_items + (a.n_tail_items + kXcd - 1) / kXcd;
     const int64_t per_queue = std::max<int64_t>(1, (int64_t)plan->cu_count * c.per_cu / kXcd);
@@ -1750,7 +2059,7 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
         return TW_OK;
     }
 
-    const Choice c = choose_shape(plan, M, lda);
+    const Choice c = choose_shape(plan, M, lda, beta != 0.0f);
     fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
     if ((int64_t)a.n_all_u * a.n_mblk > kMaxItems)
         return fail(TW_ERR_SHAPE, "%lld work items (M=%d): a launch takes at most %lld",

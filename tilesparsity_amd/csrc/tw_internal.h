@@ -62,6 +62,12 @@ struct GemmArgs {
     const UnitDev *units;   // sorted by k_kept descending
     const TileDev *tiles;
     const int32_t *kept_k;
+    // The kept-K lists once more for the A-stationary kernel: one word per lane and group of 16
+    // k rows, the two rows a lane addresses in the group as 16-bit halves.  Entry
+    // kk_off / 2 + step * 32 + e * 4 + group holds rows (e / 4) * 8 + e % 4 and that + 4 of the
+    // group, so that the four words of a step a lane needs are one 16-byte load (null when K
+    // does not fit 16 bits).
+    const uint32_t *kept_pairs;
     const int32_t *kept_n;
     const int32_t *pruned_n;
     const void *Bp;
@@ -111,6 +117,11 @@ struct tw_plan {
     tw::TileDev *d_tiles = nullptr;
     void *d_Bp = nullptr;
     int32_t *d_tickets = nullptr; // kTicketSlots slots of kTicketInts counters
+    // every (unit, 32-column block) pair of the plan, in unit order: unit * 4 + block (the work
+    // list of the A-stationary kernel)
+    int32_t *d_blocks = nullptr;
+    int n_blocks = 0;
+    uint32_t *d_kept_pairs = nullptr; // GemmArgs::kept_pairs
     // Ownership: every pointer above points into one of these two allocations.  d_lists holds the
     // four index arrays when the pre-pass compacted them on the device (else they sit in d_slab);
     // d_slab holds the unit / tile tables, the pruned-column and padded kept-K lists, the packing

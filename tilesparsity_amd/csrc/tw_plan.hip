@@ -660,6 +660,24 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
     const size_t o_pruned = put(pruned_n.data(), pruned_n.size() * sizeof(int32_t));
     const size_t o_kkpad = put(kept_k_pad.data(), kept_k_pad.size() * sizeof(int32_t));
     const size_t o_ptab = put(ptab.data(), ptab.size() * sizeof(PackTile));
+    std::vector<int32_t> blocks;
+    for (size_t ui = 0; ui < units.size(); ++ui)
+        for (int nb = 0; nb < units[ui].nb_cnt; ++nb)
+            blocks.push_back((int32_t)ui * 4 + nb);
+    p->n_blocks = (int)blocks.size();
+    const size_t o_blocks = put(blocks.data(), blocks.size() * sizeof(int32_t));
+    std::vector<uint32_t> kpairs; // see GemmArgs::kept_pairs
+    if (p->K <= 0xFFFF) {
+        kpairs.resize(kept_k_pad.size() / 2);
+        for (size_t st = 0; st < kept_k_pad.size() / 64; ++st)
+            for (int g16 = 0; g16 < 4; ++g16)
+                for (int e = 0; e < 8; ++e) {
+                    const size_t lo = st * 64 + g16 * 16 + (e >> 2) * 8 + (e & 3);
+                    kpairs[st * 32 + e * 4 + g16] =
+                        (uint32_t)kept_k_pad[lo] | ((uint32_t)kept_k_pad[lo + 4] << 16);
+                }
+    }
+    const size_t o_kpairs = put(kpairs.data(), kpairs.size() * sizeof(uint32_t));
     size_t o_kk = 0, o_kn = 0, o_rk = 0, o_rn = 0;
     if (lists_here) {
         o_kk = put(p->kept_k_idx.data(), p->kept_k_idx.size() * sizeof(int32_t));
@@ -686,6 +704,8 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
     p->d_pruned_n = reinterpret_cast<int32_t *>(slab + o_pruned);
     p->d_kept_k_pad = reinterpret_cast<int32_t *>(slab + o_kkpad);
     p->d_pack_tiles = slab + o_ptab;
+    p->d_blocks = reinterpret_cast<int32_t *>(slab + o_blocks);
+    p->d_kept_pairs = kpairs.empty() ? nullptr : reinterpret_cast<uint32_t *>(slab + o_kpairs);
     if (lists_here) {
         p->d_kept_k = reinterpret_cast<int32_t *>(slab + o_kk);
         p->d_kept_n = reinterpret_cast<int32_t *>(slab + o_kn);

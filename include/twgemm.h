@@ -288,7 +288,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  *   TW_OPT_PIECE        columns of a tile handed out as one work item: 128, 64 or 32
  *   TW_OPT_XCD_QUEUES   1: one work queue per accelerator die, each owning whole row blocks of A
  *                       (the workgroups of a die then share those rows in their L2);
- *                       0 (default): the work items are dealt out over the dies in turn
+ *                       0: the work items are dealt out over the dies in turn; automatic: 0
+ *                       unless nearly every tile keeps nearly every row (a 0 %-sparse plan)
  * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
  * TWGEMM_PIECE and TWGEMM_XCD_QUEUES, read once. */
 #define TW_OPT_SHAPE 0

@@ -1770,7 +1770,9 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     auto items = [&](int bm, int piece) {
         return units * ((width + piece - 1) / piece) * ((M + bm - 1) / bm);
     };
-    c.xcd = option(TW_OPT_XCD_QUEUES) == 1;
+    // one queue per die where the tiles share their rows (a 0 %-sparse plan reads A once per die
+    // then instead of once per tile); no sparse plan gained from it, see below
+    c.xcd = option(TW_OPT_XCD_QUEUES) == 1 || (option(TW_OPT_XCD_QUEUES) == -1 && plan->rows_shared);
     c.piece = 128;
     // The A-stationary kernel (K short enough for a panel of A in LDS, C not read) is never the
     // automatic choice: measured against the streaming shapes it gains 3 % on BERT-base (17.7

@@ -629,6 +629,9 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
         steps += u.k_pad / kBlockK;
     }
     p->mean_steps = p->n_pipe_units ? (int)(steps / p->n_pipe_units) : 0;
+    // (kept rows summed over the tiles that have any, against all rows for each of them)
+    p->rows_shared = nt > 1 && p->n_pipe_units > 0 &&
+                     (int64_t)p->kept_k_idx.size() * 10 >= (int64_t)p->K * nt * 9;
     p->n_zero_tiles = (int)ztiles.size();
 
     // One device allocation for everything the plan owns besides lists that were compacted on

@@ -1754,8 +1754,7 @@ struct Choice {
 };
 
 // Picks the shape from the plan and M.  Wide tiles run 256-row items (half the weight traffic
-// per row of A), or 128-row items with two workgroups per CU when 256-row items would leave a
-// quarter of the chip without work.  Launches with too few items for the chip (skinny M) hand a
+// per row of A of 128-row items).  Launches with too few items for the chip (skinny M) hand a
 // unit out in pieces of 64 or 32 columns.  One queue per die is an option, not the default: the
 // workgroups of a die then share the rows of A in their L2 (measured on the 0 %-sparse plan of
 // the headline shape: a third of the reads from memory), but no benchmark shape ran faster for
@@ -1774,23 +1773,35 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     // then instead of once per tile); no sparse plan gained from it, see below
     c.xcd = option(TW_OPT_XCD_QUEUES) == 1 || (option(TW_OPT_XCD_QUEUES) == -1 && plan->rows_shared);
     c.piece = 128;
-    // The A-stationary kernel (K short enough for a panel of A in LDS, C not read) is never the
-    // automatic choice: measured against the streaming shapes it gains 3 % on BERT-base (17.7
-    // against 18.3 us) and loses on the NMT gates (9.5 against 9.2) and on BERT-large FFN1
-    // (43 - 62 against 38 - 55 us at 50 - 90 % sparsity).
+    // The A-stationary kernel (K short enough for a panel of A in LDS, C not read).  Measured on a
+    // grid of M 128 .. 16384, K 512 .. 2048, N 512 .. 4096, tiles of 64 and 128 columns, 25 and
+    // 50 % of the rows kept, against every streaming shape: it wins by 5 - 50 % for tiles of 64
+    // columns at any size, and for tiles of 128 where the streaming kernel would run at most one
+    // 256-row item on every other compute unit (its start-up and epilogue are most of such a
+    // launch); 32-row panels below about a thousand rows of A, 64-row panels above.  Elsewhere
+    // (BERT-base, BERT-large FFN1: several items per unit) it ties or loses up to 10 %.
     auto as_ok = [&](int shape) {
         return ws_ok && !reads_c && plan->n_blocks > 0 && plan->d_kept_pairs &&
                as_lds_bytes(plan->K, kShapes[shape].bm) <= kLdsBytes;
     };
+    const bool as_few = width <= 64 || items(256, 128) * 2 <= cu;
     if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
+    } else if (as_ok(TW_SHAPE_AS64) && as_few && (M > 128 || plan->n_blocks >= 96)) {
+        // 64-row panels where they still give three quarters of the compute units a workgroup
+        const int mblk64 = (M + 63) / 64;
+        const int groups64 = std::min(std::max(1, cu / mblk64), (plan->n_blocks + kAsWaves - 1) / kAsWaves);
+        c.shape = (int64_t)mblk64 * groups64 * 4 >= (int64_t)cu * 3 ? TW_SHAPE_AS64 : TW_SHAPE_AS32;
+    } else if (!as_ok(TW_SHAPE_AS64) && as_ok(TW_SHAPE_AS32) && M > 128 && M <= 512) {
+        c.shape = TW_SHAPE_AS32;
     } else if (width > 64) {
         if (items(128, 128) * 2 < cu) { // skinny: split the units until half the chip has work
             c.piece = items(128, 64) * 2 >= cu ? 64 : 32;
             c.shape = c.piece == 64 ? TW_SHAPE_128x64 : TW_SHAPE_128x32;
-        } else if (items(256, 128) * 4 < 3 * cu) {
-            c.shape = TW_SHAPE_128x128;
         } else {
+            // (128 x 128 on two workgroups per CU fills more of the chip when 256-row items are
+            // few, and is slower all the same: 17.8 against 12.4 us and 36.6 against 26.9 us on the
+            // reference driver's first two shapes, 150 items each)
             c.shape = TW_SHAPE_256x128;
         }
     } else if (width > 32) {

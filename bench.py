@@ -415,6 +415,59 @@ def bench_producers(steps, warmup, torch):
     }
 
 
+def bench_shape_grid(torch, Ms=(128, 512, 2048, 8192, 16384), Ks=(512, 1024, 2048, 4096),
+                     Ns=(512, 2048, 4096), Gs=(64, 128), keeps=(0.25, 0.5)):
+    """The automatic shape choice against every kernel shape forced in turn, on a grid of
+    problems (random tiles, kept-K within +-30 % of keep * K, 90 % of the columns kept).  One line
+    per problem: the automatic choice's time, the best forced shape and its time, and their
+    ratio; a summary line at the end.  A forced shape that cannot take a plan falls back to the
+    automatic one, so its time then repeats that."""
+    import itertools
+    from tilesparsity_amd import twgemm as tw
+    rng = np.random.default_rng(7)
+    s = torch.cuda.current_stream().cuda_stream
+    shapes = [(tw.SHAPE_128x128, -1), (tw.SHAPE_512x64, -1), (tw.SHAPE_128x64, 64), (tw.SHAPE_256x128, -1),
+              (tw.SHAPE_128x32, 32), (tw.SHAPE_256x64, -1), (tw.SHAPE_AS64, -1), (tw.SHAPE_AS32, -1)]
+    worst, n_all, n_off = 1.0, 0, 0
+    for M, K, N, G, keep in itertools.product(Ms, Ks, Ns, Gs, keeps):
+        tiles = []
+        for c0 in range(0, N, G):
+            w = min(G, N - c0)
+            kt = int(np.clip(round(K * keep * rng.uniform(0.7, 1.3)), 1, K))
+            tiles.append(dict(col0=c0, width=w,
+                              kept_k=np.sort(rng.choice(K, kt, replace=False)).astype(np.int32),
+                              kept_n=np.sort(rng.choice(w, max(1, round(w * 0.9)), replace=False)).astype(np.int32)))
+        B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+        plan = tw.Plan.create(K, N, "f16", tiles, B)
+        n_sets = max(2, min(6, (256 << 20) // ((K + N) * M * 2)))
+        bufs = [(torch.randn((K, M), device="cuda").half(),
+                 torch.zeros((N, M), dtype=torch.float16, device="cuda")) for _ in range(n_sets)]
+        steps = 30 if M * K * N < 1 << 34 else 10
+        time_plan(plan, bufs, M, 60, 0, torch)        # the first launches of a new plan run slower
+        t_auto = min(time_plan(plan, bufs, M, steps, 3, torch) for _ in range(2))
+        res = []
+        for shape, piece in shapes:
+            if shape in ((tw.SHAPE_128x128, tw.SHAPE_256x128) if G == 64 else (tw.SHAPE_512x64, tw.SHAPE_256x64)):
+                continue    # 128-column shapes on 64-column tiles and the other way round
+            tw.set_option(tw.OPT_SHAPE, shape)
+            tw.set_option(tw.OPT_PIECE, piece)
+            res.append((min(time_plan(plan, bufs, M, steps, 3, torch) for _ in range(2)), shape))
+        tw.set_option(tw.OPT_SHAPE, -1)
+        tw.set_option(tw.OPT_PIECE, -1)
+        t_auto = min(t_auto, min(time_plan(plan, bufs, M, steps, 3, torch) for _ in range(2)))
+        t_best, s_best = min(res)
+        n_all += 1
+        n_off += t_auto > 1.08 * t_best
+        worst = max(worst, t_auto / t_best)
+        print("M=%d K=%d N=%d G=%d keep=%.2f: automatic %.1f us, best forced shape %d %.1f us, ratio %.2f" % (
+            M, K, N, G, keep, t_auto * 1e6, s_best, t_best * 1e6, t_auto / t_best), flush=True)
+        plan.destroy()
+        del bufs
+        torch.cuda.empty_cache()
+    print(json.dumps({"problems": n_all, "automatic_more_than_8_percent_off_the_best": n_off,
+                      "worst_ratio": worst}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -427,6 +480,9 @@ def main():
                     help="benchmark the TW mask producers instead of the GEMM (one JSON line)")
     ap.add_argument("--prepass", action="store_true",
                     help="time the mask -> kept lists -> offsets -> compaction pre-pass instead")
+    ap.add_argument("--shape-grid", action="store_true",
+                    help="time the automatic kernel-shape choice against every forced shape on a "
+                         "grid of problems (several minutes)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (4 launches over rotating buffers), "
                          "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
@@ -442,6 +498,9 @@ def main():
         return 1
     from tilesparsity_amd import twgemm as tw
     tw.lib()  # fails loudly if the HIP library has not been built
+    if args.shape_grid:
+        bench_shape_grid(torch)
+        return 0
     if args.producers:
         print(json.dumps(bench_producers(min(args.steps, 20), min(args.warmup, 3), torch)), flush=True)
         return 0

@@ -281,7 +281,7 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  * The launch configuration is otherwise picked from the plan and M.  The reference fixes its one
  * configuration at compile time (Volta884GemmTraits<..., Shape<32,128,128>, ...>,
  * basic_nn.cu:250-259, and MAX_BLOCK_NUM streams, :73); tests and tuning runs use these switches
- * to cover every kernel shape.  A forced shape or piece width that cannot take the plan (a shape
+ * to cover every kernel shape (bench.py --shape-grid times the automatic choice against each).  A forced shape or piece width that cannot take the plan (a shape
  * narrower than the plan's unit pieces, TW_SHAPE_WIDE aside operands beyond 4 GiB) is ignored.
  *   TW_OPT_SHAPE        one of the TW_SHAPE_* kernels below
  *   TW_OPT_WGS_PER_CU   workgroups launched per compute unit, 1..8

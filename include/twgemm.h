@@ -262,8 +262,9 @@ int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 
 /* tw_gemm_ex for row-major operands at the speed of the K-major kernels.  The reference's Python
  * operator multiplies a row-major x[M,K] into a row-major result (mask_dense,
- * Pruning/BERT/utils/modeling.py:992-1007); tw_gemm_ex takes such operands through a
- * layout-generic kernel that gathers 2-byte elements.  Here a row-major A is first turned into
+ * Pruning/BERT/utils/modeling.py:992-1007).  tw_gemm_ex takes such operands as they are when both
+ * are row-major, K <= 2272 and beta == 0 (a kernel that keeps a panel of A in LDS), and else
+ * through a layout-generic kernel that gathers 2-byte elements.  Here, in those other cases, a row-major A is first turned into
  * its K-major copy and a row-major C is produced K-major and turned back, both in `workspace`
  * (device memory, 16-byte aligned, at least tw_gemm_staged_workspace(plan, M, a_layout, c_layout)
  * bytes: 2 * round_up(M, 64) * (K for a row-major A + N for a row-major C)); one more pass over

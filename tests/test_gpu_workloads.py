@@ -58,11 +58,13 @@ def test_config1_bert_base_ffn(tw, oracle):
     check_workload(tw, oracle, W.bert_base_ffn())
 
 
-def test_config1_row_major_operands_staged(tw, oracle):
+def test_config1_row_major_operands(tw, oracle):
     """Config 1 with the operands of the reference's Python operator: x[M,K] and the result
     [M,N] row-major, bias in the epilogue, pruned columns receive the bias (mask_dense,
-    Pruning/BERT/utils/modeling.py:992-1007).  Through tw_gemm_staged at full size: sampled rows
-    against the oracle, and the whole result bit for bit against the K-major launch."""
+    Pruning/BERT/utils/modeling.py:992-1007).  At full size, through tw_gemm_staged (which hands
+    operands a GEMM kernel takes as they are straight on: K = 768 fits the A-stationary kernel's
+    panel) and with A alone row-major (staged): sampled rows against the oracle, and the whole
+    result bit for bit against the K-major launch."""
     import torch
     from tilesparsity_amd import workloads as W
     wl = W.bert_base_ffn()
@@ -86,7 +88,12 @@ def test_config1_row_major_operands_staged(tw, oracle):
         plan.gemm(At.data_ptr(), Ck.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
                   bias_ptr=dbias.data_ptr(), stream=s)
         torch.cuda.synchronize()
+        Ck2 = torch.full((N, M), 0x1234, dtype=torch.int16, device="cuda")
+        plan.gemm(Ar.data_ptr(), Ck2.data_ptr(), M, lda=K, a_layout=tw.ROWMAJOR, pruned_cols=tw.PRUNED_ZERO,
+                  bias_ptr=dbias.data_ptr(), stream=s, workspace_ptr=ws.data_ptr(), workspace_bytes=nbytes)
+        torch.cuda.synchronize()
     assert torch.equal(Cr, Ck.t())
+    assert torch.equal(Ck2, Ck)
     rows = np.sort(rng.choice(M, size=96, replace=False))
     got = oracle.bits_to_f32(from_device_bits(Cr[torch.from_numpy(rows).cuda()].contiguous()), dtype)
     mask = oracle.plan_mask(K, N, tiles)

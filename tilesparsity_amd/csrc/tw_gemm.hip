@@ -118,6 +118,15 @@ __device__ __forceinline__ float tw_activate(float v, int act)
         return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * v) + 1.0f);
     return v;
 }
+// The value of an output element is rounded to fp32 before it is rounded to 16 bits, in every
+// kernel: left to itself the compiler turns "multiply, add, convert" into one fused instruction
+// with a single rounding in some epilogues and not in others, and the kernels then differ in the
+// last bit of about one element in twenty thousand.
+__device__ __forceinline__ float tw_fp32_value(float v)
+{
+    asm volatile("" : "+v"(v));
+    return v;
+}
 // alpha*acc + beta*C is already in `v`: adds the bias of column c and applies the activation
 __device__ __forceinline__ float tw_finish(float v, const float *bias, int c, int act)
 {
@@ -1146,7 +1155,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                                     float v[4];
 #pragma unroll
                                     for (int e = 0; e < 4; ++e)
-                                        v[e] = tw_activate(scale * acc[mi][ni][r4 * 4 + e] + bj, ACT);
+                                        v[e] = tw_fp32_value(tw_activate(scale * acc[mi][ni][r4 * 4 + e] + bj, ACT));
                                     u32x2 pk;
                                     pk.x = E::to_bits(v[0]) | (E::to_bits(v[1]) << 16);
                                     pk.y = E::to_bits(v[2]) | (E::to_bits(v[3]) << 16);
@@ -1236,10 +1245,15 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
 //          fill the other.  Every segment issues the loads of all its 16 groups (steps past the
 //          block's end fetch its last step again), so the number of loads in flight behind a
 //          segment is the same on every path and the wait for it is an exact count.
-// Takes beta == 0 only (C is not read), K-major operands, 32-bit row offsets.
+// Takes beta == 0 only (C is not read).  RM false: K-major A and C (32-bit row offsets into A).
+// RM true: row-major A[M][lda] and C[M][ldc], the operands of the reference's Python operator
+// (mask_dense, Pruning/BERT/utils/modeling.py:992-1007): the panel is transposed on its way into
+// LDS (a lane reads 16 bytes along k of its own row m and writes them as eight 2-byte pieces
+// into eight panel rows; consecutive lanes are consecutive m, so those writes are contiguous),
+// and the product goes out as 2-byte stores, a wave covering two rows of the block's 32 columns.
 constexpr int kAsWaves = 8, kAsSegSteps = 4;
 
-template <int DT, int BMS>
+template <int DT, int BMS, bool RM>
 __global__ void __launch_bounds__(64 * kAsWaves, 1)
     tw_gemm_as_kernel(const GemmArgs p, const int32_t *__restrict__ blocks, int n_blocks, int n_groups,
                       int n_mblk, int k_rows)
@@ -1266,6 +1280,41 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
 
     // ---- the panel: 16-byte chunks, sixteen loads in flight per thread (the first segment's
     // loads of this wave are already on their way, see below)
+    auto load_panel_row_major = [&]() {
+        // lane -> row m (BMS = 32: the upper half of the wave takes the next chunk of k)
+        constexpr int LPM = 64 / BMS;                       // k chunks a wave reads per load
+        const int m = lane % BMS;
+        const int kchunks = (k_rows + 7) / 8;
+        const bool m_ok = m0 + m < p.M;
+        const uint16_t *const arow = A + (int64_t)(m0 + m) * p.lda;
+        unsigned char *const dst = panel + (m & 31) * 2;
+        constexpr int PL = 4;
+        for (int base = wave * LPM + lane / BMS; base < kchunks; base += kAsWaves * LPM * PL) {
+            u32x4 v[PL];
+#pragma unroll
+            for (int q = 0; q < PL; ++q) {
+                const int kc = base + q * kAsWaves * LPM;
+                v[q] = u32x4{0u, 0u, 0u, 0u};
+                if (kc < kchunks && m_ok)
+                    v[q] = *reinterpret_cast<const u32x4 *>(arow + kc * 8);
+            }
+#pragma unroll
+            for (int q = 0; q < PL; ++q) {
+                const int kc = base + q * kAsWaves * LPM;
+                if (kc < kchunks) {
+                    const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const int k = kc * 8 + e;
+                        const int half = BMS == 64 ? ((m >> 5) ^ ((k >> 1) & 1)) * 64 : 0;
+                        if (k < k_rows)
+                            *reinterpret_cast<uint16_t *>(dst + k * ROWB + half) =
+                                (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
+                    }
+                }
+            }
+        }
+    };
     auto load_panel = [&]() {
         const int total = k_rows * CH;
         const uint32_t lda_b = (uint32_t)p.lda * 2u;
@@ -1399,6 +1448,26 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
         if (!last_segment(c))
             return;
         const int cnt = min(32, c.u.n_cnt - c.nb * 32);
+        if (RM) {
+            // rows m_lane + 8 * g + e, g = 0 .. 4 MI - 1, e = 0 .. 3: a running pointer, so that
+            // the 16 MI addresses are not all worked out (and kept in registers) ahead
+            const int m_lane = m0 + (lane >> 5) * 4;
+            uint16_t *cp = C + (int64_t)m_lane * p.ldc + out_col;
+#pragma unroll
+            for (int g = 0; g < 4 * MI; ++g) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const uint16_t h = (uint16_t)E::to_bits(
+                        tw_fp32_value(tw_activate(p.alpha * acc[g >> 2][(g & 3) * 4 + e] + out_bias, p.act)));
+                    if (j < cnt && m_lane + g * 8 + e < m_end)
+                        cp[(int64_t)e * p.ldc] = h;
+                }
+                cp += 8 * p.ldc;
+                asm volatile("" : "+v"(cp));
+            }
+            clear();
+            return;
+        }
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
             const int mloc = (lane >> 5) * 4;
@@ -1407,7 +1476,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
                 uint32_t h[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    h[e] = E::to_bits(tw_activate(p.alpha * acc[mi][r4 * 4 + e] + out_bias, p.act));
+                    h[e] = E::to_bits(tw_fp32_value(tw_activate(p.alpha * acc[mi][r4 * 4 + e] + out_bias, p.act)));
                 u32x2 pk;
                 pk.x = h[0] | (h[1] << 16);
                 pk.y = h[2] | (h[3] << 16);
@@ -1437,7 +1506,10 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
     Cursor cur = open_block(b_first, b_first < n_blocks ? __builtin_amdgcn_readfirstlane(blocks[b_first]) : 0);
     if (valid(cur))
         issue(cur, g0); // weight and row numbers do not wait for the panel
-    load_panel();
+    if (RM)
+        load_panel_row_major();
+    else
+        load_panel();
     __syncthreads();
     if (valid(cur)) {
         for (;;) {
@@ -1461,6 +1533,15 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
     // ---- TW_PRUNED_ZERO: the pruned columns of this group's tiles receive act(bias)
     for (int z = p.n_gemm_u + group; z < p.n_all_u; z += n_groups) {
         const TileDev t = p.tiles[z - p.n_gemm_u];
+        if (RM) {
+            for (int i = tid; i < t.n_pruned * BMS; i += NT) {
+                const int m = m0 + i / t.n_pruned;
+                const int c = t.col0 + p.pruned_n[t.pn_off + i % t.n_pruned];
+                if (m < m_end)
+                    C[(int64_t)m * p.ldc + c] = (uint16_t)E::to_bits(tw_finish(0.0f, p.bias, c, p.act));
+            }
+            continue;
+        }
         for (int i = tid; i < t.n_pruned * CH; i += NT) {
             const int jz = i / CH, ch = i % CH;
             const int c = t.col0 + p.pruned_n[t.pn_off + jz];
@@ -1846,12 +1927,17 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
 }
 
 // the A-stationary kernel: one workgroup per (row block, group of blocks); no work queue
-template <int DT, int BMS> static int launch_as(const tw_plan *plan, const GemmArgs &a, int M, hipStream_t s)
+bool takes_row_major_directly(const tw_plan *plan, float beta)
+{
+    return beta == 0.0f && plan->d_kept_pairs && plan->n_blocks > 0 && as_lds_bytes(plan->K, 32) <= kLdsBytes;
+}
+
+template <int DT, int BMS, bool RM> static int launch_as(const tw_plan *plan, const GemmArgs &a, int M, hipStream_t s)
 {
     static std::once_flag once;
     static hipError_t attr_err = hipSuccess;
     std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute((const void *)tw_gemm_as_kernel<DT, BMS>,
+        attr_err = hipFuncSetAttribute((const void *)tw_gemm_as_kernel<DT, BMS, RM>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
     });
     if (attr_err != hipSuccess)
@@ -1864,7 +1950,7 @@ template <int DT, int BMS> static int launch_as(const tw_plan *plan, const GemmA
     if ((int64_t)n_mblk * n_groups > (int64_t)0x7fffffff)
         return fail(TW_ERR_SHAPE, "%lld workgroups (M=%d): a launch takes at most %lld",
                     (long long)n_mblk * n_groups, M, (long long)(int64_t)0x7fffffff);
-    hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS>), dim3((unsigned)(n_mblk * n_groups)),
+    hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS, RM>), dim3((unsigned)(n_mblk * n_groups)),
                        dim3(64 * kAsWaves), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
                        n_mblk, plan->K);
     TW_HIP(hipGetLastError());
@@ -1998,10 +2084,10 @@ int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *tick
         a.arg_units[i] = plan->h_units[i];
     if (is_as_shape(c.shape)) {
         if (plan->dtype == TW_F16)
-            return c.shape == TW_SHAPE_AS64 ? launch_as<TW_F16, 64>(plan, a, a.M, s)
-                                            : launch_as<TW_F16, 32>(plan, a, a.M, s);
-        return c.shape == TW_SHAPE_AS64 ? launch_as<TW_BF16, 64>(plan, a, a.M, s)
-                                        : launch_as<TW_BF16, 32>(plan, a, a.M, s);
+            return c.shape == TW_SHAPE_AS64 ? launch_as<TW_F16, 64, false>(plan, a, a.M, s)
+                                            : launch_as<TW_F16, 32, false>(plan, a, a.M, s);
+        return c.shape == TW_SHAPE_AS64 ? launch_as<TW_BF16, 64, false>(plan, a, a.M, s)
+                                        : launch_as<TW_BF16, 32, false>(plan, a, a.M, s);
     }
     // queue 0 is the longest: one workgroup per entry, up to the chip's share of a queue
     const int64_t qlen0 = (int64_t)a.n_own_items + (a.n_tail_items + kXcd - 1) / kXcd;
@@ -2054,6 +2140,24 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
         return st;
     GemmArgs a;
     fill_common(a, plan, A, lda, C, ldc, M, alpha, beta, ep);
+    if (a_layout == TW_LAYOUT_ROWMAJOR && c_layout == TW_LAYOUT_ROWMAJOR && takes_row_major_directly(plan, beta)) {
+        // both operands row-major, K short enough for a panel of A in LDS, C not read: the
+        // A-stationary kernel in its row-major form (64-row panels where they fit and still give
+        // three quarters of the compute units a workgroup)
+        fill_queues(a, plan, M, 64, 128, pruned_cols, false);
+        a.n_arg_units = plan->n_units <= kMaxArgUnits ? plan->n_units : 0;
+        for (int i = 0; i < a.n_arg_units; ++i)
+            a.arg_units[i] = plan->h_units[i];
+        const int mblk64 = (M + 63) / 64;
+        const int groups64 =
+            std::min(std::max(1, plan->cu_count / mblk64), (plan->n_blocks + kAsWaves - 1) / kAsWaves);
+        const bool b64 = as_lds_bytes(plan->K, 64) <= kLdsBytes &&
+                         (int64_t)mblk64 * groups64 * 4 >= (int64_t)plan->cu_count * 3;
+        hipStream_t s = (hipStream_t)stream;
+        if (plan->dtype == TW_F16)
+            return b64 ? launch_as<TW_F16, 64, true>(plan, a, M, s) : launch_as<TW_F16, 32, true>(plan, a, M, s);
+        return b64 ? launch_as<TW_BF16, 64, true>(plan, a, M, s) : launch_as<TW_BF16, 32, true>(plan, a, M, s);
+    }
     if (a_layout != TW_LAYOUT_KMAJOR || c_layout != TW_LAYOUT_KMAJOR) {
         // layout-generic path (element strides), 128-row blocks, one workgroup per item
         fill_queues(a, plan, M, 128, 128, pruned_cols, false);

@@ -172,6 +172,9 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s);
 int pack_from_dense(tw_plan *p, const float *d_B, hipStream_t s, const uint8_t *d_mask = nullptr);
 // device pack: packed weight from the reference's compacted stream layout (16-bit, device)
 int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStream_t s);
+// true when tw_gemm_ex takes a row-major A and a row-major C of this plan with a kernel of its own
+// (no layout-generic kernel, no staging): K short enough for a panel of A in LDS and C not read
+bool takes_row_major_directly(const tw_plan *p, float beta);
 // device unpack: compacted stream layout (K*N 16-bit, zero elsewhere) from the packed weight
 int unpack_to_stream(const tw_plan *p, uint16_t *d_Bs, hipStream_t s);
 

@@ -104,13 +104,15 @@ try {
     if (!plan)
         return fail(TW_ERR_NULL, "plan is NULL");
     const bool a_rm = a_layout == TW_LAYOUT_ROWMAJOR, c_rm = c_layout == TW_LAYOUT_ROWMAJOR;
-    if ((!a_rm && !c_rm) || M <= 0 || !A || !C)
+    if ((!a_rm && !c_rm) || M <= 0 || !A || !C || (a_rm && c_rm && takes_row_major_directly(plan, beta)))
         return tw_gemm_ex(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep,
-                          stream); // nothing to stage; also reports every argument error
+                          stream); // nothing to stage (K-major operands, or row-major ones a GEMM
+                                   // kernel takes as they are); also reports every argument error
     if ((a_rm && (lda < plan->K || (lda & 7))) || (c_rm && (ldc < plan->N || (ldc & 7))) ||
         ((uintptr_t)A & 15) || ((uintptr_t)C & 15))
         return tw_gemm_ex(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep,
                           stream); // reports the error
+    // (row-major operands the GEMM kernels take directly need no staging: tw_gemm_ex tells)
     const int64_t need = tw_gemm_staged_workspace(plan, M, a_layout, c_layout);
     if (!workspace || workspace_bytes < need)
         return fail(TW_ERR_BUFFER, "workspace of %lld bytes, %lld needed (tw_gemm_staged_workspace)",

@@ -461,13 +461,13 @@ def test_every_kernel_shape_agrees(tw, oracle, dtype):
     rng = np.random.default_rng(88)
     W, S1, S2, S3, S4, S5 = (tw.SHAPE_WIDE, tw.SHAPE_128x128, tw.SHAPE_512x64, tw.SHAPE_128x64,
                              tw.SHAPE_256x128, tw.SHAPE_128x32)
-    A6, A3 = tw.SHAPE_AS64, tw.SHAPE_AS32
+    A6, A3, SK = tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY
     cases = (
         (600, 320, 384, 128, ((W, -1), (S1, -1), (S4, -1), (S3, 64), (S5, 32), (S1, 64), (S4, 32),
-                              (A6, -1), (A3, -1))),
+                              (A6, -1), (A3, -1), (SK, -1))),
         (1100, 200, 256, 64, ((S2, -1), (S3, -1), (S5, 32), (S1, -1), (S4, -1), (W, -1), (A6, -1),
-                              (A3, -1))),
-        (2500, 130, 96, 32, ((S5, -1), (S3, -1), (S2, -1), (A6, -1), (A3, -1))),
+                              (A3, -1), (SK, -1))),
+        (2500, 130, 96, 32, ((S5, -1), (S3, -1), (S2, -1), (A6, -1), (A3, -1), (SK, -1))),
     )
     try:
         for (M, K, N, G, combos) in cases:
@@ -498,7 +498,8 @@ def test_a_stationary_shapes(tw, oracle, dtype):
     chosen with tw_set_option only.  Tiles from no kept row to all of them (one to five segments of
     four steps), ragged M, bias + activation, filled pruned columns: bit for bit what the streaming
     256 x 128 kernel gives, and within tolerance of the oracle.  With beta != 0 (C is read) the
-    forced shape does not apply and the launch takes the default kernel."""
+    forced shape does not apply and the launch takes the default kernel (for these few rows the
+    skinny one, whose sums run in slices: within half the tolerance)."""
     rng = np.random.default_rng(4321)
     M, K, N, G = 333, 1100, 640, 128
     A = rng.standard_normal((M, K)).astype(np.float32)
@@ -540,7 +541,7 @@ def test_a_stationary_shapes(tw, oracle, dtype):
                 want = launch(plan, tw.SHAPE_256x128, alpha, beta, pruned, with_bias, act)
                 for shape in (tw.SHAPE_AS64, tw.SHAPE_AS32):
                     got = launch(plan, shape, alpha, beta, pruned, with_bias, act)
-                    if act == tw.ACT_GELU:
+                    if act == tw.ACT_GELU or beta != 0.0:
                         # the two kernels evaluate the polynomial inside GELU in loops of their
                         # own; the compiler fuses their multiply-adds differently: last-bit ties
                         a = oracle.bits_to_f32(got[:, :M], dtype)
@@ -551,6 +552,77 @@ def test_a_stationary_shapes(tw, oracle, dtype):
                         assert np.array_equal(got, want), (shape, alpha, beta, pruned, with_bias, act)
                 if not with_bias and act == tw.ACT_NONE:
                     Cf = oracle.bits_to_f32(want[:, :M], dtype).reshape(N, M).T
+                    ref = reference(oracle, A, B, tiles, dtype, alpha, beta, C0)
+                    assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
+    finally:
+        tw.set_option(tw.OPT_SHAPE, -1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [1, 31, 64, 100, 129, 200])
+def test_skinny_kernel(tw, oracle, dtype, M):
+    """The skinny kernel (32 rows of A and half a unit per workgroup, the kept rows split over its
+    waves, the partial sums added in wave order) is what few rows of A get by default.  Tiles from
+    no kept row over one step to 23 steps (three rounds of pairs, the last one odd), 7 to 128
+    kept columns, ragged M, alpha / beta, bias + activation, filled pruned columns: within half
+    the tolerance of the streaming 256 x 128 kernel (the sum over k runs in four slices), bit for
+    bit what it gives where nothing is summed (pruned columns, tiles without kept rows), nothing
+    written outside, and the same bits on a second launch."""
+    rng = np.random.default_rng(555 + M)
+    K, N, G = 1500, 768, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tiles = []
+    for t, (kt, nt) in enumerate(((1460, 128), (64, 100), (0, 128), (333, 65), (700, 7), (1, 33))):
+        tiles.append(dict(col0=t * G, width=G,
+                          kept_k=np.sort(rng.choice(K, size=kt, replace=False)).astype(np.int32),
+                          kept_n=np.sort(rng.choice(G, size=nt, replace=False)).astype(np.int32)))
+    keep = kept_columns(tiles, N)
+    import torch
+    dbias = torch.from_numpy(bias).cuda()
+    lda = ldc = round_up(M, 8) + 8
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    dA = to_device_bits(At, At.shape)
+
+    def launch(plan, shape, alpha, beta, pruned, with_bias, act):
+        Cb = np.full((N, ldc), SENTINEL, np.uint16)
+        Cb[:, :M] = oracle.cast_bits(C0, dtype).reshape(M, N).T
+        dC = to_device_bits(Cb, Cb.shape)
+        tw.set_option(tw.OPT_SHAPE, shape)
+        print("skinny test: shape", shape, M, alpha, beta, pruned, with_bias, act, dtype, flush=True)
+        plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
+                  pruned_cols=pruned, bias_ptr=dbias.data_ptr() if with_bias else None, activation=act,
+                  stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return from_device_bits(dC)
+
+    no_sum = np.ones(N, bool)                   # columns whose value does not come from a sum over k
+    for t in tiles:
+        if len(t["kept_k"]):
+            no_sum[t["col0"] + t["kept_n"]] = False
+    try:
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            for (alpha, beta, pruned, with_bias, act) in (
+                    (1.0, 0.0, tw.PRUNED_UNTOUCHED, False, tw.ACT_NONE),
+                    (0.5, 0.0, tw.PRUNED_ZERO, True, tw.ACT_RELU),
+                    (1.0, 0.0, tw.PRUNED_ZERO, True, tw.ACT_TANH),
+                    (2.0, 0.75, tw.PRUNED_ZERO, False, tw.ACT_NONE),
+                    (1.0, -0.5, tw.PRUNED_UNTOUCHED, True, tw.ACT_GELU)):
+                want = launch(plan, tw.SHAPE_256x128, alpha, beta, pruned, with_bias, act)
+                got = launch(plan, -1, alpha, beta, pruned, with_bias, act)     # the default: skinny
+                forced = launch(plan, tw.SHAPE_SKINNY, alpha, beta, pruned, with_bias, act)
+                assert np.array_equal(got, forced)
+                assert np.array_equal(got[:, M:], want[:, M:])                  # padding untouched
+                if act != tw.ACT_GELU:
+                    assert np.array_equal(got[no_sum], want[no_sum])
+                a = oracle.bits_to_f32(got[:, :M], dtype)
+                b = oracle.bits_to_f32(want[:, :M], dtype)
+                assert oracle.rel_error(a, b) <= 0.5 * TOL[dtype], (alpha, beta, pruned, with_bias, act)
+                if not with_bias and act == tw.ACT_NONE:
+                    Cf = a.reshape(N, M).T
                     ref = reference(oracle, A, B, tiles, dtype, alpha, beta, C0)
                     assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
     finally:

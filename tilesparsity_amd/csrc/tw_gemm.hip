@@ -43,6 +43,7 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
 #define TW_LDS(T) __attribute__((address_space(3))) T *
+#define TW_GLOBAL(T) __attribute__((address_space(1))) T *
 
 #ifndef TW_A_PAD
 #define TW_A_PAD 32 // halfs of padding per staged A row: 64 B, so that the 4 rows x 2 column
@@ -117,6 +118,23 @@ __device__ __forceinline__ float tw_activate(float v, int act)
     if (act == TW_ACT_TANH)
         return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * v) + 1.0f);
     return v;
+}
+// the same for a handful of values with the test of `act` outside the loop over them
+template <int N> __device__ __forceinline__ void tw_activate_all(float (&v)[N], int act)
+{
+    if (act == TW_ACT_RELU) {
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+            v[e] = tw_activate(v[e], TW_ACT_RELU);
+    } else if (act == TW_ACT_GELU) {
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+            v[e] = tw_activate(v[e], TW_ACT_GELU);
+    } else if (act == TW_ACT_TANH) {
+#pragma unroll
+        for (int e = 0; e < N; ++e)
+            v[e] = tw_activate(v[e], TW_ACT_TANH);
+    }
 }
 // The value of an output element is rounded to fp32 before it is rounded to 16 bits, in every
 // kernel: left to itself the compiler turns "multiply, add, convert" into one fused instruction
@@ -1454,11 +1472,21 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
             const int m_lane = m0 + (lane >> 5) * 4;
             uint16_t *cp = C + (int64_t)m_lane * p.ldc + out_col;
 #pragma unroll
+            for (int mi = 0; mi < MI; ++mi) {
+                float v[16];
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    v[r] = p.alpha * acc[mi][r] + out_bias;
+                tw_activate_all(v, p.act);
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[mi][r] = tw_fp32_value(v[r]);
+            }
+#pragma unroll
             for (int g = 0; g < 4 * MI; ++g) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const uint16_t h = (uint16_t)E::to_bits(
-                        tw_fp32_value(tw_activate(p.alpha * acc[g >> 2][(g & 3) * 4 + e] + out_bias, p.act)));
+                    const uint16_t h = (uint16_t)E::to_bits(acc[g >> 2][(g & 3) * 4 + e]);
                     if (j < cnt && m_lane + g * 8 + e < m_end)
                         cp[(int64_t)e * p.ldc] = h;
                 }
@@ -1471,12 +1499,17 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
 #pragma unroll
         for (int mi = 0; mi < MI; ++mi) {
             const int mloc = (lane >> 5) * 4;
+            float v[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                v[r] = p.alpha * acc[mi][r] + out_bias;
+            tw_activate_all(v, p.act); // the test of the activation outside the loop over the elements
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 uint32_t h[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
-                    h[e] = E::to_bits(tw_fp32_value(tw_activate(p.alpha * acc[mi][r4 * 4 + e] + out_bias, p.act)));
+                    h[e] = E::to_bits(tw_fp32_value(v[r4 * 4 + e]));
                 u32x2 pk;
                 pk.x = h[0] | (h[1] << 16);
                 pk.y = h[2] | (h[3] << 16);
@@ -1549,6 +1582,280 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
             const uint32_t w = hb | (hb << 16);
             store_chunk(C + (int64_t)c * p.ldc + m0 + ch * 8, u32x4{w, w, w, w}, m0 + ch * 8, m_end,
                         p.store_through != 0);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Skinny kernel for a handful of rows of A (one time step of a recurrent cell: M = 128): the
+// launch is then a chain of dependent trips to memory on an almost empty chip, and the streaming
+// kernels walk a tile's kept rows 64 at a time, one trip per step.  Here a workgroup takes
+// 32 rows m of one half of a unit (up to 64 compact columns) and its four waves split the kept
+// rows between them: wave w takes the steps w, w + 4, ... of 64 kept rows, two at a time: it
+// fetches their row numbers, then their 8 KB of A and 16 KB of weight fragments in one go, turns
+// A through its own piece of LDS (no barrier: nobody else reads it) and multiplies.  The four
+// partial products meet in LDS once, are added in wave order (so the result does not depend on
+// timing) and leave through one rounding.  A tile of 512 kept rows is one trip to memory for the
+// numbers and one for the operands.
+//   work:  workgroup (x, y): die x % 8, unit (x / 16) * 8 + die, half (x / 8) % 2, row block y
+//          (a plan without units wider than 64 columns is launched without second halves);
+//          the unit comes from the kernel arguments at an offset that depends on the workgroup
+//          number alone, so that it arrives with the other arguments; the halves and row blocks
+//          of a unit sit on one die and share its rows of A in that L2; workgroups of a half the
+//          unit does not have fill pruned columns (TW_PRUNED_ZERO) or leave
+//   stage: per wave 2 x 64 rows k of 32 rows m (64 bytes each), then reused for the wave's
+//          partial product [64 columns][32 + 4 rows m] in fp32
+// K-major A and C; any beta.  The sum over k runs in four slices, so the result can differ from
+// the streaming kernels' in the last bit of fp32 before the rounding to 16 bits.
+constexpr int kSkWaves = 4;
+constexpr int kSkRows = 32;                            // rows m of a workgroup
+constexpr int kSkCols = 64;                            // compact columns of a workgroup
+constexpr int kSkPitch = kSkRows + 4;                  // floats per column of a partial product
+constexpr int kSkStage = kSkCols * kSkPitch * 4;       // 9216 bytes >= 2 * 64 * 64
+constexpr int kSkLdsBytes = kSkWaves * kSkStage;
+
+template <int DT>
+__global__ void __launch_bounds__(64 * kSkWaves, 1) tw_gemm_skinny_kernel(const GemmArgs p, int n_units, int halves)
+{
+    constexpr int NT = 64 * kSkWaves;
+    using E = Elem<DT>;
+    __shared__ __align__(16) unsigned char sk_smem[kSkLdsBytes];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int die = blockIdx.x % kXcd, rest = blockIdx.x / kXcd;
+    // (halves: 2, or 1 for a plan whose units all have at most 64 compact columns)
+    const int half = halves == 2 ? rest & 1 : 0, ui = (halves == 2 ? rest >> 1 : rest) * kXcd + die;
+    // the arguments the first loads need, asked for together with the unit
+    // (as integers: a pointer that has been through an asm statement is no longer known to
+    // point to global memory)
+    uintptr_t A_i = (uintptr_t)p.A, kk_i = (uintptr_t)p.kept_k, kn_i = (uintptr_t)p.kept_n, Bp_i = (uintptr_t)p.Bp;
+    int64_t lda = p.lda, ldc = p.ldc;
+    int M = p.M;
+    const bool in_range = ui < n_units;
+    const int m0 = blockIdx.y * kSkRows;
+    // the unit: asked for from the kernel arguments before anything else has arrived
+    UnitDev u;
+    {
+        const auto *ka = (const __attribute__((address_space(4))) int32_t *)__builtin_amdgcn_kernarg_segment_ptr();
+        const int ua = ui < kMaxArgUnits ? ui : 0;
+        int32_t w[12];
+#pragma unroll
+        for (int i = 0; i < 12; ++i)
+            w[i] = ka[offsetof(GemmArgs, arg_units) / 4 + ua * 12 + i];
+        const int n_arg_units = p.n_arg_units;
+#pragma unroll
+        for (int i = 0; i < 12; ++i)
+            asm volatile("" : "+s"(w[i])); // asked for here, not behind the test below
+        asm volatile("" : "+s"(A_i), "+s"(kk_i), "+s"(kn_i), "+s"(Bp_i), "+s"(lda), "+s"(ldc), "+s"(M));
+        if (!n_arg_units) {
+            const auto *gu = (const __attribute__((address_space(4))) int32_t *)(uintptr_t)(p.units + (in_range ? ui : 0));
+#pragma unroll
+            for (int i = 0; i < 12; ++i)
+                w[i] = gu[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 12; ++i)
+            w[i] = __builtin_amdgcn_readfirstlane(w[i]);
+        __builtin_memcpy(&u, w, sizeof(UnitDev));
+    }
+    const int m_end = m0 + kSkRows < M ? m0 + kSkRows : M;
+    TW_GLOBAL(const uint16_t) const A = (TW_GLOBAL(const uint16_t))A_i;
+    uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
+    TW_GLOBAL(const int32_t) const kept_k = (TW_GLOBAL(const int32_t))kk_i;
+    TW_GLOBAL(const int32_t) const kept_n = (TW_GLOBAL(const int32_t))kn_i;
+    TW_GLOBAL(const unsigned char) const Bp = (TW_GLOBAL(const unsigned char))Bp_i;
+
+    if (in_range && half * 2 < u.nb_cnt) {
+        const int nsteps = u.k_pad / kBlockK;
+        const bool two_blocks = half * 2 + 1 < u.nb_cnt;
+        unsigned char *const stage = sk_smem + wave * kSkStage;
+        // the reducing role of this lane: column jj of the half, rows m8 .. m8 + 7
+        const int jj = wave * 16 + (lane >> 2), m8 = (lane & 3) * 8;
+        const int cnt = min(kSkCols, u.n_cnt - half * kSkCols);
+
+        struct Numbers {
+            int row[2][4]; // rows of A this lane fetches a chunk of: kept row i * 16 + lane / 4 of step t
+        };
+        struct Loads {
+            u32x4 a[2][4], b[2][2][4];
+        };
+        TW_GLOBAL(const unsigned char) const bsrc = Bp + u.b_off * 2 +
+                                          (int64_t)(u.nb0 + half * 2) * 4096 + lane * 16;
+        const int64_t step_b = (int64_t)u.nblk * 4096;
+        const int ch = lane & 3, row16 = lane >> 2;
+        // Nothing on the way to the operands is conditional, so that the waits between the loads
+        // are exact counts: a chunk of rows past M is fetched from the row block's first chunk
+        // instead (those rows of the product are never stored), a second step past the end and a
+        // second block the half does not have repeat the first (and are not multiplied, or not
+        // stored).
+        TW_GLOBAL(const uint16_t) const a_lane = A + m0 + (m0 + ch * 8 < M ? ch * 8 : 0);
+        const int cb_off = two_blocks ? 4096 : 0;
+        // a pair of steps: s and s + kSkWaves (the second may be past the end)
+        auto numbers = [&](int s) {
+            Numbers n;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int st = s + t * kSkWaves < nsteps ? s + t * kSkWaves : s;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    n.row[t][i] = kept_k[u.kk_off + st * kBlockK + i * 16 + row16];
+            }
+            return n;
+        };
+        auto issue = [&](int s, const Numbers &n, Loads &l) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    l.a[t][i] = *(TW_GLOBAL(const u32x4))(a_lane + (int64_t)n.row[t][i] * lda);
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int st = s + t * kSkWaves < nsteps ? s + t * kSkWaves : s;
+#pragma unroll
+                for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+                    for (int k16 = 0; k16 < 4; ++k16)
+                        l.b[t][cb][k16] =
+                            *(TW_GLOBAL(const u32x4))(bsrc + st * step_b + cb * cb_off + k16 * 1024);
+            }
+        };
+        f32x16 acc[2];
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[cb][r] = 0.0f;
+        const int L = lane & 15;
+        const int pair_e = (lane >> 5) * 4 + (L >> 2);
+        const int lane_b = ((lane >> 4) & 1) * 32 + (L & 3) * 8;
+        const uint32_t r_first = (uint32_t)((pair_e >> 2) * 8 + (pair_e & 3));
+
+        // the steps of the pair at s out of one register set: A through the stage, the products
+        auto multiply = [&](int s, const Loads &l) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) = l.a[t][i];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the rows are in the stage
+            TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))stage + lane_b;
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+                if (s + t * kSkWaves < nsteps) {
+#pragma unroll
+                    for (int k16 = 0; k16 < 4; ++k16) {
+                        const uint32_t r_lo = t * 64 + r_first + k16 * 16, r_hi = r_lo + 4;
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_lo * 64));
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_hi * 64));
+                        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                        const u32x4 af = u32x4{l2.x, l2.y, h2.x, h2.y};
+                        acc[0] = E::mfma(af, l.b[t][0][k16], acc[0]);
+                        acc[1] = E::mfma(af, l.b[t][1][k16], acc[1]);
+                    }
+                }
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the next steps overwrite it
+        };
+        // One pair is multiplied out of one register set while the operands of the wave's next
+        // pair fill the other and the row numbers of the pair after that are on their way.
+        constexpr int kPair = 2 * kSkWaves;
+        int s = wave;
+        int out_col = 0;
+        float out_bias = 0.0f;
+        Loads l0, l1;
+        Numbers n;
+        if (s < nsteps) {
+            n = numbers(s);
+            issue(s, n, l0);
+            if (s + kPair < nsteps)
+                n = numbers(s + kPair);
+        }
+        // behind the first operands on their way: where this lane's sums go
+        out_col = u.col0 + kept_n[u.kn_off + half * kSkCols + (jj < cnt ? jj : 0)];
+        while (s < nsteps) {
+            if (s + kPair < nsteps) {
+                issue(s + kPair, n, l1);
+                if (s + 2 * kPair < nsteps)
+                    n = numbers(s + 2 * kPair);
+            }
+            multiply(s, l0);
+            s += kPair;
+            if (s >= nsteps)
+                break;
+            if (s + kPair < nsteps) {
+                issue(s + kPair, n, l0);
+                if (s + 2 * kPair < nsteps)
+                    n = numbers(s + 2 * kPair);
+            }
+            multiply(s, l1);
+            s += kPair;
+        }
+        if (p.bias)
+            out_bias = p.bias[out_col];
+        // the partial product of this wave: column cb * 32 + lane % 32, rows r4 * 8 + (lane / 32) * 4 + e
+        float *const part = reinterpret_cast<float *>(stage);
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                float *const dst = part + (cb * 32 + (lane & 31)) * kSkPitch + r4 * 8 + (lane >> 5) * 4;
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    dst[e] = acc[cb][r4 * 4 + e];
+            }
+        __syncthreads();
+        // (a wave without steps has written zeros)
+        float sum[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            sum[e] = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kSkWaves; ++w) {
+            const float *const src = reinterpret_cast<const float *>(sk_smem + w * kSkStage) + jj * kSkPitch + m8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                sum[e] += src[e];
+        }
+        if (jj < cnt && m0 + m8 < m_end) {
+            uint16_t *const dst = C + (int64_t)out_col * ldc + m0 + m8;
+            float v[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                v[e] = p.alpha * sum[e];
+            if (p.beta != 0.0f) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (m0 + m8 + e < m_end)
+                        v[e] += p.beta * E::from_bits(dst[e]);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                v[e] += out_bias;
+            tw_activate_all(v, p.act);
+            uint32_t h[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+                h[e] = E::to_bits(tw_fp32_value(v[e]));
+            store_chunk(dst, u32x4{h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)},
+                        m0 + m8, m_end, false);
+        }
+    }
+
+    // ---- TW_PRUNED_ZERO: pruned columns receive act(beta * C + bias); shared out over the
+    // workgroups of a row block
+    if (in_range) {
+        for (int z = p.n_gemm_u + ui * halves + half; z < p.n_all_u; z += n_units * halves) {
+            const TileDev t = p.tiles[z - p.n_gemm_u];
+            for (int i = tid; i < t.n_pruned * 4; i += NT) {
+                const int jz = i >> 2, m = m0 + (i & 3) * 8;
+                const int c = t.col0 + p.pruned_n[t.pn_off + jz];
+                uint16_t *const dst = C + (int64_t)c * ldc + m;
+                uint32_t w[4] = {0u, 0u, 0u, 0u};
+                for (int e = 0; e < 8 && m + e < m_end; ++e) {
+                    const float old = p.beta != 0.0f ? p.beta * E::from_bits(dst[e]) : 0.0f;
+                    w[e >> 1] |= E::to_bits(tw_finish(old, p.bias, c, p.act)) << ((e & 1) * 16);
+                }
+                store_chunk(dst, u32x4{w[0], w[1], w[2], w[3]}, m, m_end, false);
+            }
         }
     }
 }
@@ -1728,12 +2035,15 @@ static const Shape kShapes[TW_N_SHAPES] = {
     {256, 64, 1},  // TW_SHAPE_256x64
     {64, 128, 1},  // TW_SHAPE_AS64
     {32, 128, 1},  // TW_SHAPE_AS32
+    {32, 128, 1},  // TW_SHAPE_SKINNY
 };
 
 // LDS of the A-stationary kernel: the panel (all K rows, BMS rows m) and a C stage per wave
 constexpr int kLdsBytes = 160 * 1024;
 static int64_t as_lds_bytes(int K, int bms) { return (int64_t)K * bms * 2 + kAsWaves * 32 * 36 * 2; }
 static bool is_as_shape(int shape) { return shape == TW_SHAPE_AS64 || shape == TW_SHAPE_AS32; }
+// shapes that walk the plan's units themselves: no work queue, no unit pieces
+static bool is_queueless_shape(int shape) { return is_as_shape(shape) || shape == TW_SHAPE_SKINNY; }
 
 // Steps of loads a moving wave keeps in flight, per shape (bounded by its 256 registers: a step
 // takes 4 * (A loads + weight loads per thread) of them).  Measured on the benchmark shapes: two
@@ -1866,14 +2176,25 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
                as_lds_bytes(plan->K, kShapes[shape].bm) <= kLdsBytes;
     };
     const bool as_few = width <= 64 || items(256, 128) * 2 <= cu;
-    if (!ws_ok) {
+    // The skinny kernel where it gives a compute unit at most two workgroups: the launch is then
+    // a chain of trips to memory, which it keeps shortest (measured on M 16 .. 512 of the grid
+    // above, replayed from a graph: 1.6 - 3 x faster up to one workgroup per unit, 1.1 - 1.5 x
+    // up to two).
+    const bool skinny_ok = plan->n_units > 0 && (M + 31) / 32 <= 65535; // its grid: units x row blocks
+    const bool skinny = skinny_ok && (int64_t)plan->n_halves * ((M + 31) / 32) <= 2 * (int64_t)cu;
+    if (skinny) {
+        c.shape = TW_SHAPE_SKINNY;
+    } else if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
     } else if (as_ok(TW_SHAPE_AS64) && as_few && (M > 128 || plan->n_blocks >= 96)) {
         // 64-row panels where they still give three quarters of the compute units a workgroup
         const int mblk64 = (M + 63) / 64;
         const int groups64 = std::min(std::max(1, cu / mblk64), (plan->n_blocks + kAsWaves - 1) / kAsWaves);
         c.shape = (int64_t)mblk64 * groups64 * 4 >= (int64_t)cu * 3 ? TW_SHAPE_AS64 : TW_SHAPE_AS32;
-    } else if (!as_ok(TW_SHAPE_AS64) && as_ok(TW_SHAPE_AS32) && M > 128 && M <= 512) {
+    } else if (!as_ok(TW_SHAPE_AS64) && as_ok(TW_SHAPE_AS32) && M > 128 &&
+               (M <= 512 || (M <= 1024 && plan->n_blocks <= kAsWaves * std::max(1, cu / ((M + 31) / 32))))) {
+        // (up to 1024 rows where every wave still has at most one block: M 1024, K 2048, N 2048:
+        // 12.3 - 15.8 us against 14.4 - 20.2)
         c.shape = TW_SHAPE_AS32;
     } else if (width > 64) {
         if (items(128, 128) * 2 < cu) { // skinny: split the units until half the chip has work
@@ -1911,6 +2232,9 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     if (f_shape >= 0 && is_as_shape(f_shape)) {
         if (as_ok(f_shape))
             c.shape = f_shape;
+    } else if (f_shape == TW_SHAPE_SKINNY) {
+        if (skinny_ok)
+            c.shape = f_shape;
     } else if (f_shape >= 0 && (f_shape != TW_SHAPE_WIDE ? ws_ok : true)) {
         const int piece = f_piece > 0 ? f_piece : std::min(128, kShapes[f_shape].bn);
         if (std::min(piece, width) <= kShapes[f_shape].bn) {
@@ -1920,7 +2244,7 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     } else if (f_piece > 0 && std::min(f_piece, width) <= kShapes[c.shape].bn) {
         c.piece = f_piece;
     }
-    if (c.shape == TW_SHAPE_WIDE || is_as_shape(c.shape))
+    if (c.shape == TW_SHAPE_WIDE || is_queueless_shape(c.shape))
         c.piece = 128;
     c.per_cu = option(TW_OPT_WGS_PER_CU) > 0 ? option(TW_OPT_WGS_PER_CU) : kShapes[c.shape].wgs_per_cu;
     return c;
@@ -1953,6 +2277,21 @@ template <int DT, int BMS, bool RM> static int launch_as(const tw_plan *plan, co
     hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS, RM>), dim3((unsigned)(n_mblk * n_groups)),
                        dim3(64 * kAsWaves), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
                        n_mblk, plan->K);
+    TW_HIP(hipGetLastError());
+    return TW_OK;
+}
+
+// the skinny kernel: one workgroup per (half of a unit, 32-row block)
+template <int DT> static int launch_skinny(const tw_plan *plan, const GemmArgs &a, hipStream_t s)
+{
+    const int halves = plan->max_unit_n > kSkCols ? 2 : 1;
+    const int64_t gx = ((int64_t)plan->n_units + kXcd - 1) / kXcd * kXcd * halves;
+    const int64_t gy = (a.M + kSkRows - 1) / kSkRows;
+    if (gx > (int64_t)0x7fffffff || gy > 65535)
+        return fail(TW_ERR_SHAPE, "%lld x %lld workgroups (M=%d): the skinny kernel takes at most 65535 row blocks",
+                    (long long)gx, (long long)gy, a.M);
+    hipLaunchKernelGGL((tw_gemm_skinny_kernel<DT>), dim3((unsigned)gx, (unsigned)gy), dim3(64 * kSkWaves), 0, s, a,
+                       plan->n_units, halves);
     TW_HIP(hipGetLastError());
     return TW_OK;
 }
@@ -2089,6 +2428,8 @@ int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *tick
         return c.shape == TW_SHAPE_AS64 ? launch_as<TW_BF16, 64, false>(plan, a, a.M, s)
                                         : launch_as<TW_BF16, 32, false>(plan, a, a.M, s);
     }
+    if (c.shape == TW_SHAPE_SKINNY)
+        return plan->dtype == TW_F16 ? launch_skinny<TW_F16>(plan, a, s) : launch_skinny<TW_BF16>(plan, a, s);
     // queue 0 is the longest: one workgroup per entry, up to the chip's share of a queue
     const int64_t qlen0 = (int64_t)a.n_own_items + (a.n_tail_items + kXcd - 1) / kXcd;
     const int64_t per_queue = std::max<int64_t>(1, (int64_t)plan->cu_count * c.per_cu / kXcd);

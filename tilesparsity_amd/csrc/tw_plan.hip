@@ -565,6 +565,7 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
     std::vector<int32_t> pruned_n;
     std::vector<int32_t> kept_k_pad; // the GEMM kernel's copy: k_pad entries per tile
     p->max_unit_n = 0;
+    p->n_halves = 0;
     for (int t = 0; t < nt; ++t) {
         const int kt = p->kept_k_ptr[t + 1] - p->kept_k_ptr[t];
         const int ntk = p->kept_n_ptr[t + 1] - p->kept_n_ptr[t];
@@ -598,6 +599,7 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
             u.nblk = p->n_pad[t] / kMfmaN;
             units.push_back(u);
             p->max_unit_n = std::max(p->max_unit_n, u.n_cnt);
+            p->n_halves += (u.n_cnt + 63) / 64;
         }
         if (ntk < p->tile_width[t]) {
             TileDev z;

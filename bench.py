@@ -470,6 +470,48 @@ def bench_shape_grid(torch, Ms=(128, 512, 2048, 8192, 16384), Ks=(512, 1024, 204
                       "worst_ratio": worst}), flush=True)
 
 
+def bench_mix(torch, g1s=(0.1, 0.25, 0.5, 1.0, 5.0), steps=30, warmup=5):
+    """The two ways to run a mixed mask (tiled_wise_1d_mix at 75 %, i.i.d. weights) on the headline
+    shape: the covering plan, and the plan of the tile-wise stage followed by tw_side_gemm on the
+    element-wise remainder.  One JSON line per g1percent with the times in us."""
+    from tilesparsity_amd import twgemm as tw, twprune
+    M, K, N, G = 12544, 4608, 512, 128
+    rng = np.random.default_rng(3)
+    W = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    scores = twprune.img2col_forward([W])
+    n_tiles = (N + G - 1) // G
+    table = [(t * G, min(G, N - t * G)) for t in range(n_tiles)]
+    bufs = [(torch.randn((K, M), device="cuda").half(), torch.zeros((N, M), dtype=torch.float16, device="cuda"))
+            for _ in range(4)]
+    s = torch.cuda.current_stream().cuda_stream
+    for g1 in g1s:
+        mask = twprune.tiled_wise_1d_mix(scores, 75, G, g1)[0]
+        mask0 = twprune.tiled_wise_1d(scores, 75 + g1, G)[0]
+        with tw.Plan.from_mask_tiles(mask0, table, "f16", W) as plan0, \
+                tw.Plan.from_mask_tiles(mask, table, "f16", W, cover=True) as cover, \
+                tw.Side(mask & ~mask0, "f16", W) as side:
+            def run_tw(i):
+                a, c = bufs[i % 4]
+                plan0.gemm(a.data_ptr(), c.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO, stream=s)
+
+            def run_side(i):
+                a, c = bufs[i % 4]
+                side.gemm(a.data_ptr(), c.data_ptr(), M, stream=s)
+
+            def run_pair(i):
+                run_tw(i)
+                run_side(i)
+
+            def run_cover(i):
+                a, c = bufs[i % 4]
+                cover.gemm(a.data_ptr(), c.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO, stream=s)
+            t = {name: min(time_steps(fn, steps, warmup, torch) for _ in range(3)) * 1e6
+                 for name, fn in (("us_tw_stage", run_tw), ("us_side", run_side), ("us_tw_then_side", run_pair),
+                                  ("us_covering_plan", run_cover))}
+            print(json.dumps(dict(workload="vgg16_conv4_2 M=12544 K=4608 N=512 G=128, tiled_wise_1d_mix 75 %",
+                                  g1percent=g1, remainder_elements=side.nnz, **t)), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -485,6 +527,9 @@ def main():
     ap.add_argument("--shape-grid", action="store_true",
                     help="time the automatic kernel-shape choice against every forced shape on a "
                          "grid of problems (several minutes)")
+    ap.add_argument("--mix", action="store_true",
+                    help="time the two ways to run a mixed (tile-wise + element-wise) mask: the covering "
+                         "plan and the tile-wise plan followed by the side kernel")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB device copy (4 launches over rotating buffers), "
                          "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
@@ -502,6 +547,9 @@ def main():
     tw.lib()  # fails loudly if the HIP library has not been built
     if args.shape_grid:
         bench_shape_grid(torch)
+        return 0
+    if args.mix:
+        bench_mix(torch)
         return 0
     if args.producers:
         print(json.dumps(bench_producers(min(args.steps, 20), min(args.warmup, 3), torch)), flush=True)

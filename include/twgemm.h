@@ -335,6 +335,27 @@ int tw_delete_row(const void *matrix, void *matrix_2, int rows, int columns,
 int tw_insert_row(void *matrix, const void *matrix_2, int rows, int columns,
                   const int32_t *mask, void *stream);
 
+/* The element-wise remainder of a mixed mask.  The reference's mixed producers
+ * (tiled_wise_1d_mix / tiled_wise_2d_mix, tw_mix_fn, Pruning/VGG/prune_algo.py:151-193) keep a
+ * tile-wise mask mask0 plus the g1percent largest of the elements mask0 drops; the masked layer
+ * is then x @ (kernel * mask) with mask = mask0 | remainder (mask_dense,
+ * Pruning/BERT/utils/modeling.py:992-1007).  mask0 runs as a plan (tw_plan_from_mask_tiles);
+ * tw_side_create takes the remainder - a K x N byte mask, row-major, non-zero = kept, normally
+ * mask & ~mask0 - and the fp32 row-major weight B (both host memory) and keeps its elements
+ * column by column on the device, their values rounded to `dtype`.  tw_side_gemm adds
+ *   C += alpha * A * (B (.) remainder)
+ * to a K-major C (column n at C + n * ldc) from a K-major A, as tw_gemm takes them, with vector
+ * multiply-adds in fp32 and one rounding of every touched element of C; columns without a
+ * remainder element are not touched.  Run it after the plan's tw_gemm on the same stream.  Any
+ * mask at all is a valid remainder (tw_plan_from_mask_cover is the alternative for masks whose
+ * remainder clusters in few rows). */
+typedef struct tw_side tw_side;
+int tw_side_create(int K, int N, int dtype, const uint8_t *mask, const float *B, tw_side **out);
+void tw_side_destroy(tw_side *side);
+int64_t tw_side_nnz(const tw_side *side); /* elements of the remainder */
+int tw_side_gemm(const tw_side *side, const void *A, int64_t lda, void *C, int64_t ldc, int M,
+                 float alpha, void *stream);
+
 /* LSTM gate arithmetic of the reference's NMT model, whose cells are TensorFlow 1.x
  * tf.contrib.rnn.BasicLSTMCell (Pruning/NMT/nmt/model_helper.py:400-402; BasicLSTMCell.call in
  * tensorflow/python/ops/rnn_cell_impl.py): with i, j, f, o the four H-wide blocks of the gate

@@ -160,3 +160,101 @@ def test_full_size_network_all_producers(twprune, po):
     want = po.tiled_wise_2d_mix(scores, 75, 128, 1)
     got = twprune.tiled_wise_2d_mix(scores, 75, 128, 1)
     assert all(np.array_equal(w, g) for w, g in zip(want, got))
+
+
+def _mixed_layer(rng, twprune, K, N, G, sparsity, g1, structured):
+    """Weight, the TW mask of the mixed producer's first stage and the mixed mask."""
+    W = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    if structured:
+        W *= (rng.random((K, 1)) < 0.5) * 0.9 + 0.1
+    scores = twprune.img2col_forward([W])
+    mask = twprune.tiled_wise_1d_mix(scores, sparsity, G, g1)[0]
+    mask0 = twprune.tiled_wise_1d(scores, sparsity + g1, G)[0]
+    assert not (mask0 & ~mask).any()          # the mixed mask only adds elements
+    return W, mask0, mask
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M", [200, 513])
+def test_side_kernel_runs_the_remainder(tw, twprune, po, oracle, dtype, M):
+    """TW plan of the first stage's mask + tw_side_gemm on what the second stage adds = the masked
+    layer A (B (.) mask) of the mixed mask.  The two passes round their results to 16 bits one
+    after the other, so an element's error is relative to the larger of the tile-wise part and
+    the sum (where the remainder cancels the tile-wise part, the first rounding stays): within
+    the GEMM tolerance of the float64 products of the 16-bit operands on that scale.  The side
+    call alone adds exactly the remainder's product (checked against a launch on zeros, one
+    rounding: plain relative error), leaves columns without remainder elements and the padding
+    beyond M untouched, and repeats bit for bit."""
+    import torch
+    from tests.test_gpu_gemm import to_device_bits, from_device_bits, round_up, SENTINEL
+    rng = np.random.default_rng(77 + M)
+    K, N, G = 320, 384, 128
+    W, mask0, mask = _mixed_layer(rng, twprune, K, N, G, 70, 2, structured=True)
+    rem = mask & ~mask0
+    rem[:, 5] = False                          # a column without remainder elements
+    rem[:, 300:310] = False
+    mask = mask0 | rem
+    table = po.tiles_every_g_columns(N, G)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    lda = ldc = round_up(M, 8) + 8
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    dA = to_device_bits(At, At.shape)
+    s = torch.cuda.current_stream().cuda_stream
+    tol = 1e-2 if dtype == "f16" else 2e-2
+    with tw.Plan.from_mask_tiles(mask0, table, dtype, W) as plan, tw.Side(rem, dtype, W) as side:
+        assert side.nnz == int(rem.sum())
+        outs = []
+        for rep in range(2):
+            dC = to_device_bits(np.full((N, ldc), SENTINEL, np.uint16), (N, ldc))
+            print("side test: plan + side", M, dtype, rep, flush=True)
+            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, pruned_cols=tw.PRUNED_ZERO, stream=s)
+            side.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, stream=s)
+            torch.cuda.synchronize()
+            outs.append(from_device_bits(dC))
+        assert np.array_equal(outs[0], outs[1])
+        assert (outs[0][:, M:] == SENTINEL).all()
+        C = oracle.bits_to_f32(outs[0][:, :M], dtype).reshape(N, M).T
+        Aq, Wq = oracle.quantize(A, dtype).astype(np.float64), oracle.quantize(W, dtype).astype(np.float64)
+        ref, ref_tw = Aq @ (Wq * mask), Aq @ (Wq * mask0)
+        floor = 1e-2 * np.sqrt(np.mean(ref * ref))
+        assert np.max(np.abs(C - ref) / np.maximum(np.maximum(np.abs(ref), np.abs(ref_tw)), floor)) <= tol
+        # the side call alone, on zeros, with alpha: exactly alpha * A (W (.) rem), one rounding
+        dZ = to_device_bits(np.zeros((N, ldc), np.uint16), (N, ldc))
+        side.gemm(dA.data_ptr(), dZ.data_ptr(), M, lda=lda, ldc=ldc, alpha=-0.5, stream=s)
+        torch.cuda.synchronize()
+        Z = from_device_bits(dZ)
+        untouched = ~rem.any(axis=0)
+        assert (Z[untouched] == 0).all() and (Z[:, M:] == 0).all()
+        Zf = oracle.bits_to_f32(Z[:, :M], dtype).reshape(N, M).T
+        assert oracle.rel_error(Zf, -0.5 * (Aq @ (Wq * rem))) <= tol
+
+
+def test_side_edge_cases_and_errors(tw):
+    import torch
+    K, N, M = 64, 40, 16
+    W = np.ones((K, N), np.float32)
+    dA = torch.ones((K, M), dtype=torch.float16, device="cuda")
+    dC = torch.full((N, M), 3.0, dtype=torch.float16, device="cuda")
+    with tw.Side(np.zeros((K, N), bool), "f16", W) as side:       # an empty remainder does nothing
+        assert side.nnz == 0
+        side.gemm(dA.data_ptr(), dC.data_ptr(), M)
+        torch.cuda.synchronize()
+        assert (dC == 3.0).all()
+    full = np.ones((K, N), bool)
+    with tw.Side(full, "f16", W) as side:                         # every element: a dense product
+        assert side.nnz == K * N
+        side.gemm(dA.data_ptr(), dC.data_ptr(), 0)                # M = 0: nothing
+        side.gemm(dA.data_ptr(), dC.data_ptr(), M)
+        torch.cuda.synchronize()
+        assert (dC == 3.0 + K).all()
+        with pytest.raises(tw.TwError):
+            side.gemm(0, dC.data_ptr(), M)
+        with pytest.raises(tw.TwError):
+            side.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=M - 8)
+        with pytest.raises(tw.TwError):
+            side.gemm(dA.data_ptr(), dC.data_ptr(), M, ldc=M + 4)
+        with pytest.raises(tw.TwError):
+            side.gemm(dA.data_ptr() + 2, dC.data_ptr(), M)
+    with pytest.raises(ValueError):
+        tw.Side(full, "f16", W[:, :3])

@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libtwgemm.so")
 PERF_PATH = os.path.join(PKG_DIR, "test_basic_nn")
 
-SOURCES = ["tw_host.cpp", "tw_plan.hip", "tw_gemm.hip", "tw_prune.hip", "tw_cell.hip", "tw_layout.hip"]
+SOURCES = ["tw_host.cpp", "tw_plan.hip", "tw_gemm.hip", "tw_prune.hip", "tw_cell.hip", "tw_layout.hip", "tw_side.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",

@@ -52,6 +52,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
     "tw_gemm_staged", "tw_gemm_staged_workspace",
+    "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm",
 )
 
 
@@ -155,6 +156,10 @@ def lib():
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
+        "tw_side_create": (c_int, [c_int, c_int, c_int, u8p, f32p, pp]),
+        "tw_side_destroy": (None, [vp]),
+        "tw_side_nnz": (c_i64, [vp]),
+        "tw_side_gemm": (c_int, [vp, vp, c_i64, vp, c_i64, c_int, c_f, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -477,6 +482,46 @@ def stream_gemm_nn(M, N, K, dtype, alpha, A_ptr, B_ptr, beta, C_ptr, N_cal, K_ca
                                    bn, _ptr(N_cal, ctypes.c_int32), _ptr(K_cal, ctypes.c_int32),
                                    mn, mk, _ptr(off_B, ctypes.c_int64), _ptr(off_C, ctypes.c_int64),
                                    ctypes.c_void_p(int(stream or 0))))
+
+
+class Side:
+    """The element-wise remainder of a mixed mask (tw_side_*): ``remainder`` is a K x N mask, normally
+    ``mask & ~mask0`` of tiled_wise_1d_mix / tiled_wise_2d_mix (Pruning/VGG/prune_algo.py:151-193),
+    ``B`` the fp32 weight.  ``gemm`` adds ``alpha * A @ (B * remainder)`` to a K-major C after the
+    plan of mask0 has written it."""
+
+    def __init__(self, remainder, dtype, B):
+        m = np.ascontiguousarray(np.asarray(remainder) != 0, dtype=np.uint8)
+        B = np.ascontiguousarray(B, dtype=np.float32)
+        if m.ndim != 2 or B.shape != m.shape:
+            raise ValueError("remainder and B must be K x N matrices of one shape")
+        self.K, self.N, self.dtype = m.shape[0], m.shape[1], dtype
+        h = ctypes.c_void_p()
+        _check(lib().tw_side_create(self.K, self.N, dtype_code(dtype),
+                                    m.ctypes.data_as(ctypes.POINTER(ctypes.c_uint8)),
+                                    B.ctypes.data_as(ctypes.POINTER(ctypes.c_float)), ctypes.byref(h)))
+        self._h = h
+
+    @property
+    def nnz(self):
+        return int(lib().tw_side_nnz(self._h))
+
+    def gemm(self, A_ptr, C_ptr, M, lda=None, ldc=None, alpha=1.0, stream=0):
+        vp = ctypes.c_void_p
+        _check(lib().tw_side_gemm(self._h, vp(int(A_ptr or 0)), M if lda is None else lda,
+                                  vp(int(C_ptr or 0)), M if ldc is None else ldc, M, alpha,
+                                  vp(int(stream or 0))))
+
+    def destroy(self):
+        if self._h:
+            lib().tw_side_destroy(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.destroy()
 
 
 def lstm_gates(M, H, dtype, gates_ptr, ldg, forget_bias, c_prev_ptr, ldc_prev, c_new_ptr, ldc_new,

@@ -2167,21 +2167,23 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     // The A-stationary kernel (K short enough for a panel of A in LDS, C not read).  Measured on a
     // grid of M 128 .. 16384, K 512 .. 2048, N 512 .. 4096, tiles of 64 and 128 columns, 25 and
     // 50 % of the rows kept, against every streaming shape: it wins by 5 - 50 % for tiles of 64
-    // columns at any size, and for tiles of 128 where the streaming kernel would run at most one
-    // 256-row item on every other compute unit (its start-up and epilogue are most of such a
-    // launch); 32-row panels below about a thousand rows of A, 64-row panels above.  Elsewhere
-    // (BERT-base, BERT-large FFN1: several items per unit) it ties or loses up to 10 %.
+    // columns at any size, and by 5 - 15 % for tiles of 128 where the streaming kernel would run
+    // at most three 256-row items on two compute units (its start-up and epilogue are most of
+    // such a launch; BERT-base: 15.8 against 18.2 us); 32-row panels below about a thousand
+    // rows of A, 64-row panels above.  With more items per unit the two tie within 3 %.
     auto as_ok = [&](int shape) {
         return ws_ok && !reads_c && plan->n_blocks > 0 && plan->d_kept_pairs &&
                as_lds_bytes(plan->K, kShapes[shape].bm) <= kLdsBytes;
     };
-    const bool as_few = width <= 64 || items(256, 128) * 2 <= cu;
+    const bool as_few = width <= 64 || items(256, 128) * 2 <= 3 * cu;
     // The skinny kernel where it gives a compute unit at most two workgroups: the launch is then
     // a chain of trips to memory, which it keeps shortest (measured on M 16 .. 512 of the grid
     // above, replayed from a graph: 1.6 - 3 x faster up to one workgroup per unit, 1.1 - 1.5 x
     // up to two).
     const bool skinny_ok = plan->n_units > 0 && (M + 31) / 32 <= 65535; // its grid: units x row blocks
-    const bool skinny = skinny_ok && (int64_t)plan->n_halves * ((M + 31) / 32) <= 2 * (int64_t)cu;
+    // (not beyond 1024 rows: M 2048, N 512 would still be two workgroups per unit, but each then
+    // walks a whole tile's kept rows for 32 rows of A: 10 - 24 us against 6 - 15)
+    const bool skinny = skinny_ok && M <= 1024 && (int64_t)plan->n_halves * ((M + 31) / 32) <= 2 * (int64_t)cu;
     if (skinny) {
         c.shape = TW_SHAPE_SKINNY;
     } else if (!ws_ok) {

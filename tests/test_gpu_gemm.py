@@ -629,6 +629,45 @@ def test_skinny_kernel(tw, oracle, dtype, M):
         tw.set_option(tw.OPT_SHAPE, -1)
 
 
+def test_skinny_kernel_many_units(tw, oracle):
+    """More units than travel in the kernel arguments (40 tiles of 64 and 128 columns): the skinny
+    kernel reads its unit from the plan's table in memory.  Against the oracle, the streaming
+    kernel and itself."""
+    rng = np.random.default_rng(909)
+    M, K = 96, 700
+    widths = [128, 64] * 20
+    N = sum(widths)
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles, c0 = [], 0
+    for t, w in enumerate(widths):
+        kt = int(rng.integers(0, 400))
+        nt = int(rng.integers(1, w + 1))
+        tiles.append(dict(col0=c0, width=w,
+                          kept_k=np.sort(rng.choice(K, size=kt, replace=False)).astype(np.int32),
+                          kept_n=np.sort(rng.choice(w, size=nt, replace=False)).astype(np.int32)))
+        c0 += w
+    keep = kept_columns(tiles, N)
+    ref = reference(oracle, A, B, tiles, "f16")
+    try:
+        with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+            assert plan.info()["n_tiles"] > 32
+            tw.set_option(tw.OPT_SHAPE, tw.SHAPE_SKINNY)
+            print("skinny, many units: launch", flush=True)
+            C1, bits1 = run_gemm(tw, oracle, plan, A, "f16", N, pruned=1)
+            C2, bits2 = run_gemm(tw, oracle, plan, A, "f16", N, pruned=1)
+            tw.set_option(tw.OPT_SHAPE, tw.SHAPE_128x64)
+            tw.set_option(tw.OPT_PIECE, 64)
+            C3, _ = run_gemm(tw, oracle, plan, A, "f16", N, pruned=1)
+            assert np.array_equal(bits1, bits2)
+            assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL["f16"]
+            assert oracle.rel_error(C1, C3) <= 0.5 * TOL["f16"]
+            assert (C1[:, ~keep] == 0).all()
+    finally:
+        tw.set_option(tw.OPT_SHAPE, -1)
+        tw.set_option(tw.OPT_PIECE, -1)
+
+
 def test_operand_beyond_four_gib(tw, oracle):
     """A of 4.4 GiB: byte offsets into A no longer fit 32 bits, the launch falls back to the
     kernel with 64-bit addressing.  Checked on sampled rows (a row of C depends on the same row

@@ -263,7 +263,7 @@ int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 /* tw_gemm_ex for row-major operands at the speed of the K-major kernels.  The reference's Python
  * operator multiplies a row-major x[M,K] into a row-major result (mask_dense,
  * Pruning/BERT/utils/modeling.py:992-1007).  tw_gemm_ex takes such operands as they are when both
- * are row-major, K <= 2272 and beta == 0 (a kernel that keeps a panel of A in LDS), and else
+ * are row-major, K <= 2128 and beta == 0 (a kernel that keeps a panel of A in LDS), and else
  * through a layout-generic kernel that gathers 2-byte elements.  Here, in those other cases, a row-major A is first turned into
  * its K-major copy and a row-major C is produced K-major and turned back, both in `workspace`
  * (device memory, 16-byte aligned, at least tw_gemm_staged_workspace(plan, M, a_layout, c_layout)
@@ -305,8 +305,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU */
 #define TW_SHAPE_128x32 5  /* wave-specialised, 128 x 32: skinny M */
 #define TW_SHAPE_256x64 6  /* wave-specialised, 256 x 64 */
-#define TW_SHAPE_AS64 7    /* A-stationary, 64 rows of all K in LDS: K up to 1136, beta == 0 */
-#define TW_SHAPE_AS32 8    /* A-stationary, 32 rows: K up to 2272, beta == 0 */
+#define TW_SHAPE_AS64 7    /* A-stationary, 64 rows of all K in LDS: K up to 1064, beta == 0 */
+#define TW_SHAPE_AS32 8    /* A-stationary, 32 rows: K up to 2128, beta == 0 */
 #define TW_SHAPE_SKINNY 9  /* 64 rows x 32 columns per workgroup, the kept rows split over its waves: few rows of A */
 #define TW_N_SHAPES 10
 int tw_set_option(int option, int value);

@@ -1256,38 +1256,52 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
 //          in rows with bit 1 set, so that the four rows a transposed read touches (consecutive
 //          kept rows are mostly a few rows apart) tend to fall into different bank groups
 //   work:  block b of the plan (unit, 32-column block) belongs to group b % n_groups; workgroup
-//          (row block, group); wave w takes every eighth block of the group
-//   loads: a block is cut into segments of kAsSegSteps steps (16 groups of 16 k rows: per lane
-//          a 16-byte weight fragment and a word with its two row numbers each).  A wave computes one segment out
-//          of one register set while the loads of the next segment - of this block or the next -
-//          fill the other.  Every segment issues the loads of all its 16 groups (steps past the
-//          block's end fetch its last step again), so the number of loads in flight behind a
-//          segment is the same on every path and the wait for it is an exact count.
+//          (row block, group); wave w takes every twelfth block of the group
+//   loads: a block is cut into segments of two steps (8 groups of 16 k rows: per lane a 16-byte
+//          weight fragment and a word with its two row numbers each).  A wave computes one
+//          segment out of one register set while the loads of the next segment - of this block
+//          or the next - fill the other.  Every segment issues the loads of all its 8 groups
+//          (steps past the block's end fetch its last step again), so the number of loads in
+//          flight behind a segment is the same on every path and the wait for it is an exact
+//          count.
 // Takes beta == 0 only (C is not read).  RM false: K-major A and C (32-bit row offsets into A).
 // RM true: row-major A[M][lda] and C[M][ldc], the operands of the reference's Python operator
 // (mask_dense, Pruning/BERT/utils/modeling.py:992-1007): the panel is transposed on its way into
 // LDS (a lane reads 16 bytes along k of its own row m and writes them as eight 2-byte pieces
 // into eight panel rows; consecutive lanes are consecutive m, so those writes are contiguous),
 // and the product goes out as 2-byte stores, a wave covering two rows of the block's 32 columns.
-constexpr int kAsWaves = 8, kAsSegSteps = 4;
+// Waves of a workgroup, steps of a segment, and waves that share a block of a 64-row panel (each
+// then multiplies one 32-row half of it).  A wave's life is a chain of short dependent phases
+// (loads, LDS reads, MFMAs, stage, stores), so more waves fill each other's gaps: twelve waves
+// with two-step segments (157 registers of the 170 a wave may then have) run BERT-base in 14.2
+// us, eight waves with four-step segments in 15.7; sixteen waves leave 128 registers, which
+// only a 32-row product with one-step segments fits, and two such waves sharing a block of a
+// 64-row panel load its weight fragments twice: 16.7 us.
+constexpr int as_waves(int bms, bool rm) { return 12; }
+constexpr int as_seg_steps(int bms, bool rm) { return 2; }
+constexpr int as_split(int bms, bool rm) { return 1; }
+constexpr int as_task_waves(int bms, bool rm) { return as_waves(bms, rm) / as_split(bms, rm); }
 
 template <int DT, int BMS, bool RM>
-__global__ void __launch_bounds__(64 * kAsWaves, 1)
+__global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     tw_gemm_as_kernel(const GemmArgs p, const int32_t *__restrict__ blocks, int n_blocks, int n_groups,
                       int n_mblk, int k_rows)
 {
+    constexpr int kAsWaves = as_waves(BMS, RM), SPLIT = as_split(BMS, RM), TWV = kAsWaves / SPLIT;
     constexpr int NT = 64 * kAsWaves;
     constexpr int ROWB = BMS * 2; // bytes of a panel row
     constexpr int CH = BMS / 8;   // 16-byte chunks of a panel row
-    constexpr int MI = BMS / 32;
+    constexpr int MI = BMS / 32 / SPLIT; // 32-row MFMA blocks of a wave
     constexpr int CP = 32 + 4;    // pitch of a wave's C stage: [32 columns][CP] elements, 32 rows at a time
-    constexpr int DS = kAsSegSteps, GS = DS * 4;
+    constexpr int DS = as_seg_steps(BMS, RM), GS = DS * 4;
     using E = Elem<DT>;
     extern __shared__ __align__(16) unsigned char as_smem[];
     unsigned char *const panel = as_smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int task = wave / SPLIT;           // which of the workgroup's block sequences
+    const int mi0 = (wave % SPLIT) * MI;     // first 32-row block of the panel this wave multiplies
     const int mblk = blockIdx.x % n_mblk, group = blockIdx.x / n_mblk;
     const int m0 = mblk * BMS;
     const int m_end = m0 + BMS < p.M ? m0 + BMS : p.M;
@@ -1337,7 +1351,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
         const int total = k_rows * CH;
         const uint32_t lda_b = (uint32_t)p.lda * 2u;
         const char *const a0 = reinterpret_cast<const char *>(A + m0);
-        constexpr int PL = 16;
+        constexpr int PL = 128 / kAsWaves; // loads in flight per thread: 128 per SIMD lane of the unit
         for (int base = tid; base < total; base += NT * PL) {
             u32x4 v[PL];
 #pragma unroll
@@ -1373,7 +1387,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
         int code_after; // list entry of the wave's block after this one, fetched a block ahead
         UnitDev u;
     };
-    const int b_stride = n_groups * kAsWaves;
+    const int b_stride = n_groups * TWV;
     auto open_block = [&](int b, int code) {
         Cursor c;
         c.b = b;
@@ -1449,8 +1463,8 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
                     const uint32_t o_hi = r_hi * ROWB + (BMS == 64 ? (r_hi & 2u) << 5 : 0u);
 #pragma unroll
                     for (int mi = 0; mi < MI; ++mi) {
-                        TW_LDS(unsigned char) qlo = lds_lane + (o_lo ^ (uint32_t)(mi * 64));
-                        TW_LDS(unsigned char) qhi = lds_lane + (o_hi ^ (uint32_t)(mi * 64));
+                        TW_LDS(unsigned char) qlo = lds_lane + (o_lo ^ (uint32_t)((mi0 + mi) * 64));
+                        TW_LDS(unsigned char) qhi = lds_lane + (o_hi ^ (uint32_t)((mi0 + mi) * 64));
                         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))qlo);
                         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))qhi);
                         const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
@@ -1469,7 +1483,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
         if (RM) {
             // rows m_lane + 8 * g + e, g = 0 .. 4 MI - 1, e = 0 .. 3: a running pointer, so that
             // the 16 MI addresses are not all worked out (and kept in registers) ahead
-            const int m_lane = m0 + (lane >> 5) * 4;
+            const int m_lane = m0 + mi0 * 32 + (lane >> 5) * 4;
             uint16_t *cp = C + (int64_t)m_lane * p.ldc + out_col;
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi) {
@@ -1523,7 +1537,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
                 const int col = __shfl(out_col, jj);
                 const u32x2 lo = *reinterpret_cast<const u32x2 *>(cst + jj * CP + ch * 8);
                 const u32x2 hi = *reinterpret_cast<const u32x2 *>(cst + jj * CP + ch * 8 + 4);
-                const int m = m0 + mi * 32 + ch * 8;
+                const int m = m0 + (mi0 + mi) * 32 + ch * 8;
                 if (jj < cnt)
                     store_chunk(C + (int64_t)col * p.ldc + m, u32x4{lo.x, lo.y, hi.x, hi.y}, m, m_end,
                                 p.store_through != 0);
@@ -1535,7 +1549,7 @@ __global__ void __launch_bounds__(64 * kAsWaves, 1)
 
     clear();
     Seg g0, g1;
-    const int b_first = group + n_groups * wave;
+    const int b_first = group + n_groups * task;
     Cursor cur = open_block(b_first, b_first < n_blocks ? __builtin_amdgcn_readfirstlane(blocks[b_first]) : 0);
     if (valid(cur))
         issue(cur, g0); // weight and row numbers do not wait for the panel
@@ -2040,7 +2054,7 @@ static const Shape kShapes[TW_N_SHAPES] = {
 
 // LDS of the A-stationary kernel: the panel (all K rows, BMS rows m) and a C stage per wave
 constexpr int kLdsBytes = 160 * 1024;
-static int64_t as_lds_bytes(int K, int bms) { return (int64_t)K * bms * 2 + kAsWaves * 32 * 36 * 2; }
+static int64_t as_lds_bytes(int K, int bms) { return (int64_t)K * bms * 2 + as_waves(bms, false) * 32 * 36 * 2; }
 static bool is_as_shape(int shape) { return shape == TW_SHAPE_AS64 || shape == TW_SHAPE_AS32; }
 // shapes that walk the plan's units themselves: no work queue, no unit pieces
 static bool is_queueless_shape(int shape) { return is_as_shape(shape) || shape == TW_SHAPE_SKINNY; }
@@ -2166,16 +2180,14 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     c.piece = 128;
     // The A-stationary kernel (K short enough for a panel of A in LDS, C not read).  Measured on a
     // grid of M 128 .. 16384, K 512 .. 2048, N 512 .. 4096, tiles of 64 and 128 columns, 25 and
-    // 50 % of the rows kept, against every streaming shape: it wins by 5 - 50 % for tiles of 64
-    // columns at any size, and by 5 - 15 % for tiles of 128 where the streaming kernel would run
-    // at most three 256-row items on two compute units (its start-up and epilogue are most of
-    // such a launch; BERT-base: 15.8 against 18.2 us); 32-row panels below about a thousand
-    // rows of A, 64-row panels above.  With more items per unit the two tie within 3 %.
+    // 50 % of the rows kept, against every streaming shape: wherever a 64-row panel fits it is
+    // the fastest shape or within 8 % of it (tiles of 64 columns: by 5 - 50 %; BERT-base 14.2
+    // against 18.2 us, BERT-large FFN1 at 50 / 75 / 90 %: 52 / 33 / 24 against 55 / 38 / 30);
+    // 32-row panels below about a thousand rows of A, 64-row panels above.
     auto as_ok = [&](int shape) {
         return ws_ok && !reads_c && plan->n_blocks > 0 && plan->d_kept_pairs &&
                as_lds_bytes(plan->K, kShapes[shape].bm) <= kLdsBytes;
     };
-    const bool as_few = width <= 64 || items(256, 128) * 2 <= 3 * cu;
     // The skinny kernel where it gives a compute unit at most two workgroups: the launch is then
     // a chain of trips to memory, which it keeps shortest (measured on M 16 .. 512 of the grid
     // above, replayed from a graph: 1.6 - 3 x faster up to one workgroup per unit, 1.1 - 1.5 x
@@ -2188,13 +2200,14 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
         c.shape = TW_SHAPE_SKINNY;
     } else if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
-    } else if (as_ok(TW_SHAPE_AS64) && as_few && (M > 128 || plan->n_blocks >= 96)) {
+    } else if (as_ok(TW_SHAPE_AS64) && (M > 128 || plan->n_blocks >= 96)) {
         // 64-row panels where they still give three quarters of the compute units a workgroup
         const int mblk64 = (M + 63) / 64;
-        const int groups64 = std::min(std::max(1, cu / mblk64), (plan->n_blocks + kAsWaves - 1) / kAsWaves);
+        constexpr int tw64 = as_task_waves(64, false);
+        const int groups64 = std::min(std::max(1, cu / mblk64), (plan->n_blocks + tw64 - 1) / tw64);
         c.shape = (int64_t)mblk64 * groups64 * 4 >= (int64_t)cu * 3 ? TW_SHAPE_AS64 : TW_SHAPE_AS32;
     } else if (!as_ok(TW_SHAPE_AS64) && as_ok(TW_SHAPE_AS32) && M > 128 &&
-               (M <= 512 || (M <= 1024 && plan->n_blocks <= kAsWaves * std::max(1, cu / ((M + 31) / 32))))) {
+               (M <= 512 || (M <= 1024 && plan->n_blocks <= as_task_waves(32, false) * std::max(1, cu / ((M + 31) / 32))))) {
         // (up to 1024 rows where every wave still has at most one block: M 1024, K 2048, N 2048:
         // 12.3 - 15.8 us against 14.4 - 20.2)
         c.shape = TW_SHAPE_AS32;
@@ -2270,14 +2283,14 @@ template <int DT, int BMS, bool RM> static int launch_as(const tw_plan *plan, co
         return fail(TW_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(attr_err));
     const int n_mblk = (M + BMS - 1) / BMS;
     // as many groups as keep every compute unit at one workgroup, each wave with a block or more
-    const int per_wg = kAsWaves;
+    const int per_wg = as_task_waves(BMS, RM);
     int n_groups = std::max(1, plan->cu_count / n_mblk);
     n_groups = std::min(n_groups, std::max(1, (plan->n_blocks + per_wg - 1) / per_wg));
     if ((int64_t)n_mblk * n_groups > (int64_t)0x7fffffff)
         return fail(TW_ERR_SHAPE, "%lld workgroups (M=%d): a launch takes at most %lld",
                     (long long)n_mblk * n_groups, M, (long long)(int64_t)0x7fffffff);
     hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS, RM>), dim3((unsigned)(n_mblk * n_groups)),
-                       dim3(64 * kAsWaves), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
+                       dim3(64 * as_waves(BMS, RM)), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
                        n_mblk, plan->K);
     TW_HIP(hipGetLastError());
     return TW_OK;
@@ -2493,7 +2506,7 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
             a.arg_units[i] = plan->h_units[i];
         const int mblk64 = (M + 63) / 64;
         const int groups64 =
-            std::min(std::max(1, plan->cu_count / mblk64), (plan->n_blocks + kAsWaves - 1) / kAsWaves);
+            std::min(std::max(1, plan->cu_count / mblk64), (plan->n_blocks + as_task_waves(64, true) - 1) / as_task_waves(64, true));
         const bool b64 = as_lds_bytes(plan->K, 64) <= kLdsBytes &&
                          (int64_t)mblk64 * groups64 * 4 >= (int64_t)plan->cu_count * 3;
         hipStream_t s = (hipStream_t)stream;

@@ -2200,7 +2200,10 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
         c.shape = TW_SHAPE_SKINNY;
     } else if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
-    } else if (as_ok(TW_SHAPE_AS64) && (M > 128 || plan->n_blocks >= 96)) {
+    } else if (as_ok(TW_SHAPE_AS64) && (M > 128 || plan->n_blocks >= 96) &&
+               (!plan->rows_shared || width <= 64 || items(256, 128) * 2 <= 3 * cu)) {
+        // (a 0 %-sparse plan with many 256-row items is better off streaming with one queue per
+        // die: M 12800, K 768, N 3072: 87 against 96 us)
         // 64-row panels where they still give three quarters of the compute units a workgroup
         const int mblk64 = (M + 63) / 64;
         constexpr int tw64 = as_task_waves(64, false);

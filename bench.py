@@ -33,6 +33,8 @@ MEASURED_TRAFFIC_BYTES = {
     "bert_base_ffn_in": (2 * 7897 + 24576) * 1024,
     "nmt_lstm_gates": (2 * 3558.5 + 1024) * 1024,
     "imbalance_stress": (2 * 908806 + 212608) * 1024,
+    "bert_large_ffn1_keep25": (2 * 16649 + 65536) * 1024,
+    "bert_large_ffn2_keep25": (2 * 38143 + 16400) * 1024,
 }
 
 

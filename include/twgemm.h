@@ -243,6 +243,13 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
                int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
                const tw_epilogue *ep, void *stream);
 
+/* Re-arms the work-queue counters of a plan (all 256 slots to zero) with a small kernel on
+ * `stream`.  A launch leaves its slot at zero when it ends; one that was aborted mid-flight (a
+ * device fault elsewhere in the process, a reset) does not, and the next launch to draw that slot
+ * would skip work.  Call it with no launch of the plan in flight.  No counterpart in the
+ * reference, whose per-tile launches share no state (basic_nn.cu:408-430). */
+int tw_plan_reset(tw_plan *plan, void *stream);
+
 /* tw_gemm_ex for callers that cannot allocate device memory: code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc.
  * It has no counterpart in the reference (Stream_Gemm_NN creates and destroys 32 streams per call,

@@ -324,6 +324,33 @@ def test_repeated_launches_and_slot_reuse(tw, oracle):
         assert np.array_equal(from_device_bits(dC)[keep], first[keep, :M])
 
 
+def test_plan_reset_leaves_results_unchanged(tw, oracle):
+    """tw_plan_reset between launches (the call that re-arms every ticket slot after an aborted
+    launch): the launches after it give the bits of the launches before it."""
+    import torch
+    rng = np.random.default_rng(28)
+    M, K, N, G, dtype = 300, 192, 640, 128, "f16"
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.5, n_keep=0.9)
+    stream = torch.cuda.current_stream().cuda_stream
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        _, first = run_gemm(tw, oracle, plan, A, dtype, N)
+        ld = (M + 7) // 8 * 8
+        At = np.zeros((K, ld), np.uint16)
+        At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+        dA = to_device_bits(At, (K, ld))
+        keep = kept_columns(tiles, N)
+        for _ in range(3):
+            plan.reset(stream)
+            dC = torch.zeros((N, ld), dtype=torch.int16, device="cuda")
+            for _ in range(5):
+                plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=ld, ldc=ld, stream=stream)
+            torch.cuda.synchronize()
+            assert np.array_equal(from_device_bits(dC)[keep, :M], first[keep, :M])
+    assert tw.lib().tw_plan_reset(None, None) == tw.ERR_NULL
+
+
 def test_queue_is_rearmed_between_launches_of_different_sizes(tw, oracle):
     """Launches with few items (one per workgroup), with several rounds of items per workgroup,
     and with items that have no step or only fill zeros alternate on one plan, through every

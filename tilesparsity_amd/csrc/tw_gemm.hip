@@ -2466,6 +2466,13 @@ __global__ void clear_counters_kernel(int32_t *counters)
         counters[threadIdx.x] = 0;
 }
 
+__global__ void clear_all_slots_kernel(int32_t *tickets)
+{
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < kTicketSlots * kTicketInts)
+        tickets[i] = 0;
+}
+
 // Device address of `scratch` on the current device, looked up once per device (the array's name
 // is only a host-side stand-in; every GPU holds its own copy at its own address).
 int static_scratch(int32_t **out)
@@ -2585,6 +2592,23 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
 {
     return gemm_impl(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep, stream,
                      false);
+}
+
+int tw_plan_reset(tw_plan *plan, void *stream)
+{
+    if (!plan)
+        return fail(TW_ERR_NULL, "plan is NULL");
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev != plan->device)
+        return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d", plan->device, dev);
+    if (!plan->d_tickets)
+        return TW_OK;
+    // a kernel, not a memset: the call may be recorded into a graph
+    hipLaunchKernelGGL(clear_all_slots_kernel, dim3((kTicketSlots * kTicketInts + 255) / 256), dim3(256), 0,
+                       (hipStream_t)stream, plan->d_tickets);
+    TW_HIP(hipGetLastError());
+    return TW_OK;
 }
 
 int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,

@@ -52,7 +52,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
     "tw_gemm_staged", "tw_gemm_staged_workspace",
-    "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm",
+    "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm", "tw_plan_reset",
 )
 
 
@@ -156,6 +156,7 @@ def lib():
         "tw_plan_from_export": (c_int, [c_int, c_int, c_int, c_int, i32p, c_int, i32p, f32p, pp]),
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
+        "tw_plan_reset": (c_int, [vp, vp]),
         "tw_side_create": (c_int, [c_int, c_int, c_int, u8p, f32p, pp]),
         "tw_side_destroy": (None, [vp]),
         "tw_side_nnz": (c_i64, [vp]),
@@ -383,6 +384,10 @@ class Plan:
         return cls(h.value, K, N, dtype_code(dtype))
 
     # -- inspection
+    def reset(self, stream=0):
+        """Re-arms the plan's work-queue counters (after a launch of it was aborted mid-flight)."""
+        _check(lib().tw_plan_reset(self._h, ctypes.c_void_p(int(stream or 0))))
+
     def info(self):
         v = np.zeros(12, np.int64)
         _check(lib().tw_plan_info(self._h, _ptr(v, ctypes.c_int64), 12))

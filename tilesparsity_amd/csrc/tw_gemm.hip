@@ -1285,7 +1285,7 @@ constexpr int as_task_waves(int bms, bool rm) { return as_waves(bms, rm) / as_sp
 template <int DT, int BMS, bool RM>
 __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     tw_gemm_as_kernel(const GemmArgs p, const int32_t *__restrict__ blocks, int n_blocks, int n_groups,
-                      int n_mblk, int k_rows)
+                      int n_mblk, int k_rows, int blocks_per_unit)
 {
     constexpr int kAsWaves = as_waves(BMS, RM), SPLIT = as_split(BMS, RM), TWV = kAsWaves / SPLIT;
     constexpr int NT = 64 * kAsWaves;
@@ -1347,29 +1347,28 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
             }
         }
     };
-    auto load_panel = [&]() {
-        const int total = k_rows * CH;
+    constexpr int PL = 128 / kAsWaves; // loads in flight per thread: 128 per SIMD lane of the unit
+    const int panel_chunks = k_rows * CH;
+    auto panel_fetch = [&](int base, u32x4 (&v)[PL]) {
         const uint32_t lda_b = (uint32_t)p.lda * 2u;
         const char *const a0 = reinterpret_cast<const char *>(A + m0);
-        constexpr int PL = 128 / kAsWaves; // loads in flight per thread: 128 per SIMD lane of the unit
-        for (int base = tid; base < total; base += NT * PL) {
-            u32x4 v[PL];
 #pragma unroll
-            for (int q = 0; q < PL; ++q) {
-                const int idx = base + q * NT;
-                const int row = idx / CH, ch = idx % CH;
-                v[q] = u32x4{0u, 0u, 0u, 0u};
-                if (idx < total && m0 + ch * 8 < p.M)
-                    v[q] = *reinterpret_cast<const u32x4 *>(a0 + (uint32_t)row * lda_b + ch * 16);
-            }
+        for (int q = 0; q < PL; ++q) {
+            const int idx = base + q * NT;
+            const int row = idx / CH, ch = idx % CH;
+            v[q] = u32x4{0u, 0u, 0u, 0u};
+            if (idx < panel_chunks && m0 + ch * 8 < p.M)
+                v[q] = *reinterpret_cast<const u32x4 *>(a0 + (uint32_t)row * lda_b + ch * 16);
+        }
+    };
+    auto panel_put = [&](int base, const u32x4 (&v)[PL]) {
 #pragma unroll
-            for (int q = 0; q < PL; ++q) {
-                const int idx = base + q * NT;
-                const int row = idx / CH, ch = idx % CH;
-                const int chs = BMS == 64 ? ch ^ (((row >> 1) & 1) << 2) : ch;
-                if (idx < total)
-                    *reinterpret_cast<u32x4 *>(panel + row * ROWB + chs * 16) = v[q];
-            }
+        for (int q = 0; q < PL; ++q) {
+            const int idx = base + q * NT;
+            const int row = idx / CH, ch = idx % CH;
+            const int chs = BMS == 64 ? ch ^ (((row >> 1) & 1) << 2) : ch;
+            if (idx < panel_chunks)
+                *reinterpret_cast<u32x4 *>(panel + row * ROWB + chs * 16) = v[q];
         }
     };
 
@@ -1388,6 +1387,16 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
         UnitDev u;
     };
     const int b_stride = n_groups * TWV;
+    // entry b of the plan's list of blocks, unit * 4 + block of the unit: worked out where every
+    // unit has the same number of blocks (no trip to memory before the first loads), else the
+    // value fetched a block ahead
+    auto block_code = [&](int b, int fetched) {
+        if (blocks_per_unit) {
+            const int ui = b / blocks_per_unit;
+            return ui * 4 + (b - ui * blocks_per_unit);
+        }
+        return __builtin_amdgcn_readfirstlane(fetched);
+    };
     auto open_block = [&](int b, int code) {
         Cursor c;
         c.b = b;
@@ -1396,7 +1405,8 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
         c.nb = 0;
         c.code_after = 0;
         if (b < n_blocks) {
-            c.code_after = blocks[b + b_stride < n_blocks ? b + b_stride : b];
+            if (!blocks_per_unit)
+                c.code_after = blocks[b + b_stride < n_blocks ? b + b_stride : b];
             c.u = load_unit(p, code >> 2);
             c.nb = code & 3;
             c.nsteps = c.u.k_pad / kBlockK;
@@ -1411,7 +1421,7 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
             n.seg = c.seg + 1;
             return n;
         }
-        return open_block(c.b + b_stride, __builtin_amdgcn_readfirstlane(c.code_after));
+        return open_block(c.b + b_stride, block_code(c.b + b_stride, c.code_after));
     };
     struct Seg {
         u32x4 bq[GS];
@@ -1550,13 +1560,29 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     clear();
     Seg g0, g1;
     const int b_first = group + n_groups * task;
-    Cursor cur = open_block(b_first, b_first < n_blocks ? __builtin_amdgcn_readfirstlane(blocks[b_first]) : 0);
-    if (valid(cur))
-        issue(cur, g0); // weight and row numbers do not wait for the panel
-    if (RM)
+    Cursor cur_first;
+    if (RM) {
+        Cursor first = open_block(b_first, b_first < n_blocks ? block_code(b_first, blocks_per_unit ? 0 : blocks[b_first]) : 0);
+        if (valid(first))
+            issue(first, g0); // weight and row numbers do not wait for the panel
         load_panel_row_major();
-    else
-        load_panel();
+        cur_first = first;
+    } else {
+        // the panel's first loads leave before anything else is known: the unit of the wave's
+        // first block and that block's loads follow them while they are on their way
+        u32x4 pv[PL];
+        panel_fetch(tid, pv);
+        Cursor first = open_block(b_first, b_first < n_blocks ? block_code(b_first, blocks_per_unit ? 0 : blocks[b_first]) : 0);
+        if (valid(first))
+            issue(first, g0);
+        panel_put(tid, pv);
+        for (int base = tid + NT * PL; base < panel_chunks; base += NT * PL) {
+            panel_fetch(base, pv);
+            panel_put(base, pv);
+        }
+        cur_first = first;
+    }
+    Cursor cur = cur_first;
     __syncthreads();
     if (valid(cur)) {
         for (;;) {
@@ -1716,12 +1742,9 @@ __global__ void __launch_bounds__(64 * kSkWaves, 1) tw_gemm_skinny_kernel(const 
             }
             return n;
         };
+        // (the weight fragments first: they do not wait for the row numbers, so on a wave's
+        // first pair they travel while the numbers are still on their way)
         auto issue = [&](int s, const Numbers &n, Loads &l) {
-#pragma unroll
-            for (int t = 0; t < 2; ++t)
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    l.a[t][i] = *(TW_GLOBAL(const u32x4))(a_lane + (int64_t)n.row[t][i] * lda);
 #pragma unroll
             for (int t = 0; t < 2; ++t) {
                 const int st = s + t * kSkWaves < nsteps ? s + t * kSkWaves : s;
@@ -1732,6 +1755,11 @@ __global__ void __launch_bounds__(64 * kSkWaves, 1) tw_gemm_skinny_kernel(const 
                         l.b[t][cb][k16] =
                             *(TW_GLOBAL(const u32x4))(bsrc + st * step_b + cb * cb_off + k16 * 1024);
             }
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    l.a[t][i] = *(TW_GLOBAL(const u32x4))(a_lane + (int64_t)n.row[t][i] * lda);
         };
         f32x16 acc[2];
 #pragma unroll
@@ -2294,7 +2322,7 @@ template <int DT, int BMS, bool RM> static int launch_as(const tw_plan *plan, co
                     (long long)n_mblk * n_groups, M, (long long)(int64_t)0x7fffffff);
     hipLaunchKernelGGL((tw_gemm_as_kernel<DT, BMS, RM>), dim3((unsigned)(n_mblk * n_groups)),
                        dim3(64 * as_waves(BMS, RM)), (size_t)as_lds_bytes(plan->K, BMS), s, a, plan->d_blocks, plan->n_blocks, n_groups,
-                       n_mblk, plan->K);
+                       n_mblk, plan->K, plan->blocks_per_unit);
     TW_HIP(hipGetLastError());
     return TW_OK;
 }

@@ -670,6 +670,10 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
         for (int nb = 0; nb < units[ui].nb_cnt; ++nb)
             blocks.push_back((int32_t)ui * 4 + nb);
     p->n_blocks = (int)blocks.size();
+    p->blocks_per_unit = units.empty() ? 0 : units[0].nb_cnt;
+    for (const UnitDev &u : units)
+        if (u.nb_cnt != p->blocks_per_unit)
+            p->blocks_per_unit = 0;
     const size_t o_blocks = put(blocks.data(), blocks.size() * sizeof(int32_t));
     std::vector<uint32_t> kpairs; // see GemmArgs::kept_pairs
     if (p->K <= 0xFFFF) {

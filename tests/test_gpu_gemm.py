@@ -124,6 +124,73 @@ def test_gemm_alpha_beta_and_zero_mode(tw, oracle, dtype):
         assert oracle.rel_error(C, full) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_row_major_columns_in_groups_of_four(tw, oracle, dtype):
+    """Row-major A and C on a plan whose kept columns are neighbours in C (no column pruned: the
+    A-stationary kernel then stores 16-byte pieces of rows) or come in groups of four (element-wise
+    stores in the blocks that hold an odd group).  Bit for bit the K-major result with bias and
+    ReLU, within tolerance with GELU; ragged M, padding and pruned columns untouched, a C that
+    starts 16 bytes into its buffer, a bias that is not 16-byte aligned."""
+    import torch
+    rng = np.random.default_rng(77)
+    M, K, N, G = 203, 320, 512, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tiles = []
+    for t in range(N // G):
+        quads = np.arange(G // 4) if t % 2 == 0 else np.sort(rng.choice(G // 4, 19, replace=False))
+        kept_n = (quads[:, None] * 4 + np.arange(4)).reshape(-1).astype(np.int32)
+        kept_k = np.sort(rng.choice(K, K * 2 // 5, replace=False)).astype(np.int32)
+        tiles.append(dict(col0=t * G, width=G, kept_k=kept_k, kept_n=kept_n))
+    keep = kept_columns(tiles, N)
+    Ab = oracle.cast_bits(A, dtype).reshape(M, K)
+    d_bias = torch.from_numpy(bias).cuda()
+    d_bias1 = torch.from_numpy(np.concatenate([[0.0], bias]).astype(np.float32)).cuda()
+    ld8 = round_up(M, 8)
+    Ak = np.zeros((K, ld8), np.uint16)
+    Ak[:, :M] = Ab.T
+    lda = K + 8
+    Ar = np.zeros((M, lda), np.uint16)
+    Ar[:, :K] = Ab
+    pre = 0.75 * reference(oracle, A, B, tiles, dtype) + bias
+    refs = {tw.ACT_RELU: np.maximum(pre, 0.0),
+            tw.ACT_GELU: 0.5 * pre * (1.0 + np.tanh(np.sqrt(2.0 / np.pi) * (pre + 0.044715 * pre ** 3)))}
+    with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+        dAk, dAr = to_device_bits(Ak, Ak.shape), to_device_bits(Ar, Ar.shape)
+        for act, ref in refs.items():
+            dCk = to_device_bits(np.full((N, ld8), SENTINEL, np.uint16), (N, ld8))
+            tw.set_option(tw.OPT_SHAPE, tw.SHAPE_AS32)   # (the default for so few rows sums k in four slices)
+            try:
+                plan.gemm(dAk.data_ptr(), dCk.data_ptr(), M, lda=ld8, ldc=ld8, alpha=0.75,
+                          bias_ptr=d_bias.data_ptr(), activation=act)
+            finally:
+                tw.set_option(tw.OPT_SHAPE, -1)
+            torch.cuda.synchronize()
+            want = from_device_bits(dCk)[:, :M].T
+            want_f = oracle.bits_to_f32(np.ascontiguousarray(want), dtype).reshape(M, N)
+            assert oracle.rel_error(want_f[:, keep], ref[:, keep]) <= TOL[dtype]
+            # 8-byte stores; a bias that is not 16-byte aligned: element-wise stores
+            for ldc, shift, bias_shift in ((N + 8, 0, 0), (N + 16, 8, 0), (N + 8, 0, 1)):
+                full = torch.full((M * ldc + 16,), SENTINEL, dtype=torch.int16, device="cuda")
+                plan.gemm(dAr.data_ptr(), full.data_ptr() + 2 * shift, M, lda=lda, ldc=ldc, alpha=0.75,
+                          a_layout=tw.ROWMAJOR, c_layout=tw.ROWMAJOR,
+                          bias_ptr=(d_bias1.data_ptr() + 4) if bias_shift else d_bias.data_ptr(),
+                          activation=act)
+                torch.cuda.synchronize()
+                flat = full.cpu().numpy().view(np.uint16)
+                assert np.all(flat[:shift] == SENTINEL) and np.all(flat[shift + M * ldc:] == SENTINEL)
+                got = flat[shift:shift + M * ldc].reshape(M, ldc)
+                assert np.all(got[:, N:] == SENTINEL)
+                assert np.all(got[:, :N][:, ~keep] == SENTINEL)
+                if act == tw.ACT_RELU:      # the same arithmetic in every kernel: the same bits
+                    assert np.array_equal(got[:, :N][:, keep], want[:, keep])
+                else:
+                    got_f = oracle.bits_to_f32(np.ascontiguousarray(got[:, :N]), dtype).reshape(M, N)
+                    assert oracle.rel_error(got_f[:, keep], ref[:, keep]) <= TOL[dtype]
+                    assert oracle.rel_error(got_f[:, keep], want_f[:, keep]) <= 0.5 * TOL[dtype]
+
+
 @pytest.mark.parametrize("staged", [False, True])
 @pytest.mark.parametrize("a_layout,c_layout", [(1, 1), (1, 0), (0, 1)])
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

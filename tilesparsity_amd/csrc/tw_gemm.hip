@@ -1267,9 +1267,10 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
 // Takes beta == 0 only (C is not read).  RM false: K-major A and C (32-bit row offsets into A).
 // RM true: row-major A[M][lda] and C[M][ldc], the operands of the reference's Python operator
 // (mask_dense, Pruning/BERT/utils/modeling.py:992-1007): the panel is transposed on its way into
-// LDS (a lane reads 16 bytes along k of its own row m and writes them as eight 2-byte pieces
-// into eight panel rows; consecutive lanes are consecutive m, so those writes are contiguous),
-// and the product goes out as 2-byte stores, a wave covering two rows of the block's 32 columns.
+// LDS (pieces of 16 rows m x 64 k, read along k and turned with the transposed LDS read), and
+// the product goes out as 16-byte pieces of rows of C where a block's kept columns are
+// neighbours in C in aligned groups of eight, else as 2-byte stores, a wave covering two rows
+// of the block's 32 columns.
 // Waves of a workgroup, steps of a segment, and waves that share a block of a 64-row panel (each
 // then multiplies one 32-row half of it).  A wave's life is a chain of short dependent phases
 // (loads, LDS reads, MFMAs, stage, stores), so more waves fill each other's gaps: twelve waves
@@ -1310,39 +1311,59 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     const unsigned char *const Bp = reinterpret_cast<const unsigned char *>(p.Bp);
     uint16_t *const cst = reinterpret_cast<uint16_t *>(as_smem + (size_t)k_rows * ROWB) + wave * 32 * CP;
 
+    const int L = lane & 15;
     // ---- the panel: 16-byte chunks, sixteen loads in flight per thread (the first segment's
     // loads of this wave are already on their way, see below)
+    // Row-major A: a wave takes pieces of 16 rows m x 64 columns k.  It reads a piece with
+    // 16-byte loads along k (eight lanes a row: whole 128-byte lines), puts it into its own stage
+    // as it came, [m][k], and takes it out again with transposed reads: by the symmetry of that
+    // instruction a lane then holds eight neighbouring m of one k, one 16-byte piece of a panel row.
     auto load_panel_row_major = [&]() {
-        // lane -> row m (BMS = 32: the upper half of the wave takes the next chunk of k)
-        constexpr int LPM = 64 / BMS;                       // k chunks a wave reads per load
-        const int m = lane % BMS;
+        constexpr int MB = BMS / 16;  // pieces across the rows of the panel
+        constexpr int TP = 144;       // bytes of a row of the piece in the stage (16 rows: the whole stage)
+        static_assert(16 * TP <= 32 * CP * 2, "a piece has to fit the wave's stage");
         const int kchunks = (k_rows + 7) / 8;
-        const bool m_ok = m0 + m < p.M;
-        const uint16_t *const arow = A + (int64_t)(m0 + m) * p.lda;
-        unsigned char *const dst = panel + (m & 31) * 2;
-        constexpr int PL = 4;
-        for (int base = wave * LPM + lane / BMS; base < kchunks; base += kAsWaves * LPM * PL) {
-            u32x4 v[PL];
+        const int n_pieces = MB * ((k_rows + 63) / 64);
+        unsigned char *const tmp = reinterpret_cast<unsigned char *>(cst);
+        const int lrow = lane >> 3, lkc = lane & 7; // as a reader of A: row of the piece (and + 8), 16-byte chunk
+        const int gq = lane >> 4;                   // as a writer of the panel: k = 16 gq + L of the piece
+        TW_LDS(unsigned char) const tr_lane = (TW_LDS(unsigned char))tmp + (L >> 2) * TP + (gq * 16 + (L & 3) * 4) * 2;
+        constexpr int PP = 4; // pieces in flight per wave
+        for (int c0 = wave; c0 < n_pieces; c0 += kAsWaves * PP) {
+            u32x4 v[PP][2];
 #pragma unroll
-            for (int q = 0; q < PL; ++q) {
-                const int kc = base + q * kAsWaves * LPM;
-                v[q] = u32x4{0u, 0u, 0u, 0u};
-                if (kc < kchunks && m_ok)
-                    v[q] = *reinterpret_cast<const u32x4 *>(arow + kc * 8);
+            for (int q = 0; q < PP; ++q) {
+                const int c = c0 + q * kAsWaves;
+                const int mb = c % MB, kb = c / MB;
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int m = m0 + mb * 16 + h * 8 + lrow, kc = kb * 8 + lkc;
+                    v[q][h] = u32x4{0u, 0u, 0u, 0u};
+                    if (c < n_pieces && m < p.M && kc < kchunks)
+                        v[q][h] = *reinterpret_cast<const u32x4 *>(A + (int64_t)m * p.lda + kc * 8);
+                }
             }
 #pragma unroll
-            for (int q = 0; q < PL; ++q) {
-                const int kc = base + q * kAsWaves * LPM;
-                if (kc < kchunks) {
-                    const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+            for (int q = 0; q < PP; ++q) {
+                const int c = c0 + q * kAsWaves;
+                if (c < n_pieces) {
+                    const int mb = c % MB, kb = c / MB;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const int k = kc * 8 + e;
-                        const int half = BMS == 64 ? ((m >> 5) ^ ((k >> 1) & 1)) * 64 : 0;
+                    for (int h = 0; h < 2; ++h)
+                        *reinterpret_cast<u32x4 *>(tmp + (h * 8 + lrow) * TP + lkc * 16) = v[q][h];
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                    const int k = kb * 64 + gq * 16 + L;
+#pragma unroll
+                    for (int cc = 0; cc < 2; ++cc) {
+                        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(tr_lane + cc * 8 * TP));
+                        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(tr_lane + (cc * 8 + 4) * TP));
+                        const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                        const int mch = mb * 2 + cc;
+                        const int chs = BMS == 64 ? mch ^ (((k >> 1) & 1) << 2) : mch;
                         if (k < k_rows)
-                            *reinterpret_cast<uint16_t *>(dst + k * ROWB + half) =
-                                (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
+                            *reinterpret_cast<u32x4 *>(panel + k * ROWB + chs * 16) = u32x4{l2.x, l2.y, h2.x, h2.y};
                     }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the stage is free for the next piece
                 }
             }
         }
@@ -1373,7 +1394,6 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     };
 
     // ---- this wave's blocks, segment by segment
-    const int L = lane & 15;
     const int pair_e = (lane >> 5) * 4 + (L >> 2);            // this lane's word of a group's row pairs
     const int lane_b = ((lane >> 4) & 1) * 32 + (L & 3) * 8;  // its byte offset inside a 64-byte half row
     const int j = lane & 31;                                  // its compact column inside a block
@@ -1491,10 +1511,6 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
             return;
         const int cnt = min(32, c.u.n_cnt - c.nb * 32);
         if (RM) {
-            // rows m_lane + 8 * g + e, g = 0 .. 4 MI - 1, e = 0 .. 3: a running pointer, so that
-            // the 16 MI addresses are not all worked out (and kept in registers) ahead
-            const int m_lane = m0 + mi0 * 32 + (lane >> 5) * 4;
-            uint16_t *cp = C + (int64_t)m_lane * p.ldc + out_col;
 #pragma unroll
             for (int mi = 0; mi < MI; ++mi) {
                 float v[16];
@@ -1506,6 +1522,43 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
                 for (int r = 0; r < 16; ++r)
                     acc[mi][r] = tw_fp32_value(v[r]);
             }
+            // Where the block's compact columns are neighbours in C in aligned groups of eight
+            // (no column of the tile pruned, or whole groups), the product is turned through
+            // the wave's stage, [row][column], and leaves as 16-byte pieces of rows of C.
+            const int prev_col = __shfl_up(out_col, 1);
+            const bool octets = cnt % 8 == 0 &&
+                                __all(j >= cnt || ((j & 7) ? out_col == prev_col + 1 : (out_col & 7) == 0));
+            if (octets) {
+                const int r = lane >> 2, ch = lane & 3;
+                const int col = __shfl(out_col, ch * 8);
+#pragma unroll
+                for (int mi = 0; mi < MI; ++mi) {
+#pragma unroll
+                    for (int r4 = 0; r4 < 4; ++r4) {
+                        uint16_t *const dst = cst + ((lane >> 5) * 4 + r4 * 8) * CP + j;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            dst[e * CP] = (uint16_t)E::to_bits(acc[mi][r4 * 4 + e]);
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const int row = r + q * 16;
+                        const u32x2 lo = *reinterpret_cast<const u32x2 *>(cst + row * CP + ch * 8);
+                        const u32x2 hi = *reinterpret_cast<const u32x2 *>(cst + row * CP + ch * 8 + 4);
+                        const int m = m0 + (mi0 + mi) * 32 + row;
+                        if (ch * 8 < cnt && m < m_end)
+                            *reinterpret_cast<u32x4 *>(C + (int64_t)m * p.ldc + col) = u32x4{lo.x, lo.y, hi.x, hi.y};
+                    }
+                    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the stage is free again
+                }
+                clear();
+                return;
+            }
+            // rows m_lane + 8 * g + e, g = 0 .. 4 MI - 1, e = 0 .. 3: a running pointer, so that
+            // the 16 MI addresses are not all worked out (and kept in registers) ahead
+            const int m_lane = m0 + mi0 * 32 + (lane >> 5) * 4;
+            uint16_t *cp = C + (int64_t)m_lane * p.ldc + out_col;
 #pragma unroll
             for (int g = 0; g < 4 * MI; ++g) {
 #pragma unroll

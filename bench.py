@@ -140,7 +140,8 @@ def time_nmt_recurrence(wl, steps, torch):
     """One NMT time step is the masked gate GEMM (bias in its epilogue) followed by the LSTM gate
     arithmetic, which writes h_t into the rows of the next step's A (A_t = [x_t ; h_{t-1}],
     K-major).  `steps` time steps are recorded into a HIP graph and replayed; returns seconds per
-    step for the pair and for the gate kernel alone."""
+    step for the pair, for the gate kernel alone, and for the fused step (tw_lstm_step: GEMM, bias
+    and cell in one launch)."""
     from tilesparsity_amd import twgemm as tw
     M, K, N, dtype = wl["M"], wl["K"], wl["N"], wl["dtype"]
     H = N // 4
@@ -152,7 +153,7 @@ def time_nmt_recurrence(wl, steps, torch):
     bias = torch.zeros((N,), dtype=torch.float32, device="cuda")
     plan = tw.Plan.create(K, N, dtype, wl["tiles"], B)
     out = []
-    for with_gemm in (True, False):
+    for mode in ("pair", "gates", "fused"):
         side = torch.cuda.Stream()
         graph = torch.cuda.CUDAGraph()
         side.wait_stream(torch.cuda.current_stream())
@@ -161,7 +162,12 @@ def time_nmt_recurrence(wl, steps, torch):
                 s = torch.cuda.current_stream().cuda_stream
                 for i in range(steps):
                     a, a_next = At[i % 2], At[(i + 1) % 2]
-                    if with_gemm:
+                    if mode == "fused":
+                        plan.lstm_step(a.data_ptr(), M, cell.data_ptr(), cell.data_ptr(),
+                                       a_next.data_ptr() + (K - H) * M * 2, bias_ptr=bias.data_ptr(),
+                                       gates_ptr=gates.data_ptr(), stream=s)
+                        continue
+                    if mode == "pair":
                         plan.gemm(a.data_ptr(), gates.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO,
                                   stream=s, bias_ptr=bias.data_ptr())
                     tw.lstm_gates(M, H, dtype, gates.data_ptr(), M, 1.0, cell.data_ptr(), M,
@@ -180,7 +186,7 @@ def time_nmt_recurrence(wl, steps, torch):
         out.append(float(np.median(ts[1:])))
         del graph
     plan.destroy()
-    return out[0], out[1]
+    return out[0], out[1], out[2]
 
 
 def roofline_of(M, K, N, tiles, t, traffic=None):
@@ -620,9 +626,10 @@ def main():
             others[name]["us_row_major_a_and_c"] = t_direct * 1e6
             others[name]["us_row_major_a_staged_c_k_major"] = t_a_staged * 1e6
         if nmt:
-            t_step, t_gates = time_nmt_recurrence(make_workload(name), 50, torch)
+            t_step, t_gates, t_fused = time_nmt_recurrence(make_workload(name), 50, torch)
             others[name]["us_step_gemm_and_gates"] = t_step * 1e6
             others[name]["us_gates_alone"] = t_gates * 1e6
+            others[name]["us_step_fused"] = t_fused * 1e6
         print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
     if others:
         out["other_workloads"] = others

@@ -378,6 +378,21 @@ int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg, float
                   const float *c_prev, int64_t ldc_prev, float *c_new, int64_t ldc_new,
                   void *h_new, int64_t ldh, void *stream);
 
+/* One LSTM time step in one launch: the masked gate GEMM (N = 4H: the i, j, f, o blocks), the
+ * bias and the cell arithmetic of tw_lstm_gates, without the gate matrix going to memory (the
+ * pre-activations stay in fp32).  A is the K-major concat([x, h]) of the step, as for tw_gemm;
+ * bias fp32 [4H] or NULL; c_prev, c_new, h_new as for tw_lstm_gates.  h_new must not overlap
+ * the rows of A this launch reads: keep two A buffers and alternate (Pruning/NMT/nmt/
+ * model_helper.py:400-402 builds the cell; TensorFlow's dynamic_rnn double-buffers the state).
+ * The fused kernel takes plans whose tiles keep every column and are multiples of 32 columns
+ * wide (at most 128), with H a multiple of 32 up to 1024; for any other plan the call runs
+ * tw_gemm_ex (TW_PRUNED_ZERO, bias) into `gates_ws` ([4H][ldg] elements of the plan's dtype)
+ * and then tw_lstm_gates, or fails with TW_ERR_LAYOUT when gates_ws is NULL. */
+int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int M, const float *bias,
+                 float forget_bias, const float *c_prev, int64_t ldc_prev, float *c_new,
+                 int64_t ldc_new, void *h_new, int64_t ldh, void *gates_ws, int64_t ldg,
+                 void *stream);
+
 /* ---- TW mask producers ---------------------------------------------------------------
  * The reference derives its masks from importance scores with NumPy: per layer a 2-D score
  * matrix [K,N] (|w|; conv kernels HWIO reshaped to (H*W*I) x O, Pruning/VGG/prune_algo.py:16-24),

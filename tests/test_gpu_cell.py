@@ -109,3 +109,117 @@ def test_two_step_recurrence(tw, oracle, dtype):
     got_c = dC.cpu().numpy().T
     assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
     assert oracle.rel_error(got_c, c) <= 2 * TOL[dtype]
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,G,k_keep", [(128, 128, 0.5), (100, 64, 0.3), (33, 32, 0.6), (1, 128, 0.25)])
+def test_fused_step_recurrence(tw, oracle, dtype, M, G, k_keep):
+    """tw_lstm_step: gate GEMM, bias and cell in one launch, two time steps in a row with h_t
+    written into the next step's A (two A buffers in turn).  Against the oracle's recurrence with
+    fp32 pre-activations (the fused kernel never rounds the gate matrix), and against the
+    two-kernel form (tw_gemm_ex then tw_lstm_gates), which rounds it to 16 bits in between.
+    Ragged M; rows and padding beyond M stay untouched."""
+    import torch
+    rng = np.random.default_rng(97 + M + G)
+    I, H = 160, 256
+    K, N = I + H, 4 * H
+    W = (rng.standard_normal((K, N)) * 0.08).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.5).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=k_keep, n_keep=1.0, empty_every=7 if G == 32 else 0)
+    mask = oracle.plan_mask(K, N, tiles)
+    xs = [rng.standard_normal((M, I)).astype(np.float32) for _ in range(2)]
+    h0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    ld = (M + 7) // 8 * 8
+    PAD = 0x5a5a
+    s = torch.cuda.current_stream().cuda_stream
+
+    def operands():
+        A = []
+        for t in range(3):
+            a = np.full((K, ld), PAD, np.uint16)
+            a[:, :M] = 0
+            if t < 2:
+                a[:I, :M] = oracle.cast_bits(xs[t], dtype).reshape(M, I).T
+            A.append(a)
+        A[0][I:, :M] = oracle.cast_bits(h0, dtype).reshape(M, H).T
+        c = np.full((H, ld), 7.5, np.float32)
+        c[:, :M] = c0.T
+        return [to_device_bits(a, a.shape) for a in A], torch.from_numpy(c).cuda()
+
+    dbias = torch.from_numpy(bias).cuda()
+    with tw.Plan.create(K, N, dtype, tiles, W) as plan:
+        dA, dC = operands()
+        for t in range(2):
+            plan.lstm_step(dA[t].data_ptr(), M, dC.data_ptr(), dC.data_ptr(),
+                           dA[t + 1].data_ptr() + I * ld * 2, lda=ld, ldc_prev=ld, ldc_new=ld, ldh=ld,
+                           bias_ptr=dbias.data_ptr(), forget_bias=1.0, stream=s)
+        torch.cuda.synchronize()
+        dA2, dC2 = operands()
+        dG = torch.zeros((N, ld), dtype=torch.int16, device="cuda")
+        for t in range(2):
+            plan.gemm(dA2[t].data_ptr(), dG.data_ptr(), M, lda=ld, ldc=ld, pruned_cols=tw.PRUNED_ZERO,
+                      stream=s, bias_ptr=dbias.data_ptr())
+            tw.lstm_gates(M, H, dtype, dG.data_ptr(), ld, 1.0, dC2.data_ptr(), ld, dC2.data_ptr(), ld,
+                          dA2[t + 1].data_ptr() + I * ld * 2, ld, s)
+        torch.cuda.synchronize()
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+    h, c = q(h0), c0.astype(np.float64)
+    for t in range(2):
+        gates = oracle.mask_dense(np.concatenate([q(xs[t]), h], 1), q(W), mask, bias.astype(np.float64))
+        c, h = oracle.basic_lstm_cell(gates, c, 1.0)
+        h = q(h)
+    out = from_device_bits(dA[2])
+    got_h = oracle.bits_to_f32(np.ascontiguousarray(out[I:, :M]), dtype).reshape(H, M).T
+    got_c = dC.cpu().numpy()
+    assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
+    assert oracle.rel_error(got_c[:, :M].T, c) <= 2 * TOL[dtype]
+    # nothing beyond M, and the x rows of the last A, were written
+    assert np.all(out[:, M:] == PAD) and np.all(out[:I, :M] == 0)
+    assert np.all(got_c[:, M:] == 7.5)
+    # the two-kernel form rounds the pre-activations to 16 bits (an absolute error of 2^-11 or
+    # 2^-8 of a gate's magnitude, which can be most of a small h): close in absolute terms
+    two_h = oracle.bits_to_f32(np.ascontiguousarray(from_device_bits(dA2[2])[I:, :M]), dtype).reshape(H, M).T
+    bound = {"f16": 5e-3, "bf16": 4e-2}[dtype]      # |h| < 1, |c| of order 1, gates of order 4
+    assert np.max(np.abs(got_h - two_h)) <= bound
+    assert np.max(np.abs(got_c[:, :M].T - dC2.cpu().numpy()[:, :M].T)) <= bound
+
+
+def test_fused_step_without_bias_and_fallback(tw, oracle):
+    """No bias; and a plan the fused kernel does not take (pruned columns): the call then runs
+    tw_gemm_ex + tw_lstm_gates through the caller's gate matrix, and fails without one."""
+    import torch
+    rng = np.random.default_rng(131)
+    M, I, H, G, dtype = 64, 64, 128, 128, "f16"
+    K, N = I + H, 4 * H
+    W = (rng.standard_normal((K, N)) * 0.08).astype(np.float32)
+    x = rng.standard_normal((M, I)).astype(np.float32)
+    h0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+    a = np.zeros((K, M), np.uint16)
+    a[:I] = oracle.cast_bits(x, dtype).reshape(M, I).T
+    a[I:] = oracle.cast_bits(h0, dtype).reshape(M, H).T
+    s = torch.cuda.current_stream().cuda_stream
+    for n_keep in (1.0, 0.8):
+        tiles = random_tiles(rng, K, N, G, k_keep=0.5, n_keep=n_keep)
+        mask = oracle.plan_mask(K, N, tiles)
+        dA = to_device_bits(a, a.shape)
+        dC = torch.from_numpy(np.ascontiguousarray(c0.T)).cuda()
+        dH = torch.zeros((H, M), dtype=torch.int16, device="cuda")
+        dG = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+        with tw.Plan.create(K, N, dtype, tiles, W) as plan:
+            if n_keep < 1.0:
+                with pytest.raises(tw.TwError) as e:
+                    plan.lstm_step(dA.data_ptr(), M, dC.data_ptr(), dC.data_ptr(), dH.data_ptr(), stream=s)
+                assert e.value.status == tw.ERR_LAYOUT
+            plan.lstm_step(dA.data_ptr(), M, dC.data_ptr(), dC.data_ptr(), dH.data_ptr(),
+                           gates_ptr=dG.data_ptr(), stream=s)
+            torch.cuda.synchronize()
+        gates = oracle.mask_dense(np.concatenate([q(x), q(h0)], 1), q(W), mask, np.zeros(N))
+        c, h = oracle.basic_lstm_cell(gates if n_keep == 1.0 else q(gates), c0.astype(np.float64), 1.0)
+        got_h = oracle.bits_to_f32(from_device_bits(dH), dtype).reshape(H, M).T
+        assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
+        assert oracle.rel_error(dC.cpu().numpy().T, c) <= 2 * TOL[dtype]
+        # the fused path leaves the caller's gate matrix alone
+        assert (int(dG.abs().max()) == 0) == (n_keep == 1.0)

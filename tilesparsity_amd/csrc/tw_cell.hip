@@ -4,6 +4,9 @@
 // the launch itself is most of its time.
 #include "tw_internal.h"
 
+#include <cstddef>
+#include <cstring>
+
 namespace tw {
 namespace {
 
@@ -89,10 +92,335 @@ __global__ void __launch_bounds__(256)
     }
 }
 
+// ---------------------------------------------------------------------------------
+// One LSTM time step in one launch: the gate GEMM of a tile-wise plan and the cell arithmetic,
+// for a handful of rows (the batch of a decoding step).  The i, j, f, o pre-activations of a
+// hidden unit are columns h, H + h, 2H + h, 3H + h of the GEMM, four different tiles with four
+// kept-row lists, so a workgroup takes 32 hidden units x 32 rows m and runs four K loops side
+// by side: wave w multiplies gate w / 2 and every second step of 64 kept rows (w % 2), two steps
+// at a time out of one register set, A turned through the wave's own piece of LDS as in the
+// skinny GEMM kernel.  The eight partial products meet in LDS; a thread then owns two rows of
+// one hidden unit, adds its 4 x 2 partial sums in a fixed order, adds the bias and applies the
+// cell in fp32: the gate matrix never goes to memory and is never rounded to 16 bits.
+//   work:  workgroup (x, y): hidden units 32 x .. 32 x + 31, rows 32 y .. 32 y + 31
+//   table: entry 4 x + gate of the kernel arguments describes the 32-column block of that gate
+//          (its offset depends on the workgroup and wave numbers alone, so it arrives with the
+//          other arguments)
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+#define TW_LDS(T) __attribute__((address_space(3))) T *
+#define TW_GLOBAL(T) __attribute__((address_space(1))) T *
+
+template <int DT> __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32x16 c)
+{
+    if (DT == TW_F16)
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+
+struct LstmBlk {
+    int32_t kk_off;      // the tile's kept-K list in the padded array
+    int32_t nsteps;      // steps of 64 kept rows
+    int64_t b_first;     // byte offset of the block's first weight fragment
+    int64_t step_b;      // bytes from one step's fragments to the next
+};
+constexpr int kLstmMaxBlks = 128;        // 4 gates x 32 blocks of 32 hidden units: H <= 1024
+constexpr int kLstmWaves = 8;
+constexpr int kLstmStage = 2 * 64 * 64;  // bytes per wave: two steps of 64 rows k x 32 rows m
+constexpr int kLstmPitch = 36;           // floats per column of a partial product
+static_assert(32 * kLstmPitch * 4 <= kLstmStage, "a partial product reuses the wave's stage");
+
+struct LstmArgs {
+    const void *A;
+    const int32_t *kept_k;
+    const void *Bp;
+    const float *bias;
+    const float *c_prev;
+    float *c_new;
+    void *h_new;
+    int64_t lda, ldcp, ldcn, ldh;
+    int32_t M, H;
+    float forget_bias;
+    int32_t pad_;
+    LstmBlk blk[kLstmMaxBlks];
+};
+static_assert(sizeof(LstmArgs) <= 4096, "kernel arguments");
+
+template <int DT>
+__global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_step_kernel(const LstmArgs p)
+{
+    __shared__ __align__(16) unsigned char smem[kLstmWaves * kLstmStage];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int gate = wave >> 1, kh = wave & 1;
+    const int hb = blockIdx.x, m0 = blockIdx.y * 32;
+    // the block of this wave's gate, and the arguments the first loads need, asked for at once
+    uintptr_t A_i = (uintptr_t)p.A, kk_i = (uintptr_t)p.kept_k, Bp_i = (uintptr_t)p.Bp;
+    int64_t lda = p.lda;
+    int M = p.M;
+    LstmBlk blk;
+    {
+        const auto *ka = (const __attribute__((address_space(4))) int32_t *)__builtin_amdgcn_kernarg_segment_ptr();
+        int32_t w[6];
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+            w[i] = ka[offsetof(LstmArgs, blk) / 4 + (hb * 4 + gate) * 6 + i];
+#pragma unroll
+        for (int i = 0; i < 6; ++i)
+            asm volatile("" : "+s"(w[i]));
+        asm volatile("" : "+s"(A_i), "+s"(kk_i), "+s"(Bp_i), "+s"(lda), "+s"(M));
+        __builtin_memcpy(&blk, w, sizeof(LstmBlk));
+    }
+    static_assert(sizeof(LstmBlk) == 24, "LstmBlk is read as 6 words");
+    TW_GLOBAL(const uint16_t) const A = (TW_GLOBAL(const uint16_t))A_i;
+    TW_GLOBAL(const int32_t) const kept_k = (TW_GLOBAL(const int32_t))kk_i;
+    TW_GLOBAL(const unsigned char) const Bp = (TW_GLOBAL(const unsigned char))Bp_i;
+    const int nsteps = blk.nsteps;
+    unsigned char *const stage = smem + wave * kLstmStage;
+
+    struct Numbers {
+        int row[2][4];
+    };
+    struct Loads {
+        u32x4 a[2][4], b[2][4];
+    };
+    TW_GLOBAL(const unsigned char) const bsrc = Bp + blk.b_first + lane * 16;
+    const int ch = lane & 3, row16 = lane >> 2;
+    // nothing on the way to the operands is conditional (exact wait counts): a chunk of rows past
+    // M is fetched from the row block's first chunk, a second step past the end repeats the first
+    TW_GLOBAL(const uint16_t) const a_lane = A + m0 + (m0 + ch * 8 < M ? ch * 8 : 0);
+    constexpr int kStride = 2;           // this wave's steps: kh, kh + 2, ...
+    constexpr int kPair = 2 * kStride;   // a pair: steps s and s + 2
+    auto numbers = [&](int s) {
+        Numbers n;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int st = s + t * kStride < nsteps ? s + t * kStride : s;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                n.row[t][i] = kept_k[blk.kk_off + st * kBlockK + i * 16 + row16];
+        }
+        return n;
+    };
+    auto issue = [&](int s, const Numbers &n, Loads &l) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const int st = s + t * kStride < nsteps ? s + t * kStride : s;
+#pragma unroll
+            for (int k16 = 0; k16 < 4; ++k16)
+                l.b[t][k16] = *(TW_GLOBAL(const u32x4))(bsrc + st * blk.step_b + k16 * 1024);
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                l.a[t][i] = *(TW_GLOBAL(const u32x4))(a_lane + (int64_t)n.row[t][i] * lda);
+    };
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+        acc[r] = 0.0f;
+    const int L = lane & 15;
+    const int pair_e = (lane >> 5) * 4 + (L >> 2);
+    const int lane_b = ((lane >> 4) & 1) * 32 + (L & 3) * 8;
+    const uint32_t r_first = (uint32_t)((pair_e >> 2) * 8 + (pair_e & 3));
+    auto multiply = [&](int s, const Loads &l) {
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) = l.a[t][i];
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))stage + lane_b;
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+            if (s + t * kStride < nsteps) {
+#pragma unroll
+                for (int k16 = 0; k16 < 4; ++k16) {
+                    const uint32_t r_lo = t * 64 + r_first + k16 * 16, r_hi = r_lo + 4;
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_lo * 64));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_hi * 64));
+                    const u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
+                    acc = mfma16<DT>(u32x4{l2.x, l2.y, h2.x, h2.y}, l.b[t][k16], acc);
+                }
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // read before the next steps overwrite it
+    };
+    int s = kh;
+    Loads l0, l1;
+    Numbers n;
+    if (s < nsteps) {
+        n = numbers(s);
+        issue(s, n, l0);
+        if (s + kPair < nsteps)
+            n = numbers(s + kPair);
+    }
+    // behind the first operands on their way: what the cell needs of this thread's two rows of
+    // hidden unit hb * 32 + tid / 16
+    const int ju = tid >> 4, m2 = (tid & 15) * 2;
+    const int hu = hb * 32 + ju;
+    const bool row_ok = m0 + m2 < p.M;
+    float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (p.bias) {
+        TW_GLOBAL(const float) const gb = (TW_GLOBAL(const float))(uintptr_t)p.bias;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            bias4[g] = gb[g * p.H + hu];
+    }
+    f32x2 c_old = f32x2{0.0f, 0.0f};
+    if (row_ok)
+        c_old = *(TW_GLOBAL(const f32x2))(uintptr_t)(p.c_prev + (int64_t)hu * p.ldcp + m0 + m2);
+    while (s < nsteps) {
+        if (s + kPair < nsteps) {
+            issue(s + kPair, n, l1);
+            if (s + 2 * kPair < nsteps)
+                n = numbers(s + 2 * kPair);
+        }
+        multiply(s, l0);
+        s += kPair;
+        if (s >= nsteps)
+            break;
+        if (s + kPair < nsteps) {
+            issue(s + kPair, n, l0);
+            if (s + 2 * kPair < nsteps)
+                n = numbers(s + 2 * kPair);
+        }
+        multiply(s, l1);
+        s += kPair;
+    }
+    // the partial product of this wave: column lane % 32, rows r4 * 8 + (lane / 32) * 4 + e
+    float *const part = reinterpret_cast<float *>(stage);
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+        float *const dst = part + (lane & 31) * kLstmPitch + r4 * 8 + (lane >> 5) * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            dst[e] = acc[r4 * 4 + e];
+    }
+    __syncthreads();
+    if (!row_ok)
+        return;
+    float pre[4][2];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const float *const lo = reinterpret_cast<const float *>(smem + (2 * g) * kLstmStage) + ju * kLstmPitch + m2;
+        const float *const hi = reinterpret_cast<const float *>(smem + (2 * g + 1) * kLstmStage) + ju * kLstmPitch + m2;
+#pragma unroll
+        for (int e = 0; e < 2; ++e)
+            pre[g][e] = (lo[e] + hi[e]) + bias4[g];
+    }
+    float c2[2] = {c_old.x, c_old.y}, h2[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e)
+        cell_update(pre[0][e], pre[1][e], pre[2][e], pre[3][e], p.forget_bias, c2[e], h2[e]);
+    float *const cdst = p.c_new + (int64_t)hu * p.ldcn + m0 + m2;
+    uint16_t *const hdst = reinterpret_cast<uint16_t *>(p.h_new) + (int64_t)hu * p.ldh + m0 + m2;
+    if (m0 + m2 + 1 < p.M) {
+        *reinterpret_cast<f32x2 *>(cdst) = f32x2{c2[0], c2[1]};
+        *reinterpret_cast<uint32_t *>(hdst) = (uint32_t)to16(h2[0], DT) | ((uint32_t)to16(h2[1], DT) << 16);
+    } else {
+        cdst[0] = c2[0];
+        hdst[0] = to16(h2[0], DT);
+    }
+}
+
 } // namespace
 } // namespace tw
 
 using namespace tw;
+
+extern "C" int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int M, const float *bias,
+                            float forget_bias, const float *c_prev, int64_t ldc_prev, float *c_new,
+                            int64_t ldc_new, void *h_new, int64_t ldh, void *gates_ws, int64_t ldg,
+                            void *stream)
+{
+    if (!plan)
+        return fail(TW_ERR_NULL, "plan is NULL");
+    if (M < 0)
+        return fail(TW_ERR_SHAPE, "M=%d", M);
+    if (plan->N % 4)
+        return fail(TW_ERR_SHAPE, "N=%d is not four gates wide", plan->N);
+    const int H = plan->N / 4;
+    if (M == 0)
+        return TW_OK;
+    if (!A || !c_prev || !c_new || !h_new)
+        return fail(TW_ERR_NULL, "A, c_prev, c_new or h_new is NULL");
+    // what the fused kernel takes: every column kept, tiles that are whole blocks of 32 columns and
+    // one work item each, at most 128 blocks in all
+    bool fused = H % 32 == 0 && H / 32 * 4 <= kLstmMaxBlks && plan->n_units == plan->n_tiles;
+    for (int t = 0; t < plan->n_tiles && fused; ++t)
+        fused = plan->tile_col0[t] % 32 == 0 && plan->tile_width[t] % 32 == 0 &&
+                plan->kept_n_ptr[t + 1] - plan->kept_n_ptr[t] == plan->tile_width[t];
+    if (!fused) {
+        if (!gates_ws)
+            return fail(TW_ERR_LAYOUT, "this plan needs the two-kernel form (pruned columns, tiles that are no "
+                                       "multiple of 32 columns, or H > 1024): pass a gate matrix of 4H x ldg elements");
+        tw_epilogue ep;
+        ep.bias = bias;
+        ep.activation = TW_ACT_NONE;
+        int rc = tw_gemm_ex(plan, A, TW_LAYOUT_KMAJOR, lda, gates_ws, TW_LAYOUT_KMAJOR, ldg, M, 1.0f, 0.0f,
+                            TW_PRUNED_ZERO, &ep, stream);
+        if (rc != TW_OK)
+            return rc;
+        return tw_lstm_gates(M, H, plan->dtype, gates_ws, ldg, forget_bias, c_prev, ldc_prev, c_new, ldc_new,
+                             h_new, ldh, stream);
+    }
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev != plan->device)
+        return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d", plan->device, dev);
+    if (lda < M || ldc_prev < M || ldc_new < M || ldh < M)
+        return fail(TW_ERR_SHAPE, "leading dimensions %lld %lld %lld %lld must be >= M=%d", (long long)lda,
+                    (long long)ldc_prev, (long long)ldc_new, (long long)ldh, M);
+    if ((lda & 7) || (ldh & 7) || (ldc_prev & 3) || (ldc_new & 3))
+        return fail(TW_ERR_ALIGNMENT, "lda and ldh must be multiples of 8 elements, ldc_prev and ldc_new of 4");
+    if (((uintptr_t)A & 15) || ((uintptr_t)h_new & 15) || ((uintptr_t)c_prev & 15) || ((uintptr_t)c_new & 15))
+        return fail(TW_ERR_ALIGNMENT, "all buffers must be 16-byte aligned");
+    const int64_t row_blocks = ((int64_t)M + 31) / 32;
+    if (row_blocks > 65535)
+        return fail(TW_ERR_SHAPE, "M=%d: the fused step takes at most %d rows", M, 65535 * 32);
+    LstmArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.A = A;
+    a.kept_k = plan->d_kept_k_pad;
+    a.Bp = plan->d_Bp;
+    a.bias = bias;
+    a.c_prev = c_prev;
+    a.c_new = c_new;
+    a.h_new = h_new;
+    a.lda = lda;
+    a.ldcp = ldc_prev;
+    a.ldcn = ldc_new;
+    a.ldh = ldh;
+    a.M = M;
+    a.H = H;
+    a.forget_bias = forget_bias;
+    a.pad_ = 0;
+    for (const UnitDev &u : plan->h_units) {
+        // the unit's blocks: columns col0 + 32 nb of C, i.e. gate (col / H), hidden block (col % H) / 32
+        for (int nb = 0; nb < u.nb_cnt; ++nb) {
+            const int col = u.col0 + 32 * nb;
+            LstmBlk &b = a.blk[(col % H) / 32 * 4 + col / H];
+            b.kk_off = u.kk_off;
+            b.nsteps = u.k_pad / kBlockK;
+            b.b_first = u.b_off * 2 + (int64_t)(u.nb0 + nb) * 4096;
+            b.step_b = (int64_t)u.nblk * 4096;
+        }
+    }
+    if (plan->dtype == TW_F16)
+        hipLaunchKernelGGL((tw_lstm_step_kernel<TW_F16>), dim3((unsigned)(H / 32), (unsigned)row_blocks),
+                           dim3(64 * kLstmWaves), 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((tw_lstm_step_kernel<TW_BF16>), dim3((unsigned)(H / 32), (unsigned)row_blocks),
+                           dim3(64 * kLstmWaves), 0, (hipStream_t)stream, a);
+    TW_HIP(hipGetLastError());
+    return TW_OK;
+}
 
 extern "C" int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg,
                              float forget_bias, const float *c_prev, int64_t ldc_prev, float *c_new,

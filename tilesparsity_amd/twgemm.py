@@ -52,7 +52,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_granularity", "tw_plan_from_export", "tw_plan_from_mask_cover", "tw_tiles_from_mask",
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
     "tw_gemm_staged", "tw_gemm_staged_workspace",
-    "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm", "tw_plan_reset",
+    "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm", "tw_plan_reset", "tw_lstm_step",
 )
 
 
@@ -157,6 +157,7 @@ def lib():
         "tw_plan_from_mask_cover": (c_int, [c_int, c_int, c_int, c_int, i32p, i32p, u8p, f32p, pp]),
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
         "tw_plan_reset": (c_int, [vp, vp]),
+        "tw_lstm_step": (c_int, [vp, vp, c_i64, c_int, vp, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
         "tw_side_create": (c_int, [c_int, c_int, c_int, u8p, f32p, pp]),
         "tw_side_destroy": (None, [vp]),
         "tw_side_nnz": (c_i64, [vp]),
@@ -384,6 +385,19 @@ class Plan:
         return cls(h.value, K, N, dtype_code(dtype))
 
     # -- inspection
+    def lstm_step(self, A_ptr, M, c_prev_ptr, c_new_ptr, h_new_ptr, lda=None, ldc_prev=None,
+                  ldc_new=None, ldh=None, bias_ptr=None, forget_bias=1.0, gates_ptr=None, ldg=None,
+                  stream=0):
+        """One LSTM time step on K-major device buffers (see tw_lstm_step): the gate GEMM of this
+        plan (N = 4H) and the cell arithmetic in one launch where the plan allows it, else
+        tw_gemm_ex into `gates_ptr` followed by tw_lstm_gates."""
+        vp = ctypes.c_void_p
+        ld = lambda v: M if v is None else v
+        _check(lib().tw_lstm_step(self._h, vp(int(A_ptr or 0)), ld(lda), M, vp(int(bias_ptr or 0)),
+                                  forget_bias, vp(int(c_prev_ptr or 0)), ld(ldc_prev),
+                                  vp(int(c_new_ptr or 0)), ld(ldc_new), vp(int(h_new_ptr or 0)), ld(ldh),
+                                  vp(int(gates_ptr or 0)), ld(ldg), vp(int(stream or 0))))
+
     def reset(self, stream=0):
         """Re-arms the plan's work-queue counters (after a launch of it was aborted mid-flight)."""
         _check(lib().tw_plan_reset(self._h, ctypes.c_void_p(int(stream or 0))))

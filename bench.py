@@ -82,6 +82,34 @@ def time_plan(plan, bufs, M, steps, warmup, torch):
     return time_steps(launch, steps, warmup, torch)
 
 
+def time_plan_streams(plan, bufs, M, steps, warmup, torch, n_streams=2):
+    """Seconds per launch when the launches, which do not depend on each other (each has its own
+    A and C), are issued on `n_streams` streams in turn, as the reference issues its per-tile
+    GEMMs on streams of their own (Stream_Gemm_NN, basic_nn.cu:396-430): the last workgroups of
+    one launch then run next to the first of the next.  Throughput of independent launches, not
+    the duration of one: the headline figure and the roofline stay with the single stream."""
+    main = torch.cuda.current_stream()
+    streams = [torch.cuda.Stream() for _ in range(n_streams)]
+    n = len(bufs)
+
+    def run(count):
+        for i in range(count):
+            a, c = bufs[i % n]
+            plan.gemm(a.data_ptr(), c.data_ptr(), M, stream=streams[i % n_streams].cuda_stream)
+    run(warmup)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(main)
+    for st in streams:
+        st.wait_event(start)
+    run(steps)
+    for st in streams:
+        main.wait_stream(st)
+    stop.record(main)
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / steps
+
+
 def time_plan_graph(plan, bufs, M, steps, warmup, torch):
     """The same with the `steps` launches recorded once into a HIP graph and the graph replayed:
     for launches of a few microseconds, which the host cannot issue as fast as the GPU runs them
@@ -226,6 +254,10 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
     t_sparse = timer(sparse, bufs, M, steps, warmup, torch)
     reps_sparse = [timer(sparse, bufs, M, steps, 2, torch) for _ in range(repeats)]
     reps_dense = [timer(dense, bufs, M, steps, 2, torch) for _ in range(repeats)]
+    two = None
+    if not graph:
+        two = [float(np.median([time_plan_streams(pl, bufs, M, steps, 2, torch) for _ in range(3)]))
+               for pl in (sparse, dense)]
     sparse.destroy()
     dense.destroy()
     # the library's dense GEMM in the same layout: C^T [N, M] = W^T [N, K] . A^T [K, M]
@@ -251,6 +283,11 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
         algorithmic_bytes=by, hbm_gbs=by / t_sparse / 1e9, rotating_buffer_sets=n_sets,
         kept_flops=fk, dense_flops=fd,
         roofline=roofline_of(M, K, N, tiles, t_sparse, MEASURED_TRAFFIC_BYTES.get(wl["name"])))
+    if two:
+        # independent launches on two streams in turn (throughput, see time_plan_streams)
+        res["two_streams"] = dict(us_sparse=two[0] * 1e6, us_dense_plan=two[1] * 1e6,
+                                  speedup_vs_dense_plan=two[1] / two[0],
+                                  effective_tflops=fd / two[0] / 1e12, hbm_gbs=by / two[0] / 1e9)
     del bufs, At, Wt
     torch.cuda.empty_cache()
     return res, (A, B)
@@ -600,6 +637,8 @@ def main():
         "repeats_for_medians": res["repeats"],
         "roofline": roof,
     }
+    if "two_streams" in res:
+        out["independent_launches_on_two_streams"] = res["two_streams"]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, A, B)
     del A, B
@@ -621,6 +660,8 @@ def main():
                                           "us_dense_library", "effective_tflops", "actual_tflops",
                                           "speedup_vs_dense", "speedup_vs_dense_library",
                                           "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "roofline")}
+        if "two_streams" in r:
+            others[name]["independent_launches_on_two_streams"] = r["two_streams"]
         if name == "bert_base_ffn":
             t_direct, t_a_staged = time_row_major(make_workload(name), args.steps, args.warmup, torch)
             others[name]["us_row_major_a_and_c"] = t_direct * 1e6

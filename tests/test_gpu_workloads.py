@@ -125,6 +125,49 @@ def test_config3_nmt_lstm_gates_50_steps(tw, oracle):
         assert np.array_equal(from_device_bits(C), first)
 
 
+def test_config3_fused_time_steps(tw, oracle):
+    """The NMT configuration at full size through tw_lstm_step: three time steps of the fused
+    launch (gate GEMM, bias, cell) against the oracle's recurrence, with h handed on in fp16
+    through the rows of the next step's A; and the same launches once more, bit for bit."""
+    import torch
+    from tilesparsity_amd import workloads as W
+    wl = W.nmt_lstm_gates()
+    M, K, N = wl["M"], wl["K"], wl["N"]
+    H = N // 4
+    I = K - H
+    A, B = wl["values"]()
+    rng = np.random.default_rng(5)
+    bias = (rng.standard_normal(N) * 0.3).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    mask = oracle.plan_mask(K, N, wl["tiles"])
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), "f16").astype(np.float64)
+    s = torch.cuda.current_stream().cuda_stream
+    dbias = torch.from_numpy(bias).cuda()
+    At = torch.from_numpy(A).cuda().half().t().contiguous()        # [K, M]: x rows, then h rows
+    with tw.Plan.create(K, N, "f16", wl["tiles"], B) as plan:
+        runs = []
+        for rep in range(2):
+            bufs = [At.clone(), At.clone()]
+            cell = torch.from_numpy(np.ascontiguousarray(c0.T)).cuda()
+            for t in range(3):
+                a, a_next = bufs[t % 2], bufs[(t + 1) % 2]
+                plan.lstm_step(a.data_ptr(), M, cell.data_ptr(), cell.data_ptr(),
+                               a_next.data_ptr() + I * M * 2, bias_ptr=dbias.data_ptr(), stream=s)
+            torch.cuda.synchronize()
+            runs.append((bufs[1][I:].clone(), cell.clone()))
+        assert torch.equal(runs[0][0], runs[1][0]) and torch.equal(runs[0][1], runs[1][1])
+    x = q(A[:, :I])
+    h, c = q(A[:, I:]), c0.astype(np.float64)
+    for t in range(3):
+        gates = oracle.mask_dense(np.concatenate([x, h], 1), q(B), mask, bias.astype(np.float64))
+        c, h = oracle.basic_lstm_cell(gates, c, 1.0)
+        h = q(h)
+    got_h = runs[0][0].float().cpu().numpy().T
+    got_c = runs[0][1].cpu().numpy().T
+    assert oracle.rel_error(got_h, h) <= 2e-2
+    assert oracle.rel_error(got_c, c) <= 2e-2
+
+
 @pytest.mark.parametrize("which,keep", [(1, 0.5), (1, 0.25), (1, 0.10), (2, 0.5), (2, 0.25), (2, 0.10)])
 def test_config4_bert_large_ffn_bf16(tw, oracle, which, keep):
     from tilesparsity_amd import workloads as W

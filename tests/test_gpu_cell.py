@@ -223,3 +223,43 @@ def test_fused_step_without_bias_and_fallback(tw, oracle):
         assert oracle.rel_error(dC.cpu().numpy().T, c) <= 2 * TOL[dtype]
         # the fused path leaves the caller's gate matrix alone
         assert (int(dG.abs().max()) == 0) == (n_keep == 1.0)
+
+
+def test_fused_step_limits(tw, oracle):
+    """H = 1024 is the widest cell the fused kernel takes (bf16, ragged M); H = 1056 needs the
+    caller's gate matrix.  Both against the oracle."""
+    import torch
+    rng = np.random.default_rng(137)
+    s = torch.cuda.current_stream().cuda_stream
+    for H, G, dtype in ((1024, 128, "bf16"), (1056, 96, "f16")):
+        M, I = 40, 32
+        K, N = I + H, 4 * H
+        W = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+        bias = (rng.standard_normal(N) * 0.3).astype(np.float32)
+        tiles = random_tiles(rng, K, N, G, k_keep=0.3, n_keep=1.0)
+        mask = oracle.plan_mask(K, N, tiles)
+        xh = (rng.standard_normal((M, K)) * 0.7).astype(np.float32)
+        c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+        q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+        a = np.zeros((K, M), np.uint16)
+        a[:] = oracle.cast_bits(xh, dtype).reshape(M, K).T
+        dA = to_device_bits(a, a.shape)
+        dC = torch.from_numpy(np.ascontiguousarray(c0.T)).cuda()
+        dH = torch.zeros((H, M), dtype=torch.int16, device="cuda")
+        dG = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+        dbias = torch.from_numpy(bias).cuda()
+        with tw.Plan.create(K, N, dtype, tiles, W) as plan:
+            if H > 1024:
+                with pytest.raises(tw.TwError) as e:
+                    plan.lstm_step(dA.data_ptr(), M, dC.data_ptr(), dC.data_ptr(), dH.data_ptr(),
+                                   bias_ptr=dbias.data_ptr(), stream=s)
+                assert e.value.status == tw.ERR_LAYOUT
+            plan.lstm_step(dA.data_ptr(), M, dC.data_ptr(), dC.data_ptr(), dH.data_ptr(),
+                           bias_ptr=dbias.data_ptr(), gates_ptr=dG.data_ptr(), stream=s)
+            torch.cuda.synchronize()
+        assert (int(dG.abs().max()) == 0) == (H <= 1024)
+        gates = oracle.mask_dense(q(xh), q(W), mask, bias.astype(np.float64))
+        c, h = oracle.basic_lstm_cell(gates if H <= 1024 else q(gates), c0.astype(np.float64), 1.0)
+        got_h = oracle.bits_to_f32(from_device_bits(dH), dtype).reshape(H, M).T
+        assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
+        assert oracle.rel_error(dC.cpu().numpy().T, c) <= 2 * TOL[dtype]

@@ -382,8 +382,8 @@ int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg, float
  * bias and the cell arithmetic of tw_lstm_gates, without the gate matrix going to memory (the
  * pre-activations stay in fp32).  A is the K-major concat([x, h]) of the step, as for tw_gemm;
  * bias fp32 [4H] or NULL; c_prev, c_new, h_new as for tw_lstm_gates.  h_new must not overlap
- * the rows of A this launch reads: keep two A buffers and alternate (Pruning/NMT/nmt/
- * model_helper.py:400-402 builds the cell; TensorFlow's dynamic_rnn double-buffers the state).
+ * the rows of A this launch reads: keep two A buffers and alternate (the cell is built at
+ * Pruning/NMT/nmt/model_helper.py:400-402).
  * The fused kernel takes plans whose tiles keep every column and are multiples of 32 columns
  * wide (at most 128), with H a multiple of 32 up to 1024; for any other plan the call runs
  * tw_gemm_ex (TW_PRUNED_ZERO, bias) into `gates_ws` ([4H][ldg] elements of the plan's dtype)

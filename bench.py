@@ -232,7 +232,8 @@ def roofline_of(M, K, N, tiles, t, traffic=None):
             "frac": ach / MFMA_PEAK_TFLOPS, "traffic": traffic, "algorithmic_flops": fk}
 
 
-def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, graph=False):
+def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, graph=False,
+                 two_streams=False):
     """Times the TW plan (`steps` launches after `warmup`: the headline figure), then `repeats`
     more rounds of the same length each for the TW plan, for the 0 %-sparse plan of the same
     kernel and for the library's dense GEMM (torch.matmul, i.e. hipBLASLt / rocBLAS) on the same
@@ -255,7 +256,7 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
     reps_sparse = [timer(sparse, bufs, M, steps, 2, torch) for _ in range(repeats)]
     reps_dense = [timer(dense, bufs, M, steps, 2, torch) for _ in range(repeats)]
     two = None
-    if not graph:
+    if two_streams and not graph:
         two = [float(np.median([time_plan_streams(pl, bufs, M, steps, 2, torch) for _ in range(3)]))
                for pl in (sparse, dense)]
     sparse.destroy()
@@ -562,7 +563,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="vgg16_conv4_2")
+    ap.add_argument("--workload", default=None,
+                    help="one configuration only (default: vgg16_conv4_2 with the full report: the "
+                         "other target shapes and the two-stream leg)")
+    ap.add_argument("--two-streams", action="store_true",
+                    help="also time independent launches issued on two streams in turn")
     ap.add_argument("--all", action="store_true", help="also run the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--producers", action="store_true",
@@ -580,6 +585,9 @@ def main():
                          "so that FETCH_SIZE / WRITE_SIZE read under rocprofv3 can be scaled by what "
                          "the same counters show for a copy of known size")
     args = ap.parse_args()
+    full_report = args.workload is None   # no configuration named: the headline with everything
+    if full_report:
+        args.workload = "vgg16_conv4_2"
     if args.gpus != 1:
         print("bench.py: this engine and this benchmark use exactly one GPU; "
               "--gpus %d is not supported (run with --gpus 1)" % args.gpus, file=sys.stderr)
@@ -615,8 +623,9 @@ def main():
         del srcs, dsts
         torch.cuda.empty_cache()
 
+    two_streams = args.two_streams or full_report
     wl = make_workload(args.workload)
-    res, (A, B) = run_workload(wl, args.steps, args.warmup, torch)
+    res, (A, B) = run_workload(wl, args.steps, args.warmup, torch, two_streams=two_streams)
     roof = dict(res["roofline"])
     out = {
         "metric": "effective TFLOP/s (dense flops / time) at 75% TW sparsity, G=128",
@@ -655,7 +664,7 @@ def main():
     for name in names:
         nmt = name == "nmt_lstm_gates"
         r, _ = run_workload(make_workload(name), 50 if nmt else args.steps, args.warmup, torch,
-                            repeats=3, graph=nmt)
+                            repeats=3, graph=nmt, two_streams=two_streams)
         others[name] = {k: r[k] for k in ("us_sparse", "us_sparse_median", "us_dense",
                                           "us_dense_library", "effective_tflops", "actual_tflops",
                                           "speedup_vs_dense", "speedup_vs_dense_library",

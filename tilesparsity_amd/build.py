@@ -43,14 +43,33 @@ def _run(cmd):
         sys.stderr.write(out + "\n")
 
 
-def build_library(verbose=False):
-    srcs = [os.path.join(CSRC, s) for s in SOURCES]
-    cmd = [hipcc()] + HIPCC_FLAGS + ["-shared", "-o", LIB_PATH]
-    for s in srcs:
-        cmd += ["-x", "hip", s]
+def _compile_object(job):
+    src, obj = job
+    _run([hipcc()] + HIPCC_FLAGS + ["-c", "-x", "hip", src, "-o", obj])
+    return obj
+
+
+def build_library(verbose=False, force=True):
+    """Compiles every source to an object of its own (in parallel) and links them.  With
+    force=False a source is recompiled only when it, or a header, is newer than its object."""
+    from concurrent.futures import ThreadPoolExecutor
+    objdir = os.path.join(PKG_DIR, "build")
+    os.makedirs(objdir, exist_ok=True)
+    headers = [os.path.join(CSRC, "tw_internal.h"), os.path.join(ROOT, "include", "twgemm.h"),
+               os.path.abspath(__file__)]
+    newest_header = max(os.path.getmtime(h) for h in headers)
+    jobs, objs = [], []
+    for s in SOURCES:
+        src = os.path.join(CSRC, s)
+        obj = os.path.join(objdir, os.path.splitext(s)[0] + ".o")
+        objs.append(obj)
+        if force or not os.path.exists(obj) or os.path.getmtime(obj) < max(os.path.getmtime(src), newest_header):
+            jobs.append((src, obj))
     if verbose:
-        print(" ".join(cmd))
-    _run(cmd)
+        print("compiling: %s" % ", ".join(os.path.basename(j[0]) for j in jobs))
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as pool:
+        list(pool.map(_compile_object, jobs))
+    _run([hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
     return LIB_PATH
 
 
@@ -66,10 +85,11 @@ def build_perf_driver(verbose=False):
     return PERF_PATH
 
 
-def build_all(verbose=False):
-    build_library(verbose)
+def build_all(verbose=False, force=True):
+    build_library(verbose, force)
     build_perf_driver(verbose)
 
 
 if __name__ == "__main__":
-    build_all(verbose=True)
+    # `--changed` recompiles only the sources that are newer than their objects
+    build_all(verbose=True, force="--changed" not in sys.argv[1:])

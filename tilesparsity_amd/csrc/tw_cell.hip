@@ -125,7 +125,7 @@ template <int DT> __device__ __forceinline__ f32x16 mfma16(u32x4 a, u32x4 b, f32
 
 struct LstmBlk {
     int32_t kk_off;      // the tile's kept-K list in the padded array
-    int32_t nsteps;      // steps of 64 kept rows
+    int32_t k_kept;      // kept rows of the tile (steps of 64: rounded up)
     int64_t b_first;     // byte offset of the block's first weight fragment
     int64_t step_b;      // bytes from one step's fragments to the next
 };
@@ -180,7 +180,7 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_step_kernel(const 
     TW_GLOBAL(const uint16_t) const A = (TW_GLOBAL(const uint16_t))A_i;
     TW_GLOBAL(const int32_t) const kept_k = (TW_GLOBAL(const int32_t))kk_i;
     TW_GLOBAL(const unsigned char) const Bp = (TW_GLOBAL(const unsigned char))Bp_i;
-    const int nsteps = blk.nsteps;
+    const int nsteps = (blk.k_kept + kBlockK - 1) / kBlockK;
     unsigned char *const stage = smem + wave * kLstmStage;
 
     struct Numbers {
@@ -229,12 +229,21 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_step_kernel(const 
     const int pair_e = (lane >> 5) * 4 + (L >> 2);
     const int lane_b = ((lane >> 4) & 1) * 32 + (L & 3) * 8;
     const uint32_t r_first = (uint32_t)((pair_e >> 2) * 8 + (pair_e & 3));
+    // (a list of kept rows is padded to whole steps with row 0: what was fetched for the padding
+    // is replaced by zeros here, so that no value of a row the tile does not keep reaches a product)
+    const int k_lim = blk.k_kept - row16;
     auto multiply = [&](int s, const Loads &l) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+        for (int t = 0; t < 2; ++t) {
+            const int k0 = (s + t * kStride) * kBlockK;
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-                *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) = l.a[t][i];
+            for (int i = 0; i < 4; ++i) {
+                const uint32_t keep = k0 + i * 16 < k_lim ? 0xFFFFFFFFu : 0u;
+                const u32x4 v = l.a[t][i];
+                *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) =
+                    u32x4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+            }
+        }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))stage + lane_b;
 #pragma unroll
@@ -407,7 +416,7 @@ extern "C" int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int
             const int col = u.col0 + 32 * nb;
             LstmBlk &b = a.blk[(col % H) / 32 * 4 + col / H];
             b.kk_off = u.kk_off;
-            b.nsteps = u.k_pad / kBlockK;
+            b.k_kept = u.k_pad ? u.k_kept : 0;
             b.b_first = u.b_off * 2 + (int64_t)(u.nb0 + nb) * 4096;
             b.step_b = (int64_t)u.nblk * 4096;
         }

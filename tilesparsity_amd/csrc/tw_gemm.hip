@@ -1309,7 +1309,7 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
     const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
     uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
     const unsigned char *const Bp = reinterpret_cast<const unsigned char *>(p.Bp);
-    uint16_t *const cst = reinterpret_cast<uint16_t *>(as_smem + (size_t)k_rows * ROWB) + wave * 32 * CP;
+    uint16_t *const cst = reinterpret_cast<uint16_t *>(as_smem + (size_t)(k_rows + 1) * ROWB) + wave * 32 * CP;
 
     const int L = lane & 15;
     // ---- the panel: 16-byte chunks, sixteen loads in flight per thread (the first segment's
@@ -1636,6 +1636,9 @@ __global__ void __launch_bounds__(64 * as_waves(BMS, RM), 1)
         cur_first = first;
     }
     Cursor cur = cur_first;
+    // the row of zeros behind the panel: the padding of every list of kept rows points at it
+    if (tid < CH)
+        *reinterpret_cast<u32x4 *>(panel + (size_t)k_rows * ROWB + tid * 16) = u32x4{0u, 0u, 0u, 0u};
     __syncthreads();
     if (valid(cur)) {
         for (;;) {
@@ -1826,12 +1829,22 @@ __global__ void __launch_bounds__(64 * kSkWaves, 1) tw_gemm_skinny_kernel(const 
         const uint32_t r_first = (uint32_t)((pair_e >> 2) * 8 + (pair_e & 3));
 
         // the steps of the pair at s out of one register set: A through the stage, the products
+        // (the tile's list of kept rows is padded to whole steps with row 0: what was fetched for
+        // the padding is replaced by zeros here, so that no value of a row the tile does not keep,
+        // finite or not, ever reaches a product)
+        const int k_lim = u.k_kept - row16;
         auto multiply = [&](int s, const Loads &l) {
 #pragma unroll
-            for (int t = 0; t < 2; ++t)
+            for (int t = 0; t < 2; ++t) {
+                const int k0 = (s + t * kSkWaves) * kBlockK;
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) = l.a[t][i];
+                for (int i = 0; i < 4; ++i) {
+                    const uint32_t keep = k0 + i * 16 < k_lim ? 0xFFFFFFFFu : 0u;
+                    const u32x4 v = l.a[t][i];
+                    *reinterpret_cast<u32x4 *>(stage + (t * 64 + i * 16 + row16) * 64 + ch * 16) =
+                        u32x4{v.x & keep, v.y & keep, v.z & keep, v.w & keep};
+                }
+            }
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); // the rows are in the stage
             TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))stage + lane_b;
 #pragma unroll
@@ -2135,7 +2148,8 @@ static const Shape kShapes[TW_N_SHAPES] = {
 
 // LDS of the A-stationary kernel: the panel (all K rows, BMS rows m) and a C stage per wave
 constexpr int kLdsBytes = 160 * 1024;
-static int64_t as_lds_bytes(int K, int bms) { return (int64_t)K * bms * 2 + as_waves(bms, false) * 32 * 36 * 2; }
+// (and a row of zeros behind the panel)
+static int64_t as_lds_bytes(int K, int bms) { return (int64_t)(K + 1) * bms * 2 + as_waves(bms, false) * 32 * 36 * 2; }
 static bool is_as_shape(int shape) { return shape == TW_SHAPE_AS64 || shape == TW_SHAPE_AS32; }
 // shapes that walk the plan's units themselves: no work queue, no unit pieces
 static bool is_queueless_shape(int shape) { return is_as_shape(shape) || shape == TW_SHAPE_SKINNY; }

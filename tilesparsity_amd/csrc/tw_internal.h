@@ -66,7 +66,8 @@ struct GemmArgs {
     // k rows, the two rows a lane addresses in the group as 16-bit halves.  Entry
     // kk_off / 2 + step * 32 + e * 4 + group holds rows (e / 4) * 8 + e % 4 and that + 4 of the
     // group, so that the four words of a step a lane needs are one 16-byte load (null when K
-    // does not fit 16 bits).
+    // does not fit 16 bits).  The padding of a list up to whole steps names row K: the kernel keeps
+    // a row of zeros there, behind its panel of A.
     const uint32_t *kept_pairs;
     const int32_t *kept_n;
     const int32_t *pruned_n;

@@ -676,14 +676,18 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
             p->blocks_per_unit = 0;
     const size_t o_blocks = put(blocks.data(), blocks.size() * sizeof(int32_t));
     std::vector<uint32_t> kpairs; // see GemmArgs::kept_pairs
-    if (p->K <= 0xFFFF) {
+    if (p->K < 0xFFFF) {
+        // the padding names row K here (a row of zeros behind the kernel's panel of A), not row 0
+        std::vector<uint16_t> padded(kept_k_pad.size(), (uint16_t)p->K);
+        for (const UnitDev &u : units)
+            for (int i = 0; i < u.k_kept; ++i)
+                padded[u.kk_off + i] = (uint16_t)kept_k_pad[u.kk_off + i];
         kpairs.resize(kept_k_pad.size() / 2);
         for (size_t st = 0; st < kept_k_pad.size() / 64; ++st)
             for (int g16 = 0; g16 < 4; ++g16)
                 for (int e = 0; e < 8; ++e) {
                     const size_t lo = st * 64 + g16 * 16 + (e >> 2) * 8 + (e & 3);
-                    kpairs[st * 32 + e * 4 + g16] =
-                        (uint32_t)kept_k_pad[lo] | ((uint32_t)kept_k_pad[lo + 4] << 16);
+                    kpairs[st * 32 + e * 4 + g16] = (uint32_t)padded[lo] | ((uint32_t)padded[lo + 4] << 16);
                 }
     }
     const size_t o_kpairs = put(kpairs.data(), kpairs.size() * sizeof(uint32_t));

@@ -315,7 +315,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_SHAPE_AS64 7    /* A-stationary, 64 rows of all K in LDS: K up to 1064, beta == 0 */
 #define TW_SHAPE_AS32 8    /* A-stationary, 32 rows: K up to 2128, beta == 0 */
 #define TW_SHAPE_SKINNY 9  /* 64 rows x 32 columns per workgroup, the kept rows split over its waves: few rows of A */
-#define TW_N_SHAPES 10
+#define TW_SHAPE_BS 10     /* weight-stationary: a unit's packed weight in registers, A streamed: tiles of at most 192 kept rows, beta == 0 */
+#define TW_N_SHAPES 11
 int tw_set_option(int option, int value);
 
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument

@@ -555,13 +555,13 @@ def test_every_kernel_shape_agrees(tw, oracle, dtype):
     rng = np.random.default_rng(88)
     W, S1, S2, S3, S4, S5 = (tw.SHAPE_WIDE, tw.SHAPE_128x128, tw.SHAPE_512x64, tw.SHAPE_128x64,
                              tw.SHAPE_256x128, tw.SHAPE_128x32)
-    A6, A3, SK = tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY
+    A6, A3, SK, BS, S6 = tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY, tw.SHAPE_BS, tw.SHAPE_256x64
     cases = (
         (600, 320, 384, 128, ((W, -1), (S1, -1), (S4, -1), (S3, 64), (S5, 32), (S1, 64), (S4, 32),
-                              (A6, -1), (A3, -1), (SK, -1))),
+                              (A6, -1), (A3, -1), (SK, -1), (BS, -1))),
         (1100, 200, 256, 64, ((S2, -1), (S3, -1), (S5, 32), (S1, -1), (S4, -1), (W, -1), (A6, -1),
-                              (A3, -1), (SK, -1))),
-        (2500, 130, 96, 32, ((S5, -1), (S3, -1), (S2, -1), (A6, -1), (A3, -1), (SK, -1))),
+                              (A3, -1), (SK, -1), (BS, -1), (S6, -1), (S6, 32))),
+        (2500, 130, 96, 32, ((S5, -1), (S3, -1), (S2, -1), (A6, -1), (A3, -1), (SK, -1), (BS, -1), (S6, -1), (S6, 32))),
     )
     try:
         for (M, K, N, G, combos) in cases:

@@ -54,10 +54,10 @@ def test_unkept_rows_with_inf_and_nan_leave_c_finite(tw, oracle, dtype):
     cases = (
         # M, K, N, G, kept rows per tile (none a multiple of 64), shapes to force
         (200, 300, 384, 128, (70, 130, 1),
-         (tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY, tw.SHAPE_256x128, tw.SHAPE_128x128,
+         (tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY, tw.SHAPE_BS, tw.SHAPE_256x128, tw.SHAPE_128x128,
           tw.SHAPE_128x64, tw.SHAPE_WIDE, -1)),
-        (96, 520, 256, 64, (3, 200, 65, 127),
-         (tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY, tw.SHAPE_512x64, tw.SHAPE_256x64,
+        (96, 520, 256, 64, (3, 190, 65, 127),
+         (tw.SHAPE_AS64, tw.SHAPE_AS32, tw.SHAPE_SKINNY, tw.SHAPE_BS, tw.SHAPE_512x64, tw.SHAPE_256x64,
           tw.SHAPE_128x32, -1)),
     )
     s = torch.cuda.current_stream().cuda_stream

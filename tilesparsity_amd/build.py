@@ -15,7 +15,7 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 LIB_PATH = os.path.join(PKG_DIR, "libtwgemm.so")
 PERF_PATH = os.path.join(PKG_DIR, "test_basic_nn")
 
-SOURCES = ["tw_host.cpp", "tw_plan.hip", "tw_gemm.hip", "tw_prune.hip", "tw_cell.hip", "tw_layout.hip", "tw_side.hip"]
+SOURCES = ["tw_host.cpp", "tw_plan.hip", "tw_gemm.hip", "tw_gemm_bs.hip", "tw_prune.hip", "tw_cell.hip", "tw_layout.hip", "tw_side.hip"]
 
 HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -55,7 +55,8 @@ def build_library(verbose=False, force=True):
     from concurrent.futures import ThreadPoolExecutor
     objdir = os.path.join(PKG_DIR, "build")
     os.makedirs(objdir, exist_ok=True)
-    headers = [os.path.join(CSRC, "tw_internal.h"), os.path.join(ROOT, "include", "twgemm.h"),
+    headers = [os.path.join(CSRC, "tw_internal.h"), os.path.join(CSRC, "tw_device.h"),
+               os.path.join(ROOT, "include", "twgemm.h"),
                os.path.abspath(__file__)]
     newest_header = max(os.path.getmtime(h) for h in headers)
     jobs, objs = [], []

@@ -24,7 +24,7 @@
 //   * v_mfma_f32_32x32x16_{f16,bf16}, fp32 accumulators;
 //   * epilogue: alpha/beta in fp32, round to the 16-bit type, transpose through
 //     LDS, then scatter whole C columns (col0 + kept_n[j]) with 16-byte stores.
-#include "tw_internal.h"
+#include "tw_device.h"
 
 #include <algorithm>
 #include <atomic>
@@ -34,124 +34,6 @@
 #include <cstdlib>
 
 namespace tw {
-
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
-
-#define TW_LDS(T) __attribute__((address_space(3))) T *
-#define TW_GLOBAL(T) __attribute__((address_space(1))) T *
-
-#ifndef TW_A_PAD
-#define TW_A_PAD 32 // halfs of padding per staged A row: 64 B, so that the 4 rows x 2 column
-                    // halves one transposed read touches fall into 8 distinct 32-byte bank groups
-#endif
-
-template <int DT> struct Elem;
-template <> struct Elem<TW_F16> {
-    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                      __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ uint32_t to_bits(float f)
-    {
-        return __builtin_bit_cast(uint16_t, (_Float16)f);
-    }
-    static __device__ __forceinline__ float from_bits(uint16_t h)
-    {
-        return (float)__builtin_bit_cast(_Float16, h);
-    }
-};
-template <> struct Elem<TW_BF16> {
-    static __device__ __forceinline__ f32x16 mfma(u32x4 a, u32x4 b, f32x16 c)
-    {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                       __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ uint32_t to_bits(float f)
-    {
-        return __builtin_bit_cast(uint16_t, (__bf16)f); // v_cvt_pk_bf16_f32, nearest even
-    }
-    static __device__ __forceinline__ float from_bits(uint16_t h)
-    {
-        return __uint_as_float((uint32_t)h << 16);
-    }
-};
-
-// 16-byte chunk of column c, rows m..m+7 of a K-major matrix, honouring the M edge.  With
-// `through` the store writes through to memory (sc0 sc1) and does not linger in the caches (nt):
-// C is written once and not read again by this launch, and lines left dirty in the L2s would
-// otherwise all be written back after the last wave has ended, where nothing overlaps them.  A
-// small output is better left in the L2s: that write-back is short then, and shorter than the
-// last stores' way to memory.
-__device__ __forceinline__ void store_chunk(uint16_t *dst, u32x4 v, int m, int M, bool through)
-{
-    if (m + 8 <= M) {
-        if (through)
-            asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
-        else
-            *reinterpret_cast<u32x4 *>(dst) = v;
-    } else if (m < M) {
-        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-        for (int e = 0; e < M - m; ++e)
-            dst[e] = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
-    }
-}
-
-// Activation of the fused epilogue (tw_gemm_ex): the activations the reference's dense layers
-// can be given (get_activation, Pruning/BERT/utils/modeling.py:280-305); GELU in its tanh form
-// (modeling.py:264-277).
-__device__ __forceinline__ float tw_activate(float v, int act)
-{
-    if (act == TW_ACT_RELU)
-        return v > 0.0f ? v : 0.0f;
-    // tanh(u) = 1 - 2 / (exp(2u) + 1) with the hardware exponential and reciprocal (1 ulp each):
-    // exact limits at +-inf, ~1e-6 relative error in between, far below the 16-bit rounding
-    if (act == TW_ACT_GELU) {
-        const float u = 0.7978845608028654f * (v + 0.044715f * v * v * v);
-        return v - v * __builtin_amdgcn_rcpf(__expf(2.0f * u) + 1.0f); // 0.5 v (1 + tanh u)
-    }
-    if (act == TW_ACT_TANH)
-        return 1.0f - 2.0f * __builtin_amdgcn_rcpf(__expf(2.0f * v) + 1.0f);
-    return v;
-}
-// the same for a handful of values with the test of `act` outside the loop over them
-template <int N> __device__ __forceinline__ void tw_activate_all(float (&v)[N], int act)
-{
-    if (act == TW_ACT_RELU) {
-#pragma unroll
-        for (int e = 0; e < N; ++e)
-            v[e] = tw_activate(v[e], TW_ACT_RELU);
-    } else if (act == TW_ACT_GELU) {
-#pragma unroll
-        for (int e = 0; e < N; ++e)
-            v[e] = tw_activate(v[e], TW_ACT_GELU);
-    } else if (act == TW_ACT_TANH) {
-#pragma unroll
-        for (int e = 0; e < N; ++e)
-            v[e] = tw_activate(v[e], TW_ACT_TANH);
-    }
-}
-// The value of an output element is rounded to fp32 before it is rounded to 16 bits, in every
-// kernel: left to itself the compiler turns "multiply, add, convert" into one fused instruction
-// with a single rounding in some epilogues and not in others, and the kernels then differ in the
-// last bit of about one element in twenty thousand.
-__device__ __forceinline__ float tw_fp32_value(float v)
-{
-    asm volatile("" : "+v"(v));
-    return v;
-}
-// alpha*acc + beta*C is already in `v`: adds the bias of column c and applies the activation
-__device__ __forceinline__ float tw_finish(float v, const float *bias, int c, int act)
-{
-    if (bias)
-        v += bias[c];
-    return tw_activate(v, act);
-}
 
 // ---------------------------------------------------------------------------------
 // Work queue (see GemmArgs): entry q of queue x names one item, or nothing past the end.
@@ -187,49 +69,6 @@ __device__ __forceinline__ Work queue_entry(const GemmArgs &p, int x, int q)
     }
     w.kind = w.u < p.n_pipe_u ? ITEM_PIPE : (w.u < p.n_gemm_u ? ITEM_NOSTEP : ITEM_ZERO);
     return w;
-}
-
-// Piece `uv` of the unit table: unit uv / n_split, its columns [j * w, (j + 1) * w) with
-// w = 32 * piece_nb and j = uv % n_split.  A piece beyond the unit's columns keeps valid
-// offsets and has n_cnt == 0: it runs like any other and stores nothing.  The descriptor is
-// workgroup-uniform and ends up in scalar registers.
-__device__ __forceinline__ UnitDev load_unit(const GemmArgs &p, int uv)
-{
-    static_assert(sizeof(UnitDev) == 48, "UnitDev is read as 12 words");
-    const int ui = uv / p.n_split;
-    int32_t w[12];
-    if (p.n_arg_units) {
-        // from the kernel-argument segment: scalar loads, no global round trip
-        const auto *ka = (const __attribute__((address_space(4))) int32_t *)
-            __builtin_amdgcn_kernarg_segment_ptr();
-#pragma unroll
-        for (int i = 0; i < 12; ++i)
-            w[i] = ka[offsetof(GemmArgs, arg_units) / 4 + ui * 12 + i];
-    } else {
-        // the address is workgroup-uniform and the table is constant: scalar loads
-        const auto *gu = (const __attribute__((address_space(4))) int32_t *)(uintptr_t)(p.units + ui);
-#pragma unroll
-        for (int i = 0; i < 12; ++i)
-            w[i] = gu[i];
-    }
-#pragma unroll
-    for (int i = 0; i < 12; ++i)
-        w[i] = __builtin_amdgcn_readfirstlane(w[i]);
-    UnitDev u;
-    __builtin_memcpy(&u, w, sizeof(UnitDev));
-    if (p.n_split > 1) {
-        const int j = uv - ui * p.n_split;
-        const int bps = p.piece_nb; // 32-column blocks per piece
-        const int nb = min(max(u.nb_cnt - j * bps, 0), bps);
-        const int nc = min(max(u.n_cnt - j * bps * kMfmaN, 0), bps * kMfmaN);
-        if (nb > 0) {
-            u.nb0 += j * bps;
-            u.kn_off += j * bps * kMfmaN;
-        }
-        u.nb_cnt = nb;
-        u.n_cnt = nc;
-    }
-    return u;
 }
 
 // WM x WN waves of 64 x 64 outputs each: workgroup tile BM = 64*WM rows by BN = 64*WN
@@ -663,11 +502,6 @@ template <int NRD, int NMM, int I, bool READS> __device__ __forceinline__ void s
     if constexpr (I + 1 < NMM)
         sched_mfma_with_reads<NRD, NMM, I + 1, READS>();
 }
-
-// Workgroup barrier for hand-overs through LDS only: waits for this wave's LDS operations, not
-// for its global loads, stores or atomics in flight (which __syncthreads() would do for stores
-// and atomics), so prefetched loads, the item's output stores and the ticket atomic keep flying.
-#define TW_LDS_BARRIER() asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
 
 // ---------------------------------------------------------------------------------
 // Wave-specialised BM x BN kernel.  Half of the waves only multiply: multiplying wave w owns
@@ -2144,6 +1978,7 @@ static const Shape kShapes[TW_N_SHAPES] = {
     {64, 128, 1},  // TW_SHAPE_AS64
     {32, 128, 1},  // TW_SHAPE_AS32
     {32, 128, 1},  // TW_SHAPE_SKINNY
+    {64, 128, 3},  // TW_SHAPE_BS
 };
 
 // LDS of the A-stationary kernel: the panel (all K rows, BMS rows m) and a C stage per wave
@@ -2152,7 +1987,10 @@ constexpr int kLdsBytes = 160 * 1024;
 static int64_t as_lds_bytes(int K, int bms) { return (int64_t)(K + 1) * bms * 2 + as_waves(bms, false) * 32 * 36 * 2; }
 static bool is_as_shape(int shape) { return shape == TW_SHAPE_AS64 || shape == TW_SHAPE_AS32; }
 // shapes that walk the plan's units themselves: no work queue, no unit pieces
-static bool is_queueless_shape(int shape) { return is_as_shape(shape) || shape == TW_SHAPE_SKINNY; }
+static bool is_queueless_shape(int shape)
+{
+    return is_as_shape(shape) || shape == TW_SHAPE_SKINNY || shape == TW_SHAPE_BS;
+}
 
 // Steps of loads a moving wave keeps in flight, per shape (bounded by its 256 registers: a step
 // takes 4 * (A loads + weight loads per thread) of them).  Measured on the benchmark shapes: two
@@ -2259,7 +2097,7 @@ struct Choice {
 // workgroups of a die then share the rows of A in their L2 (measured on the 0 %-sparse plan of
 // the headline shape: a third of the reads from memory), but no benchmark shape ran faster for
 // it and the stress shape, whose 512-row block of A fills an L2, ran 13 % slower.
-static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c)
+static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc, bool reads_c)
 {
     Choice c;
     const int width = std::max(32, round_up32(plan->max_unit_n)); // 32, 64, 96 or 128
@@ -2291,8 +2129,19 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
     // (not beyond 1024 rows: M 2048, N 512 would still be two workgroups per unit, but each then
     // walks a whole tile's kept rows for 32 rows of A: 10 - 24 us against 6 - 15)
     const bool skinny = skinny_ok && M <= 1024 && (int64_t)plan->n_halves * ((M + 31) / 32) <= 2 * (int64_t)cu;
+    // The weight-stationary kernel where a tile keeps at most 192 rows under many rows of A, tiles
+    // wider than 64 columns.  Measured on M 512 .. 16384, K 768 / 1024 / 4096, N 1024 / 4096 with
+    // 64 .. 192 kept rows a tile against the choice below: from 2048 rows of A on it takes 0.58 -
+    // 1.05 of the time (median 0.79 - 0.86; most where K is too long for a panel of A in LDS),
+    // below that, and on tiles of 64 columns, it is as often slower as faster.
+    // Its workgroups (unit x range of rows) have to fill the chip's slots evenly: BERT-base's 24
+    // units give 384 workgroups for 512 slots, and the kernel is then 1 us slower than the
+    // A-stationary one (15 against 14), where 32 units (BERT-large FFN1 at 90 %) gain 12 %.
+    const bool bs = bs_takes(plan, lda, ldc, reads_c) && width > 64 && M >= 2048 && bs_fill(plan, M) >= 0.9;
     if (skinny) {
         c.shape = TW_SHAPE_SKINNY;
+    } else if (bs) {
+        c.shape = TW_SHAPE_BS;
     } else if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
     } else if (as_ok(TW_SHAPE_AS64) && (M > 128 || plan->n_blocks >= 96) &&
@@ -2347,6 +2196,9 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, bool reads_c
             c.shape = f_shape;
     } else if (f_shape == TW_SHAPE_SKINNY) {
         if (skinny_ok)
+            c.shape = f_shape;
+    } else if (f_shape == TW_SHAPE_BS) {
+        if (bs_takes(plan, lda, ldc, reads_c))
             c.shape = f_shape;
     } else if (f_shape >= 0 && (f_shape != TW_SHAPE_WIDE ? ws_ok : true)) {
         const int piece = f_piece > 0 ? f_piece : std::min(128, kShapes[f_shape].bn);
@@ -2543,6 +2395,8 @@ int launch_gemm(const tw_plan *plan, GemmArgs &a, const Choice &c, int32_t *tick
     }
     if (c.shape == TW_SHAPE_SKINNY)
         return plan->dtype == TW_F16 ? launch_skinny<TW_F16>(plan, a, s) : launch_skinny<TW_BF16>(plan, a, s);
+    if (c.shape == TW_SHAPE_BS)
+        return launch_bs(plan, a, option(TW_OPT_WGS_PER_CU), s);
     // queue 0 is the longest: one workgroup per entry, up to the chip's share of a queue
     const int64_t qlen0 = (int64_t)a.n_own_items + (a.n_tail_items + kXcd - 1) / kXcd;
     const int64_t per_queue = std::max<int64_t>(1, (int64_t)plan->cu_count * c.per_cu / kXcd);
@@ -2642,7 +2496,7 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
         return TW_OK;
     }
 
-    const Choice c = choose_shape(plan, M, lda, beta != 0.0f);
+    const Choice c = choose_shape(plan, M, lda, ldc, beta != 0.0f);
     fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
     if ((int64_t)a.n_all_u * a.n_mblk > kMaxItems)
         return fail(TW_ERR_SHAPE, "%lld work items (M=%d): a launch takes at most %lld",

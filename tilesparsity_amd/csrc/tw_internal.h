@@ -135,6 +135,7 @@ struct tw_plan {
     int n_halves = 0;   // pieces of 64 compact columns over all units (the skinny kernel's work per row block)
     int mean_steps = 0; // mean number of 64-row steps of the units that have any
     bool rows_shared = false; // nearly every tile keeps nearly every row (a dense or almost dense plan)
+    int max_k_pad = 0;        // most kept rows of a tile, rounded up to whole steps
     int cu_count = 0;
 };
 
@@ -178,6 +179,11 @@ int pack_from_stream(tw_plan *p, const void *d_Bs, const int64_t *off_B, hipStre
 // true when tw_gemm_ex takes a row-major A and a row-major C of this plan with a kernel of its own
 // (no layout-generic kernel, no staging): K short enough for a panel of A in LDS and C not read
 bool takes_row_major_directly(const tw_plan *p, float beta);
+// the weight-stationary kernel (tw_gemm_bs.hip): whether it takes the plan, and its launch with
+// `per_cu` workgroups meant to share a compute unit
+bool bs_takes(const tw_plan *p, int64_t lda, int64_t ldc, bool reads_c);
+int launch_bs(const tw_plan *p, const GemmArgs &a, int per_cu, hipStream_t s);
+double bs_fill(const tw_plan *p, int M); // share of the chip's workgroup slots its launch fills
 // device unpack: compacted stream layout (K*N 16-bit, zero elsewhere) from the packed weight
 int unpack_to_stream(const tw_plan *p, uint16_t *d_Bs, hipStream_t s);
 

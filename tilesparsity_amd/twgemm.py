@@ -25,7 +25,7 @@ KMAJOR, ROWMAJOR = 0, 1
 PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
 OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES = 0, 1, 2, 3
-SHAPE_AS64, SHAPE_AS32, SHAPE_SKINNY = 7, 8, 9
+SHAPE_AS64, SHAPE_AS32, SHAPE_SKINNY, SHAPE_BS = 7, 8, 9, 10
 SHAPE_WIDE, SHAPE_128x128, SHAPE_512x64, SHAPE_128x64, SHAPE_256x128, SHAPE_128x32, SHAPE_256x64 = range(7)
 
 

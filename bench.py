@@ -168,8 +168,9 @@ def time_nmt_recurrence(wl, steps, torch):
     """One NMT time step is the masked gate GEMM (bias in its epilogue) followed by the LSTM gate
     arithmetic, which writes h_t into the rows of the next step's A (A_t = [x_t ; h_{t-1}],
     K-major).  `steps` time steps are recorded into a HIP graph and replayed; returns seconds per
-    step for the pair, for the gate kernel alone, and for the fused step (tw_lstm_step: GEMM, bias
-    and cell in one launch)."""
+    step for the pair, for the gate kernel alone, for the fused step (tw_lstm_step: GEMM, bias
+    and cell in one launch), and for all `steps` time steps as one persistent launch
+    (tw_lstm_steps, timed with events around the call)."""
     from tilesparsity_amd import twgemm as tw
     M, K, N, dtype = wl["M"], wl["K"], wl["N"], wl["dtype"]
     H = N // 4
@@ -213,8 +214,20 @@ def time_nmt_recurrence(wl, steps, torch):
             ts.append(start.elapsed_time(stop) * 1e-3 / steps)
         out.append(float(np.median(ts[1:])))
         del graph
+    # the same `steps` time steps as ONE persistent launch (tw_lstm_steps), on steps + 1 matrices A_t
+    seq = torch.from_numpy(A).cuda().to(tdt).t().contiguous().unsqueeze(0).repeat(steps + 1, 1, 1).contiguous()
+    s = torch.cuda.current_stream().cuda_stream
+    ts = []
+    for _ in range(7):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record(torch.cuda.current_stream())
+        plan.lstm_steps(steps, seq.data_ptr(), M, cell.data_ptr(), bias_ptr=bias.data_ptr(), stream=s)
+        stop.record(torch.cuda.current_stream())
+        plan.lstm_steps_status(s)      # waits, and raises if the launch gave up at a barrier
+        ts.append(start.elapsed_time(stop) * 1e-3 / steps)
+    out.append(float(np.median(ts[1:])))
     plan.destroy()
-    return out[0], out[1], out[2]
+    return out[0], out[1], out[2], out[3]
 
 
 def roofline_of(M, K, N, tiles, t, traffic=None):
@@ -676,10 +689,11 @@ def main():
             others[name]["us_row_major_a_and_c"] = t_direct * 1e6
             others[name]["us_row_major_a_staged_c_k_major"] = t_a_staged * 1e6
         if nmt:
-            t_step, t_gates, t_fused = time_nmt_recurrence(make_workload(name), 50, torch)
+            t_step, t_gates, t_fused, t_persistent = time_nmt_recurrence(make_workload(name), 50, torch)
             others[name]["us_step_gemm_and_gates"] = t_step * 1e6
             others[name]["us_gates_alone"] = t_gates * 1e6
             others[name]["us_step_fused"] = t_fused * 1e6
+            others[name]["us_step_persistent"] = t_persistent * 1e6
         print("# %s %s" % (name, json.dumps(others[name])), file=sys.stderr, flush=True)
     if others:
         out["other_workloads"] = others

@@ -304,7 +304,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_WGS_PER_CU 1
 #define TW_OPT_PIECE 2
 #define TW_OPT_XCD_QUEUES 3
-#define TW_N_OPTIONS 4
+#define TW_OPT_SPIN_LIMIT 4 /* polls a workgroup of tw_lstm_steps spends at a barrier before it gives up (default 2^20) */
+#define TW_N_OPTIONS 5
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
 #define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns */
@@ -393,6 +394,28 @@ int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int M, const f
                  float forget_bias, const float *c_prev, int64_t ldc_prev, float *c_new,
                  int64_t ldc_new, void *h_new, int64_t ldh, void *gates_ws, int64_t ldg,
                  void *stream);
+
+/* T time steps of that cell in one launch.  A holds T + 1 K-major matrices [K][lda] at a_step
+ * elements from each other: A_t = [x_t ; h_(t-1)], the caller fills the K - H rows of x of A_0 ..
+ * A_(T-1) and the H rows of h of A_0; step t reads A_t and writes h_t into the rows of h of
+ * A_(t+1), so the call leaves the outputs h_0 .. h_(T-1) in A_1 .. A_T.  c (fp32 [H][ldc]) is
+ * the cell state, updated in place.  This is the recurrence the reference's dynamic_rnn runs
+ * over the cell of Pruning/NMT/nmt/model_helper.py:400-402, one kernel launch per time step
+ * there.
+ * Plans the fused step takes, with tiles of at most 512 kept rows and (H / 32) x ceil(M / 32)
+ * no larger than the number of compute units, run as ONE persistent launch: weights, row
+ * numbers, bias and cell state stay in registers, the workgroups meet at a barrier in device
+ * memory between two steps.  That barrier needs every workgroup of the launch resident at
+ * once; its polls are bounded (TW_OPT_SPIN_LIMIT), and a launch that gives up (the GPU was
+ * shared with other work) sets a status word and drains: tw_lstm_steps_status then returns
+ * TW_ERR_DEVICE.  Every other plan, and T == 1, runs as T calls of tw_lstm_step (gates_ws as
+ * there).  Asynchronous on `stream`; at most 192 such launches of one plan in flight. */
+int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, int64_t a_step, int M,
+                  const float *bias, float forget_bias, float *c, int64_t ldc, void *gates_ws,
+                  int64_t ldg, void *stream);
+/* Waits for `stream` and returns TW_ERR_DEVICE if a tw_lstm_steps launch of the plan gave up at
+ * its barrier since the last call (and clears that), else TW_OK. */
+int tw_lstm_steps_status(const tw_plan *plan, void *stream);
 
 /* ---- TW mask producers ---------------------------------------------------------------
  * The reference derives its masks from importance scores with NumPy: per layer a 2-D score

@@ -263,3 +263,163 @@ def test_fused_step_limits(tw, oracle):
         got_h = oracle.bits_to_f32(from_device_bits(dH), dtype).reshape(H, M).T
         assert oracle.rel_error(got_h, h) <= 2 * TOL[dtype]
         assert oracle.rel_error(dC.cpu().numpy().T, c) <= 2 * TOL[dtype]
+
+
+def _sequence_problem(rng, oracle, M, I, H, G, k_keep, T, dtype, ld, pad_bits=0x5a5a):
+    """x_0 .. x_(T-1), h_(-1), c_(-1) and the T + 1 K-major matrices A_t the engine takes."""
+    K, N = I + H, 4 * H
+    W = (rng.standard_normal((K, N)) * 0.08).astype(np.float32)
+    bias = (rng.standard_normal(N) * 0.5).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=k_keep, n_keep=1.0)
+    xs = [rng.standard_normal((M, I)).astype(np.float32) for _ in range(T)]
+    h0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    A = np.full((T + 1, K, ld), pad_bits, np.uint16)
+    A[:, :, :M] = 0
+    for t in range(T):
+        A[t, :I, :M] = oracle.cast_bits(xs[t], dtype).reshape(M, I).T
+    A[0, I:, :M] = oracle.cast_bits(h0, dtype).reshape(M, H).T
+    c = np.full((H, ld), 7.5, np.float32)
+    c[:, :M] = c0.T
+    return W, bias, tiles, xs, h0, c0, A, c
+
+
+def _oracle_recurrence(oracle, W, bias, tiles, xs, h0, c0, dtype):
+    """The oracle's cell on the oracle's gate GEMM, step after step, h rounded to 16 bits between
+    the steps as the engine hands it over; returns every h_t and the last c."""
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+    mask = oracle.plan_mask(W.shape[0], W.shape[1], tiles)
+    h, c, hs = q(h0), c0.astype(np.float64), []
+    for x in xs:
+        gates = oracle.mask_dense(np.concatenate([q(x), h], 1), q(W), mask, bias.astype(np.float64))
+        c, h = oracle.basic_lstm_cell(gates, c, 1.0)
+        h = q(h)
+        hs.append(h)
+    return hs, c
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("M,I,H,G,k_keep,T", [(128, 160, 256, 128, 0.5, 6), (100, 96, 128, 64, 0.3, 5),
+                                              (33, 40, 64, 32, 0.6, 9), (1, 64, 256, 128, 0.25, 3),
+                                              (200, 64, 1024, 128, 0.25, 3),    # 224 workgroups
+                                              (120, 1024, 1024, 128, 0.25, 4)])  # the NMT cell
+def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
+    """tw_lstm_steps: T time steps in one persistent launch (weights, row numbers and the cell state
+    stay in registers; a barrier in device memory between the steps).  Every h_t and the final c
+    against the oracle's recurrence (2 x the GEMM tolerance: errors of h feed the next step), within
+    the same bound of T calls of tw_lstm_step, the same bits on a second launch, nothing written beyond
+    M or into the rows of x, and a clean status."""
+    import torch
+    rng = np.random.default_rng(1000 + M + H + T)
+    K = I + H
+    ld = (M + 7) // 8 * 8
+    W, bias, tiles, xs, h0, c0, A, c = _sequence_problem(rng, oracle, M, I, H, G, k_keep, T, dtype, ld)
+    want_h, want_c = _oracle_recurrence(oracle, W, bias, tiles, xs, h0, c0, dtype)
+    dbias = torch.from_numpy(bias).cuda()
+    s = torch.cuda.current_stream().cuda_stream
+    outs = []
+    with tw.Plan.create(K, 4 * H, dtype, tiles, W) as plan:
+        for mode in ("steps", "steps", "single"):
+            dA = to_device_bits(A, A.shape)
+            dC = torch.from_numpy(c.copy()).cuda()
+            print("multi-step launch:", mode, M, I, H, G, T, dtype, flush=True)
+            if mode == "steps":
+                plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld,
+                                bias_ptr=dbias.data_ptr(), stream=s)
+                plan.lstm_steps_status(s)          # waits; raises if a barrier gave up
+            else:
+                for t in range(T):
+                    plan.lstm_step(dA[t].data_ptr(), M, dC.data_ptr(), dC.data_ptr(),
+                                   dA[t + 1].data_ptr() + I * ld * 2, lda=ld, ldc_prev=ld, ldc_new=ld, ldh=ld,
+                                   bias_ptr=dbias.data_ptr(), stream=s)
+                torch.cuda.synchronize()
+            outs.append((from_device_bits(dA).copy(), dC.cpu().numpy().copy()))
+    a_bits, c_out = outs[0]
+    for t in range(T):
+        got = oracle.bits_to_f32(np.ascontiguousarray(a_bits[t + 1, I:, :M]), dtype).reshape(H, M).T
+        assert oracle.rel_error(got, want_h[t]) <= 2 * TOL[dtype], t
+    assert oracle.rel_error(c_out[:, :M].T, want_c) <= 2 * TOL[dtype]
+    # rows of x, and everything beyond M, are as the caller left them
+    assert np.array_equal(a_bits[:, :I, :], A[:, :I, :]) and np.all(a_bits[:, :, M:] == 0x5a5a)
+    assert np.all(c_out[:, M:] == 7.5)
+    # a second launch gives the same bits; the T single launches differ from it in last bits only
+    # (the two kernels' cell arithmetic is contracted into fused multiply-adds differently, and a
+    # last-bit difference of h_t then feeds every later step)
+    assert np.array_equal(a_bits, outs[1][0]) and np.array_equal(c_out, outs[1][1])
+    single_h = oracle.bits_to_f32(np.ascontiguousarray(outs[2][0][1:, I:, :M]), dtype)
+    steps_h = oracle.bits_to_f32(np.ascontiguousarray(a_bits[1:, I:, :M]), dtype)
+    assert oracle.rel_error(steps_h, single_h) <= 2 * TOL[dtype]
+    assert oracle.rel_error(c_out[:, :M], outs[2][1][:, :M]) <= 2 * TOL[dtype]
+    assert np.array_equal(outs[2][0][:, :I, :], A[:, :I, :])
+
+
+def test_multi_step_launch_gives_up_cleanly(tw, oracle):
+    """The barrier's polls are bounded.  With no polls allowed at all a workgroup gives up at its
+    first barrier unless it happens to arrive last; every workgroup then leaves normally, the call
+    after it reports TW_ERR_DEVICE once, and the plan works again afterwards."""
+    import torch
+    rng = np.random.default_rng(5)
+    M, I, H, G, T, dtype = 128, 64, 256, 128, 4, "f16"
+    K, ld = I + H, 128
+    W, bias, tiles, xs, h0, c0, A, c = _sequence_problem(rng, oracle, M, I, H, G, 0.4, T, dtype, ld)
+    s = torch.cuda.current_stream().cuda_stream
+    with tw.Plan.create(K, 4 * H, dtype, tiles, W) as plan:
+        dA = to_device_bits(A, A.shape)
+        dC = torch.from_numpy(c.copy()).cuda()
+        try:
+            tw.set_option(tw.OPT_SPIN_LIMIT, 0)
+            print("multi-step launch with no polls", flush=True)
+            plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld, stream=s)
+            with pytest.raises(tw.TwError) as e:
+                plan.lstm_steps_status(s)
+            assert e.value.status == tw.ERR_DEVICE
+        finally:
+            tw.set_option(tw.OPT_SPIN_LIMIT, -1)
+        plan.lstm_steps_status(s)                  # the status was cleared by the report
+        dA = to_device_bits(A, A.shape)
+        dC = torch.from_numpy(c.copy()).cuda()
+        plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld, stream=s)
+        plan.lstm_steps_status(s)
+        want_h, want_c = _oracle_recurrence(oracle, W, np.zeros(4 * H, np.float32), tiles, xs, h0, c0, dtype)
+        got = oracle.bits_to_f32(np.ascontiguousarray(from_device_bits(dA)[T, I:, :M]), dtype).reshape(H, M).T
+        assert oracle.rel_error(got, want_h[-1]) <= 2 * TOL[dtype]
+
+
+def test_multi_step_launch_falls_back(tw, oracle):
+    """A plan the persistent kernel does not take (pruned columns) runs step by step through the
+    caller's gate matrix; without one the call fails like tw_lstm_step."""
+    import torch
+    rng = np.random.default_rng(6)
+    M, I, H, G, T, dtype = 64, 64, 128, 128, 3, "f16"
+    K, N, ld = I + H, 4 * H, 64
+    W = (rng.standard_normal((K, N)) * 0.08).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.5, n_keep=0.8)
+    xs = [rng.standard_normal((M, I)).astype(np.float32) for _ in range(T)]
+    h0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    c0 = (rng.standard_normal((M, H)) * 0.5).astype(np.float32)
+    A = np.zeros((T + 1, K, ld), np.uint16)
+    for t in range(T):
+        A[t, :I] = oracle.cast_bits(xs[t], dtype).reshape(M, I).T
+    A[0, I:] = oracle.cast_bits(h0, dtype).reshape(M, H).T
+    s = torch.cuda.current_stream().cuda_stream
+    q = lambda v: oracle.quantize(np.asarray(v, np.float32), dtype).astype(np.float64)
+    mask = oracle.plan_mask(K, N, tiles)
+    with tw.Plan.create(K, N, dtype, tiles, W) as plan:
+        dA = to_device_bits(A, A.shape)
+        dC = torch.from_numpy(np.ascontiguousarray(c0.T)).cuda()
+        dG = torch.zeros((N, ld), dtype=torch.int16, device="cuda")
+        with pytest.raises(tw.TwError) as e:
+            plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), stream=s)
+        assert e.value.status == tw.ERR_LAYOUT
+        plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), gates_ptr=dG.data_ptr(), stream=s)
+        plan.lstm_steps_status(s)
+    h, cc = q(h0), c0.astype(np.float64)
+    for x in xs:
+        gates = oracle.mask_dense(np.concatenate([q(x), h], 1), q(W), mask, np.zeros(N))
+        cc, h = oracle.basic_lstm_cell(q(gates), cc, 1.0)   # the two-kernel form rounds the gate matrix
+        h = q(h)
+    got = oracle.bits_to_f32(np.ascontiguousarray(from_device_bits(dA)[T, I:]), dtype).reshape(H, M).T
+    # (the gate matrix goes through 16 bits here: an absolute error of 2^-11 of a gate's magnitude,
+    # which can be most of a small h, so the bound is absolute: |h| < 1, |c| of order 1)
+    assert np.max(np.abs(got - h)) <= 1e-2
+    assert np.max(np.abs(dC.cpu().numpy().T - cc)) <= 1e-2

@@ -338,6 +338,294 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_step_kernel(const 
     }
 }
 
+
+// ---------------------------------------------------------------------------------
+// T time steps of the LSTM in one launch (tw_lstm_steps): the recurrence of the NMT cells
+// (Pruning/NMT/nmt/model_helper.py:400-402 builds the cell once and dynamic_rnn applies it step
+// after step with the same kernel) as a persistent kernel.  Same decomposition as the single
+// step above (workgroup = 32 hidden units x 32 rows, wave = one gate and every second step of 64
+// kept rows), but the weight fragments, the row offsets, the bias and the cell state of a
+// workgroup are fetched once and stay in registers for all T steps; per step a workgroup reads
+// its rows of A_t = [x_t ; h_(t-1)], multiplies, applies the cell, writes its piece of h_t into
+// the rows of A_(t+1), and meets all other workgroups at a barrier in device memory before it
+// reads the rows of h of A_(t+1).  The rows of x of A_(t+1) do not wait: the steps of a tile's
+// kept rows that hold nothing else are fetched and multiplied while the barrier fills.
+//   coherence: h crosses from one die to another between two steps.  Its stores write through
+//           (sc0 sc1) and the loads of steps that hold rows of h bypass the die's L2 (sc0 sc1), so
+//           no cache is written back or invalidated inside the launch.
+//   barrier: one counter; a workgroup waits for its own stores, adds one and polls until the
+//           counter has reached (t + 1) x workgroups.  The poll is bounded: a workgroup that runs
+//           out of polls (the launch does not fit the chip next to whatever else runs there, so
+//           some workgroup never started) sets the status word and leaves; every other
+//           workgroup then runs out of polls too, and the host reports the launch as failed.
+//   edges:  A_t is addressed through a buffer descriptor; the padding of a list of kept rows and
+//           rows m beyond M get an offset beyond the buffer, for which the hardware delivers
+//           zeros.
+constexpr int kSeqSteps = 4; // steps of 64 kept rows a wave holds in registers: tiles of at most 512 kept rows
+constexpr int kSeqRsrcFlags = 0x00020000;
+constexpr int kSeqAuxCoherent = 1 | 16; // sc0 sc1
+
+struct LstmSeqArgs {
+    const void *A;
+    const int32_t *kept_k;
+    const void *Bp;
+    const float *bias;
+    float *c;
+    int32_t *sync;   // arrivals at the barrier: zero at the start
+    int32_t *status; // set to 1 by a workgroup that gave up
+    int64_t lda, a_step, ldc;
+    int32_t M, H, K, T;
+    float forget_bias;
+    int32_t spin_limit;
+    uint32_t a_bytes; // K * lda * 2
+    int32_t pad_;
+    LstmBlk blk[kLstmMaxBlks];
+};
+static_assert(sizeof(LstmSeqArgs) <= 4096, "kernel arguments");
+
+// RB rows m of A per workgroup (32 is what the launch uses).
+template <int DT, int RB>
+__global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const LstmSeqArgs p)
+{
+    static_assert(RB == 32 || RB == 16, "rows of a workgroup");
+    constexpr int LPS = RB / 8;       // 16-byte loads per lane and step of 64 kept rows
+    constexpr int RPL = kBlockK / LPS; // kept rows a load of the wave covers
+    constexpr int PITCH = RB * 2;     // bytes of a staged row
+    constexpr int STEPB = kBlockK * PITCH;
+    constexpr int RPT = RB / 16;      // rows of a hidden unit a thread applies the cell to
+    __shared__ __align__(16) unsigned char smem[kLstmWaves * kLstmStage];
+    __shared__ int s_ok;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int gate = wave >> 1, kh = wave & 1;
+    const int hb = blockIdx.x, m0 = blockIdx.y * RB;
+    const int n_wgs = gridDim.x * gridDim.y;
+    const LstmBlk blk = p.blk[hb * 4 + gate];
+    const int nsteps = (blk.k_kept + kBlockK - 1) / kBlockK;
+    unsigned char *const stage = smem + wave * kLstmStage;
+
+    // ---- what stays for all T steps: weight fragments and row offsets of this wave's steps
+    // kh, kh + 2, ... (a step the tile does not have repeats the tile's first and is skipped)
+    const int ch = lane % LPS, rowl = lane / LPS; // this lane's 16-byte chunk of a row, its row of a load
+    const bool m_ok = m0 + ch * 8 < p.M;
+    u32x4 bq[kSeqSteps][4];
+    uint32_t voff[kSeqSteps][LPS];
+    {
+        TW_GLOBAL(const unsigned char) const bsrc = (TW_GLOBAL(const unsigned char))p.Bp + blk.b_first + lane * 16;
+        int rows[kSeqSteps][LPS];
+#pragma unroll
+        for (int i = 0; i < kSeqSteps; ++i) {
+            const int s = kh + 2 * i, sc = s < nsteps ? s : 0;
+#pragma unroll
+            for (int k16 = 0; k16 < 4; ++k16)
+                bq[i][k16] = *(TW_GLOBAL(const u32x4))(bsrc + sc * blk.step_b + k16 * 1024);
+#pragma unroll
+            for (int r = 0; r < LPS; ++r)
+                rows[i][r] = p.kept_k[blk.kk_off + sc * kBlockK + r * RPL + rowl]; // the list is padded: in bounds
+        }
+#pragma unroll
+        for (int i = 0; i < kSeqSteps; ++i)
+#pragma unroll
+            for (int r = 0; r < LPS; ++r) {
+                const int kk = (kh + 2 * i) * kBlockK + r * RPL + rowl;
+                voff[i][r] = (kk < blk.k_kept && m_ok)
+                                 ? (uint32_t)rows[i][r] * ((uint32_t)p.lda * 2u) + (uint32_t)(m0 + ch * 8) * 2u
+                                 : 0xFFFFFFF0u;
+            }
+    }
+    const int my_steps = nsteps > kh ? (nsteps - kh + 1) / 2 : 0; // <= kSeqSteps (host check)
+    // The first n_pre of this wave's steps hold rows of x only (a list of kept rows ascends, and
+    // the rows of x come first in A): they do not depend on the step before, so they are fetched
+    // and multiplied while the workgroup waits at the barrier.
+    int n_pre = 0;
+#pragma unroll
+    for (int i = 0; i < kSeqSteps; ++i) {
+        const int s = kh + 2 * i;
+        if (s < nsteps) {
+            const int last = min(s * kBlockK + kBlockK - 1, blk.k_kept - 1);
+            if (n_pre == i && p.kept_k[blk.kk_off + last] < p.K - p.H)
+                n_pre = i + 1;
+        }
+    }
+    n_pre = __builtin_amdgcn_readfirstlane(n_pre);
+    // the cell's share of this thread: RPT rows of hidden unit hb * 32 + tid / 16
+    const int ju = tid >> 4, mt = (tid & 15) * RPT;
+    const int hu = hb * 32 + ju;
+    bool row_ok[RPT];
+#pragma unroll
+    for (int e = 0; e < RPT; ++e)
+        row_ok[e] = m0 + mt + e < p.M;
+    float bias4[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (p.bias) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            bias4[g] = p.bias[g * p.H + hu];
+    }
+    float c2[RPT];
+#pragma unroll
+    for (int e = 0; e < RPT; ++e)
+        c2[e] = row_ok[e] ? p.c[(int64_t)hu * p.ldc + m0 + mt + e] : 0.0f;
+
+    // this lane's place in a staged step for the transposed reads: row (lane / 32) * 8 + L / 4 of a
+    // group of 16 kept rows, 8 bytes at row m (lane / 16 % 2) * 16 + (L % 4) * 4; with 16 rows m
+    // the lanes of the upper 16 read what the lower 16 read (their products are never used)
+    const int L = lane & 15;
+    const int pair_e = (lane >> 5) * 4 + (L >> 2);
+    const int lane_b = (RB == 32 ? ((lane >> 4) & 1) * 32 : 0) + (L & 3) * 8;
+    const uint32_t r_first = (uint32_t)((pair_e >> 2) * 8 + (pair_e & 3));
+    float *const part = reinterpret_cast<float *>(stage);
+    const uint16_t *const A0 = reinterpret_cast<const uint16_t *>(p.A);
+
+    u32x4 av[kSeqSteps][LPS];
+    f32x16 acc;
+    auto clear = [&]() {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+            acc[e] = 0.0f;
+    };
+    // the rows of this wave's steps [lo, hi) of A_t; `coherent`: past the die's L2
+    auto load_steps = [&](int t, int lo, int hi, bool coherent) {
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<uint16_t *>(A0 + (int64_t)t * p.a_step), 0, (int)p.a_bytes, kSeqRsrcFlags);
+#pragma unroll
+        for (int i = 0; i < kSeqSteps; ++i)
+            if (i >= lo && i < hi) {
+#pragma unroll
+                for (int r = 0; r < LPS; ++r)
+                    av[i][r] = coherent ? __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff[i][r], 0, kSeqAuxCoherent))
+                                        : __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, (int)voff[i][r], 0, 0));
+            }
+    };
+    // multiplies them: a step through one half of the wave's stage (the halves in turn, so that a
+    // step's rows are written while the step before is still being read)
+    auto multiply_steps = [&](int lo, int hi) {
+#pragma unroll
+        for (int i = 0; i < kSeqSteps; ++i)
+            if (i >= lo && i < hi) {
+                unsigned char *const half = stage + (i & 1) * STEPB;
+#pragma unroll
+                for (int r = 0; r < LPS; ++r)
+                    *reinterpret_cast<u32x4 *>(half + (r * RPL + rowl) * PITCH + ch * 16) = av[i][r];
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                TW_LDS(unsigned char) lds_lane = (TW_LDS(unsigned char))half + lane_b;
+#pragma unroll
+                for (int k16 = 0; k16 < 4; ++k16) {
+                    const uint32_t r_lo = r_first + k16 * 16, r_hi = r_lo + 4;
+                    const s16x4 lo4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_lo * PITCH));
+                    const s16x4 hi4 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(lds_lane + r_hi * PITCH));
+                    const u32x2 l2 = __builtin_bit_cast(u32x2, lo4), h2 = __builtin_bit_cast(u32x2, hi4);
+                    acc = mfma16<DT>(u32x4{l2.x, l2.y, h2.x, h2.y}, bq[i][k16], acc);
+                }
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+
+    clear();
+    load_steps(0, 0, n_pre, false);
+    multiply_steps(0, n_pre);
+    for (int t = 0; t < p.T; ++t) {
+        // ---- the steps that hold rows of h (of the step before: behind the barrier); the next
+        // step's rows of x leave right behind them, so that one trip to memory covers both
+        load_steps(t, n_pre, my_steps, true);
+        if (t + 1 < p.T)
+            load_steps(t + 1, 0, n_pre, false);
+        multiply_steps(n_pre, my_steps);
+        // the partial product of this wave: column lane % 32, rows r4 * 8 + (lane / 32) * 4 + e
+        // (four rows at a time: they are neighbours in the column, 16-byte aligned)
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int r4 = 0; r4 < RB / 8; ++r4)
+            *reinterpret_cast<f32x4 *>(part + (lane & 31) * kLstmPitch + r4 * 8 + (lane >> 5) * 4) =
+                f32x4{acc[r4 * 4], acc[r4 * 4 + 1], acc[r4 * 4 + 2], acc[r4 * 4 + 3]};
+        __syncthreads();
+        {
+            float pre[4][RPT];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const float *const lo = reinterpret_cast<const float *>(smem + (2 * g) * kLstmStage) + ju * kLstmPitch + mt;
+                const float *const hi = reinterpret_cast<const float *>(smem + (2 * g + 1) * kLstmStage) + ju * kLstmPitch + mt;
+#pragma unroll
+                for (int e = 0; e < RPT; ++e)
+                    pre[g][e] = (lo[e] + hi[e]) + bias4[g];
+            }
+            float h2[RPT];
+#pragma unroll
+            for (int e = 0; e < RPT; ++e)
+                cell_update(pre[0][e], pre[1][e], pre[2][e], pre[3][e], p.forget_bias, c2[e], h2[e]);
+            // h_t into the rows of A_(t+1) that hold h; written through, for the other dies
+            uint16_t *const hdst = const_cast<uint16_t *>(A0) + (int64_t)(t + 1) * p.a_step +
+                                   (int64_t)(p.K - p.H + hu) * p.lda + m0 + mt;
+            if (RPT == 2 && row_ok[RPT - 1]) {
+                const uint32_t w = (uint32_t)to16(h2[0], DT) | ((uint32_t)to16(h2[RPT - 1], DT) << 16);
+                asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(hdst), "v"(w) : "memory");
+            } else if (row_ok[0]) {
+                const uint32_t w = to16(h2[0], DT);
+                asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(hdst), "v"(w) : "memory");
+            }
+        }
+        if (t + 1 == p.T)
+            break;
+        // ---- the barrier between two steps, with the next step's rows of x multiplied on the way
+        clear();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this thread's piece of h is out
+        __syncthreads();                                  // (and the partial sums have been read)
+        if (tid == 0)
+            __hip_atomic_fetch_add(p.sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        multiply_steps(0, n_pre);
+        if (tid == 0) {
+            const int target = (t + 1) * n_wgs;
+            int ok = 0;
+            for (int polls = p.spin_limit; polls > 0; --polls) {
+                if (__hip_atomic_load(p.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target) {
+                    ok = 1;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+            if (!ok)
+                __hip_atomic_store(p.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_ok = ok;
+        }
+        __syncthreads();
+        if (!s_ok)
+            return; // every other workgroup runs out of polls as well: the grid drains
+    }
+#pragma unroll
+    for (int e = 0; e < RPT; ++e)
+        if (row_ok[e])
+            p.c[(int64_t)hu * p.ldc + m0 + mt + e] = c2[e];
+}
+
+__global__ void clear_sync_kernel(int32_t *sync)
+{
+    if (threadIdx.x < 16)
+        sync[threadIdx.x] = 0;
+}
+
+// what tw_lstm_step and tw_lstm_steps have in common: whether the fused kernels take the plan
+bool lstm_fused_plan(const tw_plan *plan, int H)
+{
+    bool fused = H % 32 == 0 && H / 32 * 4 <= kLstmMaxBlks && plan->n_units == plan->n_tiles;
+    for (int t = 0; t < plan->n_tiles && fused; ++t)
+        fused = plan->tile_col0[t] % 32 == 0 && plan->tile_width[t] % 32 == 0 &&
+                plan->kept_n_ptr[t + 1] - plan->kept_n_ptr[t] == plan->tile_width[t];
+    return fused;
+}
+
+void lstm_fill_blocks(const tw_plan *plan, int H, LstmBlk *blk)
+{
+    for (const UnitDev &u : plan->h_units) {
+        // the unit's blocks: columns col0 + 32 nb of C, i.e. gate (col / H), hidden block (col % H) / 32
+        for (int nb = 0; nb < u.nb_cnt; ++nb) {
+            const int col = u.col0 + 32 * nb;
+            LstmBlk &b = blk[(col % H) / 32 * 4 + col / H];
+            b.kk_off = u.kk_off;
+            b.k_kept = u.k_pad ? u.k_kept : 0;
+            b.b_first = u.b_off * 2 + (int64_t)(u.nb0 + nb) * 4096;
+            b.step_b = (int64_t)u.nblk * 4096;
+        }
+    }
+}
 } // namespace
 } // namespace tw
 
@@ -361,10 +649,7 @@ extern "C" int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int
         return fail(TW_ERR_NULL, "A, c_prev, c_new or h_new is NULL");
     // what the fused kernel takes: every column kept, tiles that are whole blocks of 32 columns and
     // one work item each, at most 128 blocks in all
-    bool fused = H % 32 == 0 && H / 32 * 4 <= kLstmMaxBlks && plan->n_units == plan->n_tiles;
-    for (int t = 0; t < plan->n_tiles && fused; ++t)
-        fused = plan->tile_col0[t] % 32 == 0 && plan->tile_width[t] % 32 == 0 &&
-                plan->kept_n_ptr[t + 1] - plan->kept_n_ptr[t] == plan->tile_width[t];
+    const bool fused = lstm_fused_plan(plan, H);
     if (!fused) {
         if (!gates_ws)
             return fail(TW_ERR_LAYOUT, "this plan needs the two-kernel form (pruned columns, tiles that are no "
@@ -410,17 +695,7 @@ extern "C" int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int
     a.H = H;
     a.forget_bias = forget_bias;
     a.pad_ = 0;
-    for (const UnitDev &u : plan->h_units) {
-        // the unit's blocks: columns col0 + 32 nb of C, i.e. gate (col / H), hidden block (col % H) / 32
-        for (int nb = 0; nb < u.nb_cnt; ++nb) {
-            const int col = u.col0 + 32 * nb;
-            LstmBlk &b = a.blk[(col % H) / 32 * 4 + col / H];
-            b.kk_off = u.kk_off;
-            b.k_kept = u.k_pad ? u.k_kept : 0;
-            b.b_first = u.b_off * 2 + (int64_t)(u.nb0 + nb) * 4096;
-            b.step_b = (int64_t)u.nblk * 4096;
-        }
-    }
+    lstm_fill_blocks(plan, H, a.blk);
     if (plan->dtype == TW_F16)
         hipLaunchKernelGGL((tw_lstm_step_kernel<TW_F16>), dim3((unsigned)(H / 32), (unsigned)row_blocks),
                            dim3(64 * kLstmWaves), 0, (hipStream_t)stream, a);
@@ -429,6 +704,107 @@ extern "C" int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int
                            dim3(64 * kLstmWaves), 0, (hipStream_t)stream, a);
     TW_HIP(hipGetLastError());
     return TW_OK;
+}
+
+extern "C" int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, int64_t a_step, int M,
+                             const float *bias, float forget_bias, float *c, int64_t ldc, void *gates_ws,
+                             int64_t ldg, void *stream)
+{
+    if (!plan)
+        return fail(TW_ERR_NULL, "plan is NULL");
+    if (T < 0 || M < 0)
+        return fail(TW_ERR_SHAPE, "T=%d M=%d", T, M);
+    if (plan->N % 4)
+        return fail(TW_ERR_SHAPE, "N=%d is not four gates wide", plan->N);
+    const int H = plan->N / 4, K = plan->K;
+    if (H > K)
+        return fail(TW_ERR_SHAPE, "K=%d has no room for the H=%d rows of h", K, H);
+    if (T == 0 || M == 0)
+        return TW_OK;
+    if (!A || !c)
+        return fail(TW_ERR_NULL, "A or c is NULL");
+    if (lda < M || ldc < M)
+        return fail(TW_ERR_SHAPE, "lda=%lld ldc=%lld must be >= M=%d", (long long)lda, (long long)ldc, M);
+    if (a_step < (int64_t)K * lda)
+        return fail(TW_ERR_SHAPE, "a_step=%lld: consecutive steps' A (K x lda = %lld elements) overlap", (long long)a_step,
+                    (long long)K * lda);
+    if ((lda & 7) || (a_step & 7) || (ldc & 3))
+        return fail(TW_ERR_ALIGNMENT, "lda and a_step must be multiples of 8 elements, ldc of 4");
+    if (((uintptr_t)A & 15) || ((uintptr_t)c & 15))
+        return fail(TW_ERR_ALIGNMENT, "A and c must be 16-byte aligned");
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev != plan->device)
+        return fail(TW_ERR_DEVICE, "the plan was built on device %d, the current device is %d", plan->device, dev);
+    uint16_t *const A16 = static_cast<uint16_t *>(A);
+    // The persistent kernel: a plan the fused step takes, tiles of at most 512 kept rows, a grid
+    // that is resident at once (one workgroup per compute unit), A_t below 4 GiB.  (32 rows of A a
+    // workgroup: with 16, which fills the chip on the NMT cell, a workgroup fetches the same
+    // number of row pieces of half the size, and a step takes 8.5 us instead of 5.9.)
+    const int rb = 32;
+    const int64_t row_blocks = ((int64_t)M + rb - 1) / rb;
+    const bool persistent = lstm_fused_plan(plan, H) && plan->max_k_pad <= 2 * kSeqSteps * kBlockK &&
+                            (int64_t)(H / 32) * row_blocks <= plan->cu_count &&
+                            (uint64_t)K * (uint64_t)lda * 2u < (1ull << 32) && T > 1 && plan->d_tickets;
+    if (!persistent) {
+        // step by step: one launch (or two, through the gate matrix) per time step
+        for (int t = 0; t < T; ++t) {
+            const int rc = tw_lstm_step(plan, A16 + (int64_t)t * a_step, lda, M, bias, forget_bias, c, ldc, c, ldc,
+                                        A16 + (int64_t)(t + 1) * a_step + (int64_t)(K - H) * lda, lda, gates_ws, ldg, stream);
+            if (rc != TW_OK)
+                return rc;
+        }
+        return TW_OK;
+    }
+    LstmSeqArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.A = A;
+    a.kept_k = plan->d_kept_k_pad;
+    a.Bp = plan->d_Bp;
+    a.bias = bias;
+    a.c = c;
+    // a ticket slot of the plan holds the barrier's counter; the word behind the slots its status
+    const unsigned slot = __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kEagerSlots;
+    a.sync = plan->d_tickets + kTicketInts * slot;
+    a.status = plan->d_tickets + kTicketInts * kTicketSlots;
+    a.lda = lda;
+    a.a_step = a_step;
+    a.ldc = ldc;
+    a.M = M;
+    a.H = H;
+    a.K = K;
+    a.T = T;
+    a.forget_bias = forget_bias;
+    const int limit = get_option(TW_OPT_SPIN_LIMIT);
+    a.spin_limit = limit >= 0 ? limit : (1 << 20);
+    a.a_bytes = (uint32_t)((uint64_t)K * (uint64_t)lda * 2u);
+    lstm_fill_blocks(plan, H, a.blk);
+    // (a kernel, not a memset: the call may be recorded into a graph)
+    hipLaunchKernelGGL(clear_sync_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, a.sync);
+    const dim3 grid((unsigned)(H / 32), (unsigned)row_blocks), block(64 * kLstmWaves);
+    if (plan->dtype == TW_F16)
+        hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_F16, 32>), grid, block, 0, (hipStream_t)stream, a);
+    else
+        hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_BF16, 32>), grid, block, 0, (hipStream_t)stream, a);
+    TW_HIP(hipGetLastError());
+    return TW_OK;
+}
+
+extern "C" int tw_lstm_steps_status(const tw_plan *plan, void *stream)
+{
+    if (!plan)
+        return fail(TW_ERR_NULL, "plan is NULL");
+    if (!plan->d_tickets)
+        return TW_OK;
+    int32_t *const word = plan->d_tickets + kTicketInts * kTicketSlots;
+    int32_t v = 0;
+    TW_HIP(hipStreamSynchronize((hipStream_t)stream));
+    TW_HIP(hipMemcpy(&v, word, sizeof v, hipMemcpyDeviceToHost));
+    if (v == 0)
+        return TW_OK;
+    TW_HIP(hipMemset(word, 0, sizeof v));
+    return fail(TW_ERR_DEVICE, "a multi-step LSTM launch of this plan gave up at its barrier (its workgroups were not all "
+                               "resident at once); h and c of that call are undefined");
 }
 
 extern "C" int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg,

@@ -2047,7 +2047,7 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
 static std::atomic<int> g_opt[TW_N_OPTIONS];
 static std::once_flag g_opt_once;
 static const char *const kOptEnv[TW_N_OPTIONS] = {"TWGEMM_SHAPE", "TWGEMM_WGS_PER_CU", "TWGEMM_PIECE",
-                                                  "TWGEMM_XCD_QUEUES"};
+                                                  "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT"};
 
 static bool option_in_range(int option, int value)
 {
@@ -2062,6 +2062,8 @@ static bool option_in_range(int option, int value)
         return value == 32 || value == 64 || value == 128;
     case TW_OPT_XCD_QUEUES:
         return value == 0 || value == 1;
+    case TW_OPT_SPIN_LIMIT:
+        return value >= 0;
     }
     return false;
 }
@@ -2082,6 +2084,8 @@ static int option(int o)
     init_options();
     return g_opt[o].load(std::memory_order_relaxed);
 }
+
+int get_option(int option_id) { return option(option_id); }
 
 static int round_up32(int v) { return (v + 31) / 32 * 32; }
 

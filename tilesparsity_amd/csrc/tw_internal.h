@@ -142,6 +142,7 @@ struct tw_plan {
 namespace tw {
 
 void set_error(const char *fmt, ...);
+int get_option(int option_id); // a tw_set_option value, or -1
 int fail(int status, const char *fmt, ...);
 
 #define TW_HIP(call)                                                                     \

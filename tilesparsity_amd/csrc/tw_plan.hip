@@ -702,7 +702,7 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
         o_rn = put(rel_n.data(), rel_n.size() * sizeof(int32_t));
     }
     const size_t o_tickets = (stage.size() + 255) / 256 * 256;
-    const size_t ticket_bytes = sizeof(int32_t) * kTicketInts * kTicketSlots;
+    const size_t ticket_bytes = sizeof(int32_t) * kTicketInts * (kTicketSlots + 1); // (the last: status words)
     const size_t o_bp = (o_tickets + ticket_bytes + 1023) / 1024 * 1024;
     const size_t bp_bytes = (size_t)std::max<int64_t>(p->packed_elems, 8) * 2;
     char *slab = nullptr;

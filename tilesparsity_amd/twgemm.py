@@ -24,7 +24,7 @@ F16, BF16 = 0, 1
 KMAJOR, ROWMAJOR = 0, 1
 PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
-OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES = 0, 1, 2, 3
+OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES, OPT_SPIN_LIMIT = 0, 1, 2, 3, 4
 SHAPE_AS64, SHAPE_AS32, SHAPE_SKINNY, SHAPE_BS = 7, 8, 9, 10
 SHAPE_WIDE, SHAPE_128x128, SHAPE_512x64, SHAPE_128x64, SHAPE_256x128, SHAPE_128x32, SHAPE_256x64 = range(7)
 
@@ -53,6 +53,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
     "tw_gemm_staged", "tw_gemm_staged_workspace",
     "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm", "tw_plan_reset", "tw_lstm_step",
+    "tw_lstm_steps", "tw_lstm_steps_status",
 )
 
 
@@ -158,6 +159,8 @@ def lib():
         "tw_tiles_from_mask": (c_int, [c_int, c_int, c_int, u8p, i32p, i32p, ctypes.POINTER(c_int)]),
         "tw_plan_reset": (c_int, [vp, vp]),
         "tw_lstm_step": (c_int, [vp, vp, c_i64, c_int, vp, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
+        "tw_lstm_steps": (c_int, [vp, c_int, vp, c_i64, c_i64, c_int, vp, c_f, vp, c_i64, vp, c_i64, vp]),
+        "tw_lstm_steps_status": (c_int, [vp, vp]),
         "tw_side_create": (c_int, [c_int, c_int, c_int, u8p, f32p, pp]),
         "tw_side_destroy": (None, [vp]),
         "tw_side_nnz": (c_i64, [vp]),
@@ -397,6 +400,22 @@ class Plan:
                                   forget_bias, vp(int(c_prev_ptr or 0)), ld(ldc_prev),
                                   vp(int(c_new_ptr or 0)), ld(ldc_new), vp(int(h_new_ptr or 0)), ld(ldh),
                                   vp(int(gates_ptr or 0)), ld(ldg), vp(int(stream or 0))))
+
+    def lstm_steps(self, T, A_ptr, M, c_ptr, lda=None, a_step=None, ldc=None, bias_ptr=None, forget_bias=1.0,
+                   gates_ptr=None, ldg=None, stream=0):
+        """T LSTM time steps on T + 1 K-major matrices A_t = [x_t ; h_(t-1)] at a_step elements from
+        each other (see tw_lstm_steps): one persistent launch where the plan and the chip allow it,
+        else T calls of tw_lstm_step.  Asynchronous; lstm_steps_status() tells whether it completed."""
+        vp = ctypes.c_void_p
+        lda = M if lda is None else lda
+        a_step = self.K * lda if a_step is None else a_step
+        _check(lib().tw_lstm_steps(self._h, T, vp(int(A_ptr or 0)), lda, a_step, M, vp(int(bias_ptr or 0)),
+                                   forget_bias, vp(int(c_ptr or 0)), M if ldc is None else ldc,
+                                   vp(int(gates_ptr or 0)), M if ldg is None else ldg, vp(int(stream or 0))))
+
+    def lstm_steps_status(self, stream=0):
+        """Waits for the stream; raises TwError(ERR_DEVICE) if a persistent lstm_steps launch gave up."""
+        _check(lib().tw_lstm_steps_status(self._h, ctypes.c_void_p(int(stream or 0))))
 
     def reset(self, stream=0):
         """Re-arms the plan's work-queue counters (after a launch of it was aborted mid-flight)."""

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the tile-wise-sparse GEMM engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--headline-only]
 
 A step is one TW GEMM  C = A * (B (.) mask)  over one batch of synthetic input that
 is already resident in HBM.  The default workload is VGG16 conv4_2 as an im2col GEMM
@@ -26,15 +26,16 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 
 # HBM bytes per sparse launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
 # dispatch), each scaled by what the same counter reads for a 256 MiB copy in the same run
-# (reads x 2.0, writes x 1.0); the runs and their commands are in profiles/tw_gemm_*_kernel__*.md,
-# one file per workload.  Keyed by the workload's own name.
-MEASURED_TRAFFIC_BYTES = {
-    "vgg16_conv4_2_im2col": (2 * 62061 + 11410) * 1024,
-    "bert_base_ffn_in": (2 * 7897 + 24576) * 1024,
-    "nmt_lstm_gates": (2 * 3558.5 + 1024) * 1024,
-    "imbalance_stress": (2 * 908806 + 212608) * 1024,
-    "bert_large_ffn1_keep25": (2 * 16649 + 65536) * 1024,
-    "bert_large_ffn2_keep25": (2 * 38143 + 16400) * 1024,
+# (reads x 2.0, writes x 1.0).  Constants copied from the profile named beside them, not read in
+# this run: `traffic_source` in the line says which file, and for which kernel, they stand.
+# Keyed by the workload's own name.
+MEASURED_TRAFFIC = {
+    "vgg16_conv4_2_im2col": ((2 * 62061 + 11410) * 1024, "profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md (tw_gemm_ws_kernel 256x128)"),
+    "bert_base_ffn_in": ((2 * 7897 + 24576) * 1024, "profiles/tw_gemm_as_kernel__bert_base_ffn.md (tw_gemm_as_kernel 64 rows)"),
+    "nmt_lstm_gates": ((2 * 3558.5 + 1024) * 1024, "profiles/tw_gemm_skinny_kernel__nmt_lstm_gates.md (tw_gemm_skinny_kernel)"),
+    "imbalance_stress": ((2 * 908806 + 212608) * 1024, "profiles/tw_gemm_ws_kernel__imbalance_stress.md (tw_gemm_ws_kernel 512x64)"),
+    "bert_large_ffn1_keep25": ((2 * 16649 + 65536) * 1024, "profiles/tw_gemm_as_kernel__bert_large_ffn1.md (tw_gemm_as_kernel 64 rows)"),
+    "bert_large_ffn2_keep25": ((2 * 38143 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
 }
 
 
@@ -230,7 +231,7 @@ def time_nmt_recurrence(wl, steps, torch):
     return out[0], out[1], out[2], out[3]
 
 
-def roofline_of(M, K, N, tiles, t, traffic=None):
+def roofline_of(M, K, N, tiles, t, traffic=None, traffic_source=None):
     """Roofline block of one launch that took t seconds: the binding roof is the larger of the
     ideal HBM time (algorithmic bytes at 8 TB/s) and the ideal MFMA time (kept flops at the dense
     16-bit peak)."""
@@ -239,10 +240,23 @@ def roofline_of(M, K, N, tiles, t, traffic=None):
     if by / (HBM_PEAK_GBS * 1e9) >= fk / (MFMA_PEAK_TFLOPS * 1e12):
         ach = by / t / 1e9
         return {"bound": "hbm", "achieved": ach, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": ach / HBM_PEAK_GBS, "traffic": traffic, "algorithmic_bytes": by}
+                "frac": ach / HBM_PEAK_GBS, "traffic": traffic, "traffic_source": traffic_source,
+                "algorithmic_bytes": by}
     ach = fk / t / 1e12
     return {"bound": "mfma", "achieved": ach, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-            "frac": ach / MFMA_PEAK_TFLOPS, "traffic": traffic, "algorithmic_flops": fk}
+            "frac": ach / MFMA_PEAK_TFLOPS, "traffic": traffic, "traffic_source": traffic_source,
+            "algorithmic_flops": fk}
+
+
+def traffic_of(name, kernel):
+    """(bytes, source) of the committed counter measurement of a workload, or (None, None) when
+    there is none or the launch now runs another kernel than the one that was measured."""
+    if name not in MEASURED_TRAFFIC:
+        return None, None
+    by, src = MEASURED_TRAFFIC[name]
+    if "(%s)" % kernel not in src:
+        return None, "%s: measured on another kernel than this launch's %s" % (src, kernel)
+    return by, src
 
 
 def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, graph=False,
@@ -264,6 +278,7 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
             for i in range(n_sets)]
     sparse = tw.Plan.create(K, N, dtype, tiles, B)
     dense = tw.Plan.dense(K, N, G, dtype, B)
+    kernel_sparse, kernel_dense = sparse.choice(M)["name"], dense.choice(M)["name"]
     timer = time_plan_graph if graph else time_plan
     t_sparse = timer(sparse, bufs, M, steps, warmup, torch)
     reps_sparse = [timer(sparse, bufs, M, steps, 2, torch) for _ in range(repeats)]
@@ -295,8 +310,8 @@ def run_workload(wl, steps, warmup, torch, rotate_bytes=768 << 20, repeats=5, gr
         mfma_util_kept=fk / t_sparse / 1e12 / MFMA_PEAK_TFLOPS,
         mfma_util_dense_run=fd / t_de / 1e12 / MFMA_PEAK_TFLOPS,
         algorithmic_bytes=by, hbm_gbs=by / t_sparse / 1e9, rotating_buffer_sets=n_sets,
-        kept_flops=fk, dense_flops=fd,
-        roofline=roofline_of(M, K, N, tiles, t_sparse, MEASURED_TRAFFIC_BYTES.get(wl["name"])))
+        kept_flops=fk, dense_flops=fd, kernel_sparse=kernel_sparse, kernel_dense_plan=kernel_dense,
+        roofline=roofline_of(M, K, N, tiles, t_sparse, *traffic_of(wl["name"], kernel_sparse)))
     if two:
         # independent launches on two streams in turn (throughput, see time_plan_streams)
         res["two_streams"] = dict(us_sparse=two[0] * 1e6, us_dense_plan=two[1] * 1e6,
@@ -581,7 +596,8 @@ def main():
                          "other target shapes and the two-stream leg)")
     ap.add_argument("--two-streams", action="store_true",
                     help="also time independent launches issued on two streams in turn")
-    ap.add_argument("--all", action="store_true", help="also run the other configurations")
+    ap.add_argument("--all", action="store_true", help="(kept for old command lines: every configuration runs by default)")
+    ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--producers", action="store_true",
                     help="benchmark the TW mask producers instead of the GEMM (one JSON line)")
@@ -657,6 +673,7 @@ def main():
         "us_sparse": res["us_sparse"], "us_sparse_median": res["us_sparse_median"],
         "us_dense": res["us_dense"], "us_dense_library": res["us_dense_library"],
         "repeats_for_medians": res["repeats"],
+        "kernel_sparse": res["kernel_sparse"], "kernel_dense_plan": res["kernel_dense_plan"],
         "roofline": roof,
     }
     if "two_streams" in res:
@@ -664,24 +681,25 @@ def main():
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wl, A, B)
     del A, B
-    # the other shapes the target names: BERT-base FFN (small K per tile) and the NMT gate GEMM
-    # (skinny M; its 50 time steps are recorded into a graph and replayed), each with the
-    # roofline of its own launch; --all adds the remaining configurations
-    names = ["bert_base_ffn", "nmt_lstm_gates"]
-    if args.all:
-        names += ["bert_large_ffn1_50", "bert_large_ffn1_75", "bert_large_ffn1_90",
-                  "bert_large_ffn2_50", "bert_large_ffn2_75", "bert_large_ffn2_90", "imbalance_stress"]
-    if args.workload != "vgg16_conv4_2":
+    # the other configurations: BERT-base FFN (small K per tile), the NMT gate GEMM (skinny M; its
+    # 50 time steps are recorded into a graph and replayed), the BERT-large FFN pair at three
+    # sparsities and the imbalance stress shape, each with the roofline of its own launch and the
+    # names of the kernels its sparse and its 0 %-sparse plan ran
+    names = ["bert_base_ffn", "nmt_lstm_gates", "bert_large_ffn1_50", "bert_large_ffn1_75", "bert_large_ffn1_90",
+             "bert_large_ffn2_50", "bert_large_ffn2_75", "bert_large_ffn2_90", "imbalance_stress"]
+    if args.workload != "vgg16_conv4_2" or args.headline_only:
         names = []
     others = {}
     for name in names:
         nmt = name == "nmt_lstm_gates"
-        r, _ = run_workload(make_workload(name), 50 if nmt else args.steps, args.warmup, torch,
-                            repeats=3, graph=nmt, two_streams=two_streams)
+        big = name == "imbalance_stress"   # (launches of 0.3 - 1.5 ms: fewer of them)
+        r, _ = run_workload(make_workload(name), 50 if nmt else (min(args.steps, 30) if big else args.steps),
+                            args.warmup, torch, repeats=3, graph=nmt, two_streams=two_streams and not big)
         others[name] = {k: r[k] for k in ("us_sparse", "us_sparse_median", "us_dense",
                                           "us_dense_library", "effective_tflops", "actual_tflops",
                                           "speedup_vs_dense", "speedup_vs_dense_library",
-                                          "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "roofline")}
+                                          "mfma_util_kept", "hbm_gbs", "dtype", "timed_with", "kernel_sparse",
+                                          "kernel_dense_plan", "roofline")}
         if "two_streams" in r:
             others[name]["independent_launches_on_two_streams"] = r["two_streams"]
         if name == "bert_base_ffn":

@@ -318,6 +318,11 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_SHAPE_SKINNY 9  /* 64 rows x 32 columns per workgroup, the kept rows split over its waves: few rows of A */
 #define TW_SHAPE_BS 10     /* weight-stationary: a unit's packed weight in registers, A streamed: tiles of at most 192 kept rows, beta == 0 */
 #define TW_N_SHAPES 11
+/* What a K-major launch of `plan` on M rows would run with, under the options in force:
+ * choice[0] the TW_SHAPE_* kernel, [1] the columns of a unit piece, [2] workgroups per compute
+ * unit, [3] 1 for one work queue per die.  (No counterpart in the reference, whose kernel is
+ * fixed at compile time, basic_nn.cu:250-259; benchmarks name the kernel they timed with it.) */
+int tw_gemm_choice(const tw_plan *plan, int M, int64_t lda, int64_t ldc, float beta, int32_t *choice);
 int tw_set_option(int option, int value);
 
 /* One-shot drop-in for Stream_Gemm_NN (basic_nn.cu:378-393), same argument

@@ -53,6 +53,28 @@ def test_plan_from_mask_bit_exact(tw, oracle, K, N, G, dtype):
         check_export(oracle, plan, expect, B, dtype)
 
 
+@pytest.mark.parametrize("name", ["vgg16_conv4_2", "imbalance_stress"])
+def test_plan_from_mask_full_size_configurations(tw, oracle, name):
+    """The mask -> kept lists -> relative offsets -> compaction pre-pass at the full size of the
+    benchmark configurations, from the 0/1 mask of the configuration's tile table (VGG16 conv4_2:
+    4608 x 512, ragged kept-row counts, 13 of 128 columns pruned a tile; imbalance stress:
+    4096 x 8192, tiles of 64 columns from empty to dense): tile table, kept lists, relative offsets
+    and the compacted 16-bit weight in the reference's stream layout (basic_nn.cu:697-769), bit
+    for bit against the oracle on the same seed."""
+    from tilesparsity_amd import workloads
+    wl = workloads.vgg16_conv4_2() if name == "vgg16_conv4_2" else workloads.imbalance_stress()
+    K, N, G, dtype, tiles = wl["K"], wl["N"], wl["G"], wl["dtype"], wl["tiles"]
+    _, B = wl["values"]()
+    mask = oracle.plan_mask(K, N, tiles)
+    expect = oracle.plan_from_mask(mask, G)   # what a mask can hold: empty tiles lose their lists
+    assert sum(len(t["kept_k"]) * len(t["kept_n"]) for t in expect) == int(mask.sum())
+    print("full-size pre-pass:", name, K, N, G, dtype, flush=True)
+    with tw.Plan.from_mask(mask, G, dtype, B) as plan:
+        check_export(oracle, plan, expect, B, dtype)
+        inf = plan.info()
+        assert inf["kept_elems"] == int(mask.sum()) and inf["total_width"] == N
+
+
 def test_plan_from_mask_rejects_non_tw_mask(tw):
     K, N, G = 64, 128, 32
     mask = np.zeros((K, N), np.uint8)

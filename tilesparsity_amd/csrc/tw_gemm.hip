@@ -2227,14 +2227,9 @@ bool takes_row_major_directly(const tw_plan *plan, float beta)
 
 template <int DT, int BMS, bool RM> static int launch_as(const tw_plan *plan, const GemmArgs &a, int M, hipStream_t s)
 {
-    static std::once_flag once;
-    static hipError_t attr_err = hipSuccess;
-    std::call_once(once, [] {
-        attr_err = hipFuncSetAttribute((const void *)tw_gemm_as_kernel<DT, BMS, RM>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes);
-    });
-    if (attr_err != hipSuccess)
-        return fail(TW_ERR_DEVICE, "hipFuncSetAttribute failed: %s", hipGetErrorString(attr_err));
+    const int pst = prepare_device();
+    if (pst != TW_OK)
+        return pst;
     const int n_mblk = (M + BMS - 1) / BMS;
     // as many groups as keep every compute unit at one workgroup, each wave with a block or more
     const int per_wg = as_task_waves(BMS, RM);
@@ -2274,6 +2269,47 @@ using namespace tw;
 constexpr int kStaticScratchInts = 64; // 256 bytes, of which kTicketInts counters are used
 static_assert(kStaticScratchInts >= kTicketInts, "the counters of a launch fit the static scratch");
 static __device__ __align__(256) int32_t scratch[kStaticScratchInts];
+
+namespace tw {
+
+namespace {
+constexpr int kMaxDevices = 64;
+int32_t *g_scratch_ptr[kMaxDevices] = {};
+} // namespace
+
+// Once per device: the set-up a launch needs that may not run while a stream is being captured
+// (symbol look-up, function attributes).  Every plan runs it when it is built, so a caller that
+// records launches into a graph has it behind them; the launch paths call it again for the
+// devices no plan was built on, where it costs one flag load.
+int prepare_device()
+{
+    static std::mutex mu;
+    static std::atomic<bool> ready[kMaxDevices];
+    int dev = -1;
+    TW_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices)
+        return fail(TW_ERR_DEVICE, "device %d: the library serves devices 0..%d", dev, kMaxDevices - 1);
+    if (ready[dev].load(std::memory_order_acquire))
+        return TW_OK;
+    std::lock_guard<std::mutex> lock(mu);
+    if (ready[dev].load(std::memory_order_relaxed))
+        return TW_OK;
+    const void *as_kernels[] = {
+        (const void *)tw_gemm_as_kernel<TW_F16, 64, false>,  (const void *)tw_gemm_as_kernel<TW_F16, 32, false>,
+        (const void *)tw_gemm_as_kernel<TW_F16, 64, true>,   (const void *)tw_gemm_as_kernel<TW_F16, 32, true>,
+        (const void *)tw_gemm_as_kernel<TW_BF16, 64, false>, (const void *)tw_gemm_as_kernel<TW_BF16, 32, false>,
+        (const void *)tw_gemm_as_kernel<TW_BF16, 64, true>,  (const void *)tw_gemm_as_kernel<TW_BF16, 32, true>,
+    };
+    for (const void *k : as_kernels)
+        TW_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsBytes));
+    void *p = nullptr;
+    TW_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = static_cast<int32_t *>(p);
+    ready[dev].store(true, std::memory_order_release);
+    return TW_OK;
+}
+
+} // namespace tw
 
 extern "C" {
 
@@ -2426,29 +2462,21 @@ __global__ void clear_all_slots_kernel(int32_t *tickets)
         tickets[i] = 0;
 }
 
-// Device address of `scratch` on the current device, looked up once per device (the array's name
-// is only a host-side stand-in; every GPU holds its own copy at its own address).
+// Device address of `scratch` on the current device (the array's name is only a host-side
+// stand-in; every GPU holds its own copy at its own address), looked up by prepare_device.
 int static_scratch(int32_t **out)
 {
-    constexpr int kMaxDevices = 64;
-    static std::mutex mu;
-    static int32_t *ptr[kMaxDevices] = {};
+    const int st = prepare_device();
+    if (st != TW_OK)
+        return st;
     int dev = -1;
     TW_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= kMaxDevices)
-        return fail(TW_ERR_DEVICE, "device %d: tw_gemm_static serves devices 0..%d", dev, kMaxDevices - 1);
-    std::lock_guard<std::mutex> lock(mu);
-    if (!ptr[dev]) {
-        void *p = nullptr;
-        TW_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
-        ptr[dev] = static_cast<int32_t *>(p);
-    }
-    *out = ptr[dev];
+    *out = g_scratch_ptr[dev];
     return TW_OK;
 }
 
-// tw_gemm_ex and tw_gemm_static: the latter brings the counters (`static_ticket`), cleared on the
-// stream before the launch; the former takes a ticket slot of the plan.
+// tw_gemm_ex and tw_gemm_static: the latter brings the counters (the library's `scratch` array),
+// cleared on the stream before the launch; the former takes a ticket slot of the plan.
 int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C, int c_layout,
               int64_t ldc, int M, float alpha, float beta, int pruned_cols, const tw_epilogue *ep,
               void *stream, bool use_static)
@@ -2545,6 +2573,20 @@ int tw_gemm_ex(const tw_plan *plan, const void *A, int a_layout, int64_t lda, vo
 {
     return gemm_impl(plan, A, a_layout, lda, C, c_layout, ldc, M, alpha, beta, pruned_cols, ep, stream,
                      false);
+}
+
+int tw_gemm_choice(const tw_plan *plan, int M, int64_t lda, int64_t ldc, float beta, int32_t *choice)
+{
+    if (!plan || !choice)
+        return fail(TW_ERR_NULL, "plan or choice is NULL");
+    if (M < 0)
+        return fail(TW_ERR_SHAPE, "M=%d is negative", M);
+    const Choice c = choose_shape(plan, M, lda, ldc, beta != 0.0f);
+    choice[0] = c.shape;
+    choice[1] = c.piece;
+    choice[2] = c.per_cu;
+    choice[3] = c.xcd ? 1 : 0;
+    return TW_OK;
 }
 
 int tw_plan_reset(tw_plan *plan, void *stream)

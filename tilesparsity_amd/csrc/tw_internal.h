@@ -133,8 +133,7 @@ struct tw_plan {
     mutable unsigned next_slot = 0, next_capture_slot = 0;
     int blocks_per_unit = 0; // 32-column blocks of every unit where all units have the same number, else 0
     int n_halves = 0;   // pieces of 64 compact columns over all units (the skinny kernel's work per row block)
-    int mean_steps = 0; // mean number of 64-row steps of the units that have any
-    bool rows_shared = false; // nearly every tile keeps nearly every row (a dense or almost dense plan)
+    bool rows_shared = false; // the tiles that keep rows keep nearly all of them (a dense or almost dense plan)
     int max_k_pad = 0;        // most kept rows of a tile, rounded up to whole steps
     int cu_count = 0;
 };

@@ -625,15 +625,15 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
     p->n_units = (int)units.size();
     p->h_units = units;
     p->n_pipe_units = 0;
-    int64_t steps = 0;
-    for (const UnitDev &u : units) {
+    for (const UnitDev &u : units)
         p->n_pipe_units += u.k_pad > 0;
-        steps += u.k_pad / kBlockK;
-    }
-    p->mean_steps = p->n_pipe_units ? (int)(steps / p->n_pipe_units) : 0;
-    // (kept rows summed over the tiles that have any, against all rows for each of them)
-    p->rows_shared = nt > 1 && p->n_pipe_units > 0 &&
-                     (int64_t)p->kept_k_idx.size() * 10 >= (int64_t)p->K * nt * 9;
+    // nearly dense: kept rows summed over the tiles that keep any, against all K rows for each of
+    // those tiles (a tile pruned away whole takes no part on either side)
+    int64_t tiles_with_rows = 0;
+    for (int t = 0; t < nt; ++t)
+        tiles_with_rows += p->kept_k_ptr[t + 1] > p->kept_k_ptr[t];
+    p->rows_shared = tiles_with_rows > 1 && p->n_pipe_units > 0 &&
+                     (int64_t)p->kept_k_idx.size() * 10 >= (int64_t)p->K * tiles_with_rows * 9;
     p->n_zero_tiles = (int)ztiles.size();
     p->max_k_pad = 0;
     for (const UnitDev &u : units)

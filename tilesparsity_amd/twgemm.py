@@ -27,6 +27,10 @@ ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
 OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES, OPT_SPIN_LIMIT = 0, 1, 2, 3, 4
 SHAPE_AS64, SHAPE_AS32, SHAPE_SKINNY, SHAPE_BS = 7, 8, 9, 10
 SHAPE_WIDE, SHAPE_128x128, SHAPE_512x64, SHAPE_128x64, SHAPE_256x128, SHAPE_128x32, SHAPE_256x64 = range(7)
+SHAPE_NAMES = ("tw_gemm_kmajor_kernel 256x128", "tw_gemm_ws_kernel 128x128", "tw_gemm_ws_kernel 512x64",
+               "tw_gemm_ws_kernel 128x64", "tw_gemm_ws_kernel 256x128", "tw_gemm_ws_kernel 128x32",
+               "tw_gemm_ws_kernel 256x64", "tw_gemm_as_kernel 64 rows", "tw_gemm_as_kernel 32 rows",
+               "tw_gemm_skinny_kernel", "tw_gemm_bs_kernel")
 
 
 class Epilogue(ctypes.Structure):
@@ -53,7 +57,7 @@ EXPORTED_SYMBOLS = (
     "tw_prune_mix", "tw_lstm_gates", "tw_plan_from_device_mask", "tw_set_option", "tw_gemm_static",
     "tw_gemm_staged", "tw_gemm_staged_workspace",
     "tw_side_create", "tw_side_destroy", "tw_side_nnz", "tw_side_gemm", "tw_plan_reset", "tw_lstm_step",
-    "tw_lstm_steps", "tw_lstm_steps_status",
+    "tw_lstm_steps", "tw_lstm_steps_status", "tw_gemm_choice",
 )
 
 
@@ -161,6 +165,7 @@ def lib():
         "tw_lstm_step": (c_int, [vp, vp, c_i64, c_int, vp, c_f, vp, c_i64, vp, c_i64, vp, c_i64, vp, c_i64, vp]),
         "tw_lstm_steps": (c_int, [vp, c_int, vp, c_i64, c_i64, c_int, vp, c_f, vp, c_i64, vp, c_i64, vp]),
         "tw_lstm_steps_status": (c_int, [vp, vp]),
+        "tw_gemm_choice": (c_int, [vp, c_int, c_i64, c_i64, c_f, i32p]),
         "tw_side_create": (c_int, [c_int, c_int, c_int, u8p, f32p, pp]),
         "tw_side_destroy": (None, [vp]),
         "tw_side_nnz": (c_i64, [vp]),
@@ -416,6 +421,14 @@ class Plan:
     def lstm_steps_status(self, stream=0):
         """Waits for the stream; raises TwError(ERR_DEVICE) if a persistent lstm_steps launch gave up."""
         _check(lib().tw_lstm_steps_status(self._h, ctypes.c_void_p(int(stream or 0))))
+
+    def choice(self, M, lda=None, ldc=None, beta=0.0):
+        """The kernel a K-major launch on M rows would run: dict(shape, name, piece, per_cu, xcd_queues)."""
+        out = np.zeros(4, np.int32)
+        _check(lib().tw_gemm_choice(self._h, M, M if lda is None else lda, M if ldc is None else ldc, beta,
+                                    _ptr(out, ctypes.c_int32)))
+        return dict(shape=int(out[0]), name=SHAPE_NAMES[int(out[0])], piece=int(out[1]), per_cu=int(out[2]),
+                    xcd_queues=bool(out[3]))
 
     def reset(self, stream=0):
         """Re-arms the plan's work-queue counters (after a launch of it was aborted mid-flight)."""

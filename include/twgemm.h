@@ -218,8 +218,14 @@ int tw_plan_destroy(tw_plan *plan);
  *   M          rows of A and C; 0 is a no-op
  *   beta       C is read only when beta != 0, and only on kept columns
  *   pruned_cols  tw_pruned_cols
- * Immutable plan: may be called concurrently from several host threads on
- * distinct streams (up to 256 launches of one plan in flight at once). */
+ * Immutable plan: may be called concurrently from several host threads on distinct streams.  A
+ * launch of a kernel that draws work from a queue holds one of the plan's 256 counter slots
+ * until it ends: eager launches rotate over 192 of them, launches made while their stream is
+ * being captured over the other 64 (a recorded launch keeps its slot for every replay).  So at
+ * most 192 eager launches of one plan may be in flight at once, and at most 64 recorded launches
+ * of one plan may run at the same time as each other.  Nothing checks this: launch number 193
+ * (recorded: 65) shares the counters of a launch that has not ended, and both skip or repeat work
+ * items - wrong results, no error.  Synchronise or build a second plan before going beyond. */
 int tw_gemm(const tw_plan *plan, const void *A, int a_layout, int64_t lda,
             void *C, int c_layout, int64_t ldc, int M, float alpha, float beta,
             int pruned_cols, void *stream);
@@ -262,7 +268,10 @@ int tw_plan_reset(tw_plan *plan, void *stream);
  *   is refused with TW_ERR_SHAPE, as it is by tw_gemm_ex; devices 0..63.
  *   Every call on one GPU shares that GPU's counters: calls that overlap on one GPU (two streams,
  *   two host threads, a graph replay next to an eager call) race and give wrong results.
- *   Serialise them, or use tw_gemm_ex, whose plans carry 256 counter slots of their own. */
+ *   Serialise them, or use tw_gemm_ex, whose plans carry 256 counter slots of their own (192 for
+ *   eager launches, 64 for recorded ones; see tw_gemm).
+ *   The once-per-device set-up (the array's device address, kernel attributes) runs when a plan is
+ *   built, so a call made while `stream` is being captured does nothing capture forbids. */
 int tw_gemm_static(const tw_plan *plan, const void *A, int a_layout, int64_t lda, void *C,
                    int c_layout, int64_t ldc, int M, float alpha, float beta, int pruned_cols,
                    const tw_epilogue *ep, void *stream);

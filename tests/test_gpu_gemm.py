@@ -508,10 +508,14 @@ def test_stream_gemm_nn_drop_in(tw, oracle):
         assert np.array_equal(Bs, from_device_bits(dB))
 
 
-def test_graph_capture_replays_bitwise(tw, oracle):
+@pytest.mark.parametrize("forced", ["auto", "streaming"])
+def test_graph_capture_replays_bitwise(tw, oracle, forced):
     """tw_gemm allocates nothing, clears nothing from the host and re-arms its work queue inside
     the kernel, so a sequence of launches can be captured into a HIP graph; every replay (with
-    eager launches and synchronisations in between) gives the eager result bit for bit."""
+    eager launches and synchronisations in between) gives the eager result bit for bit.  Once with
+    the kernel the launch picks by itself (none that uses the queue at this size) and once with a
+    streaming kernel forced, whose recorded launches keep a ticket slot of the plan's captured
+    range across the replays and re-arm it each time."""
     import torch
     rng = np.random.default_rng(77)
     M, K, N, G = 384, 256, 512, 128
@@ -523,28 +527,40 @@ def test_graph_capture_replays_bitwise(tw, oracle):
     dH = torch.zeros((N, M), dtype=torch.int16, device="cuda")
     dC = torch.zeros((N, M), dtype=torch.int16, device="cuda")
     s = torch.cuda.Stream()
-    with tw.Plan.create(K, N, "f16", tiles, B) as plan:
-        def chain():
-            # two dependent launches: C = A (B.mask), then C += 0.5 * A (B.mask) on top of it
-            plan.gemm(dA.data_ptr(), dH.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO, stream=s.cuda_stream)
-            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=0.5, beta=0.0, pruned_cols=tw.PRUNED_ZERO,
-                      stream=s.cuda_stream)
-            plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=1.0, beta=1.0, stream=s.cuda_stream)
-        with torch.cuda.stream(s):
-            chain()
-            s.synchronize()
-            want_h, want_c = dH.clone(), dC.clone()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=s):
+    try:
+        if forced == "streaming":
+            tw.set_option(tw.OPT_SHAPE, tw.SHAPE_128x64)
+            tw.set_option(tw.OPT_PIECE, 64)
+            tw.set_option(tw.OPT_XCD_QUEUES, 1)
+        with tw.Plan.create(K, N, "f16", tiles, B) as plan:
+            if forced == "streaming":
+                assert plan.choice(M)["shape"] == tw.SHAPE_128x64
+
+            def chain():
+                # two dependent launches: C = A (B.mask), then C += 0.5 * A (B.mask) on top of it
+                plan.gemm(dA.data_ptr(), dH.data_ptr(), M, pruned_cols=tw.PRUNED_ZERO, stream=s.cuda_stream)
+                plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=0.5, beta=0.0, pruned_cols=tw.PRUNED_ZERO,
+                          stream=s.cuda_stream)
+                plan.gemm(dA.data_ptr(), dC.data_ptr(), M, alpha=1.0, beta=1.0, stream=s.cuda_stream)
+            with torch.cuda.stream(s):
+                print("graph capture", forced, flush=True)
                 chain()
-            for rep in range(4):
-                dH.fill_(0x1234)
-                dC.fill_(0x1234)
-                plan.gemm(dA.data_ptr(), dH.data_ptr(), M, stream=s.cuda_stream)   # eager work between replays
                 s.synchronize()
-                g.replay()
-                s.synchronize()
-                assert torch.equal(dH, want_h) and torch.equal(dC, want_c), rep
+                want_h, want_c = dH.clone(), dC.clone()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=s):
+                    chain()
+                for rep in range(4):
+                    dH.fill_(0x1234)
+                    dC.fill_(0x1234)
+                    plan.gemm(dA.data_ptr(), dH.data_ptr(), M, stream=s.cuda_stream)   # eager work between replays
+                    s.synchronize()
+                    g.replay()
+                    s.synchronize()
+                    assert torch.equal(dH, want_h) and torch.equal(dC, want_c), rep
+    finally:
+        for opt in (tw.OPT_SHAPE, tw.OPT_PIECE, tw.OPT_XCD_QUEUES):
+            tw.set_option(opt, -1)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
@@ -650,6 +666,63 @@ def test_a_stationary_shapes(tw, oracle, dtype):
                     assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
     finally:
         tw.set_option(tw.OPT_SHAPE, -1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_256x64_shape_epilogues(tw, oracle, dtype):
+    """The 256 x 64 streaming shape (64-wide tiles of plans with few items) with every epilogue:
+    alpha / beta, bias + activation, filled pruned columns, both queue layouts and both piece
+    widths it takes: bit for bit what the 128 x 64 shape gives (same step order over k, same
+    epilogue code), within tolerance of the oracle, nothing written past M."""
+    import torch
+    rng = np.random.default_rng(6464)
+    M, K, N, G = 777, 300, 320, 64
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.1).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tiles = random_tiles(rng, K, N, G, k_keep=0.4, n_keep=0.8)
+    keep = kept_columns(tiles, N)
+    dbias = torch.from_numpy(bias).cuda()
+    lda = ldc = round_up(M, 8) + 8
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    dA = to_device_bits(At, At.shape)
+
+    def launch(plan, shape, piece, xcd, alpha, beta, pruned, with_bias, act):
+        Cb = np.full((N, ldc), SENTINEL, np.uint16)
+        Cb[:, :M] = oracle.cast_bits(C0, dtype).reshape(M, N).T
+        dC = to_device_bits(Cb, Cb.shape)
+        tw.set_option(tw.OPT_SHAPE, shape)
+        tw.set_option(tw.OPT_PIECE, piece)
+        tw.set_option(tw.OPT_XCD_QUEUES, xcd)
+        print("256x64 test: shape", shape, piece, xcd, alpha, beta, pruned, with_bias, act, dtype, flush=True)
+        assert plan.choice(M, lda, ldc, beta)["shape"] == shape
+        plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
+                  pruned_cols=pruned, bias_ptr=dbias.data_ptr() if with_bias else None, activation=act,
+                  stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return from_device_bits(dC)
+
+    try:
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            for (alpha, beta, pruned, with_bias, act) in (
+                    (1.0, 0.0, tw.PRUNED_UNTOUCHED, False, tw.ACT_NONE),
+                    (0.5, 0.0, tw.PRUNED_ZERO, True, tw.ACT_RELU),
+                    (1.0, 0.0, tw.PRUNED_ZERO, True, tw.ACT_GELU),
+                    (2.0, 0.75, tw.PRUNED_ZERO, False, tw.ACT_NONE)):
+                want = launch(plan, tw.SHAPE_128x64, -1, 0, alpha, beta, pruned, with_bias, act)
+                for piece, xcd in ((-1, 0), (-1, 1), (32, 0), (32, 1)):
+                    got = launch(plan, tw.SHAPE_256x64, piece, xcd, alpha, beta, pruned, with_bias, act)
+                    assert np.array_equal(got, want), (piece, xcd, alpha, beta, pruned, with_bias, act)
+                assert (want[:, M:] == SENTINEL).all()
+                if not with_bias and act == tw.ACT_NONE:
+                    Cf = oracle.bits_to_f32(want[:, :M], dtype).reshape(N, M).T
+                    ref = reference(oracle, A, B, tiles, dtype, alpha, beta, C0)
+                    assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
+    finally:
+        for opt in (tw.OPT_SHAPE, tw.OPT_PIECE, tw.OPT_XCD_QUEUES):
+            tw.set_option(opt, -1)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

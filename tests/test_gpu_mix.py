@@ -175,7 +175,7 @@ def _mixed_layer(rng, twprune, K, N, G, sparsity, g1, structured):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
-@pytest.mark.parametrize("M", [200, 513])
+@pytest.mark.parametrize("M", [200, 513, 2100, 4300])
 def test_side_kernel_runs_the_remainder(tw, twprune, po, oracle, dtype, M):
     """TW plan of the first stage's mask + tw_side_gemm on what the second stage adds = the masked
     layer A (B (.) mask) of the mixed mask.  The two passes round their results to 16 bits one
@@ -184,7 +184,9 @@ def test_side_kernel_runs_the_remainder(tw, twprune, po, oracle, dtype, M):
     the GEMM tolerance of the float64 products of the 16-bit operands on that scale.  The side
     call alone adds exactly the remainder's product (checked against a launch on zeros, one
     rounding: plain relative error), leaves columns without remainder elements and the padding
-    beyond M untouched, and repeats bit for bit."""
+    beyond M untouched, and repeats bit for bit.  A die takes whole 256-row chunks in rounds of
+    eight and the chunks left over are shared: M = 200 and 513 have left-over chunks only, 2100
+    (nine chunks) one round and one left over, 4300 (seventeen) two rounds and one left over."""
     import torch
     from tests.test_gpu_gemm import to_device_bits, from_device_bits, round_up, SENTINEL
     rng = np.random.default_rng(77 + M)

@@ -141,7 +141,10 @@ struct tw_plan {
 namespace tw {
 
 void set_error(const char *fmt, ...);
-int get_option(int option_id); // a tw_set_option value, or -1
+int get_option(int option_id);
+// once per device: symbol look-ups and function attributes, which HIP refuses while a stream is
+// being captured; run by every plan when it is built and again (one flag load) by the launches
+int prepare_device(); // a tw_set_option value, or -1
 int fail(int status, const char *fmt, ...);
 
 #define TW_HIP(call)                                                                     \

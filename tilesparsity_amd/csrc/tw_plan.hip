@@ -555,6 +555,9 @@ struct PlanOwner {
 
 int finalize_plan_geometry(tw_plan *p, hipStream_t s)
 {
+    const int dst = prepare_device();
+    if (dst != TW_OK)
+        return dst;
     const int nt = p->n_tiles;
     p->k_pad.assign(nt, 0);
     p->n_pad.assign(nt, 0);

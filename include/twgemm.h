@@ -314,7 +314,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_PIECE 2
 #define TW_OPT_XCD_QUEUES 3
 #define TW_OPT_SPIN_LIMIT 4 /* polls a workgroup of tw_lstm_steps spends at a barrier before it gives up (default 2^20) */
-#define TW_N_OPTIONS 5
+#define TW_OPT_BALANCE 5 /* 0: every tile in row blocks of the kernel's full height; automatic (1): a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows) */
+#define TW_N_OPTIONS 6
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
 #define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns */

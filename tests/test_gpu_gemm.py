@@ -588,7 +588,7 @@ def test_every_kernel_shape_agrees(tw, oracle, dtype):
             keep = kept_columns(tiles, N)
             with tw.Plan.create(K, N, dtype, tiles, B) as plan:
                 for shape, piece in combos:
-                    for xcd in (1, 0):
+                    for xcd in (1, 0, 2):
                         tw.set_option(tw.OPT_SHAPE, shape)
                         tw.set_option(tw.OPT_PIECE, piece)
                         tw.set_option(tw.OPT_XCD_QUEUES, xcd)
@@ -666,6 +666,64 @@ def test_a_stationary_shapes(tw, oracle, dtype):
                     assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
     finally:
         tw.set_option(tw.OPT_SHAPE, -1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+def test_row_blocks_sized_per_tile(tw, oracle, dtype):
+    """A launch whose items would not fill the chip once gives the tiles with more kept rows lower
+    row blocks (multiples of 64 rows).  Tiles of 40 to 900 kept rows, one without any, ragged M,
+    pruned columns filled, bias + activation, beta: every streaming shape gives the same bits with
+    TW_OPT_BALANCE 0 and 1 and stays within tolerance of the oracle; nothing is written past M."""
+    import torch
+    rng = np.random.default_rng(8086)
+    M, K, N, G = 5003, 1000, 640, 128
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    C0 = rng.standard_normal((M, N)).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tiles = []
+    for t, (kt, nt) in enumerate(((900, 128), (40, 100), (0, 128), (333, 128), (520, 77))):
+        tiles.append(dict(col0=t * G, width=G,
+                          kept_k=np.sort(rng.choice(K, size=kt, replace=False)).astype(np.int32),
+                          kept_n=np.sort(rng.choice(G, size=nt, replace=False)).astype(np.int32)))
+    keep = kept_columns(tiles, N)
+    dbias = torch.from_numpy(bias).cuda()
+    lda = ldc = round_up(M, 8) + 8
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    dA = to_device_bits(At, At.shape)
+
+    def launch(plan, shape, balance, alpha, beta, pruned, with_bias, act):
+        Cb = np.full((N, ldc), SENTINEL, np.uint16)
+        Cb[:, :M] = oracle.cast_bits(C0, dtype).reshape(M, N).T
+        dC = to_device_bits(Cb, Cb.shape)
+        tw.set_option(tw.OPT_SHAPE, shape)
+        tw.set_option(tw.OPT_BALANCE, balance)
+        print("row blocks per tile: shape", shape, balance, alpha, beta, pruned, with_bias, act, dtype, flush=True)
+        plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, alpha=alpha, beta=beta,
+                  pruned_cols=pruned, bias_ptr=dbias.data_ptr() if with_bias else None, activation=act,
+                  stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return from_device_bits(dC)
+
+    try:
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            for (alpha, beta, pruned, with_bias, act) in (
+                    (1.0, 0.0, tw.PRUNED_UNTOUCHED, False, tw.ACT_NONE),
+                    (0.5, 0.0, tw.PRUNED_ZERO, True, tw.ACT_RELU),
+                    (2.0, 0.75, tw.PRUNED_ZERO, False, tw.ACT_NONE)):
+                for shape in (tw.SHAPE_256x128, tw.SHAPE_128x128):
+                    want = launch(plan, shape, 0, alpha, beta, pruned, with_bias, act)
+                    got = launch(plan, shape, 1, alpha, beta, pruned, with_bias, act)
+                    assert np.array_equal(got, want), (shape, alpha, beta, pruned, with_bias, act)
+                    assert (got[:, M:] == SENTINEL).all()
+                    if not with_bias and act == tw.ACT_NONE:
+                        Cf = oracle.bits_to_f32(got[:, :M], dtype).reshape(N, M).T
+                        ref = reference(oracle, A, B, tiles, dtype, alpha, beta, C0)
+                        assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
+    finally:
+        tw.set_option(tw.OPT_SHAPE, -1)
+        tw.set_option(tw.OPT_BALANCE, -1)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])

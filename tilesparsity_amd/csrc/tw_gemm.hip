@@ -42,7 +42,8 @@ enum ItemKind { ITEM_PIPE = 0, ITEM_NOSTEP = 1, ITEM_ZERO = 2, ITEM_END = 3 };
 struct Work {
     int kind; // ItemKind
     int u;    // column of the item matrix: piece of a unit, or n_gemm_u + tile to fill
-    int mb;   // row block
+    int m0;   // first row
+    int rows; // rows [m0, m0 + rows) of A and C, cut at M by the caller
 };
 
 __device__ __forceinline__ int queue_length(const GemmArgs &p, int x)
@@ -50,22 +51,41 @@ __device__ __forceinline__ int queue_length(const GemmArgs &p, int x)
     return p.n_own_items + (p.n_tail_items > x ? (p.n_tail_items - x + kXcd - 1) / kXcd : 0);
 }
 
-__device__ __forceinline__ Work queue_entry(const GemmArgs &p, int x, int q)
+// (bm: rows of a row block of this launch)
+__device__ __forceinline__ Work queue_entry(const GemmArgs &p, int x, int q, int bm)
 {
     Work w;
     w.kind = ITEM_END;
     w.u = 0;
-    w.mb = 0;
+    w.m0 = 0;
+    w.rows = bm;
     if (q < p.n_own_items) {
         const int i = q / p.n_all_u;
         w.u = q - i * p.n_all_u;
-        w.mb = x * p.n_own + i;
+        w.m0 = (x * p.n_own + i) * bm;
     } else {
         const int j = (q - p.n_own_items) * kXcd + x;
         if (j >= p.n_tail_items)
             return w;
-        w.u = j / p.n_tail_mblk;
-        w.mb = kXcd * p.n_own + (j - w.u * p.n_tail_mblk);
+        if (p.n_bal > 0) {
+            // columns with row blocks of their own height: column u owns the items
+            // bal_first[u] .. bal_first[u + 1] - 1 of the list
+            int u = 0;
+#pragma unroll
+            for (int i = 1; i < kBalColumns; ++i)
+                u += i < p.n_bal && j >= p.bal_first[i];
+            w.u = u;
+            w.rows = p.bal_rows[u];
+            w.m0 = (j - p.bal_first[u]) * w.rows;
+        } else if (p.rb_major) {
+            // all columns of a row block (heaviest first) before the next row block
+            const int mb = j / p.n_all_u;
+            w.u = j - mb * p.n_all_u;
+            w.m0 = (kXcd * p.n_own + mb) * bm;
+        } else {
+            w.u = j / p.n_tail_mblk;
+            w.m0 = (kXcd * p.n_own + (j - w.u * p.n_tail_mblk)) * bm;
+        }
     }
     w.kind = w.u < p.n_pipe_u ? ITEM_PIPE : (w.u < p.n_gemm_u ? ITEM_NOSTEP : ITEM_ZERO);
     return w;
@@ -132,9 +152,9 @@ __global__ void __launch_bounds__(64 * WM * WN, (WM * WN * WGS) / 4)
     };
     auto make_item = [&](int ticket) {
         Item it;
-        const Work w = queue_entry(p, qx, ticket);
+        const Work w = queue_entry(p, qx, ticket, BM);
         it.col = w.kind == ITEM_END ? p.n_all_u : w.u;
-        it.m0 = w.mb * BM;
+        it.m0 = w.m0;
         if (it.col < p.n_gemm_u)
             it.u = load_unit(p, it.col);
         return it;
@@ -573,10 +593,10 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
     };
     auto make_item = [&](int ticket) {
         Item it;
-        const Work w = queue_entry(p, qx, ticket);
+        const Work w = queue_entry(p, qx, ticket, BM);
         it.col = w.kind == ITEM_END ? p.n_all_u : w.u;
-        it.m0 = w.mb * BM;
-        it.m_end = it.m0 + BM < p.M ? it.m0 + BM : p.M;
+        it.m0 = w.m0;
+        it.m_end = it.m0 + w.rows < p.M ? it.m0 + w.rows : p.M;
         if (it.col < p.n_gemm_u)
             it.u = load_unit(p, it.col);
         return it;
@@ -663,9 +683,9 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
             const int c = t.col0 + p.pruned_n[t.pn_off + j];
             uint16_t *dst = C + (int64_t)c * p.ldc + m;
             u32x4 v = {0u, 0u, 0u, 0u};
-            if ((p.beta != 0.0f || p.bias || p.act) && m < p.M) {
+            if ((p.beta != 0.0f || p.bias || p.act) && m < it.m_end) {
                 uint32_t w[4] = {0u, 0u, 0u, 0u};
-                for (int e = 0; e < 8 && m + e < p.M; ++e) {
+                for (int e = 0; e < 8 && m + e < it.m_end; ++e) {
                     const float old = p.beta != 0.0f ? p.beta * E::from_bits(dst[e]) : 0.0f;
                     w[e >> 1] |= E::to_bits(tw_finish(old, p.bias, c, p.act)) << ((e & 1) * 16);
                 }
@@ -674,7 +694,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                 v.z = w[2];
                 v.w = w[3];
             }
-            store_chunk(dst, v, m, p.M, p.store_through != 0);
+            store_chunk(dst, v, m, it.m_end, p.store_through != 0);
         }
     };
     // scatters the staged C tile (all threads): whole columns col0 + kept_n[j], 16-byte stores
@@ -2047,7 +2067,7 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
 static std::atomic<int> g_opt[TW_N_OPTIONS];
 static std::once_flag g_opt_once;
 static const char *const kOptEnv[TW_N_OPTIONS] = {"TWGEMM_SHAPE", "TWGEMM_WGS_PER_CU", "TWGEMM_PIECE",
-                                                  "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT"};
+                                                  "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT", "TWGEMM_BALANCE"};
 
 static bool option_in_range(int option, int value)
 {
@@ -2061,9 +2081,11 @@ static bool option_in_range(int option, int value)
     case TW_OPT_PIECE:
         return value == 32 || value == 64 || value == 128;
     case TW_OPT_XCD_QUEUES:
-        return value == 0 || value == 1;
+        return value >= 0 && value <= 2;
     case TW_OPT_SPIN_LIMIT:
         return value >= 0;
+    case TW_OPT_BALANCE:
+        return value == 0 || value == 1;
     }
     return false;
 }
@@ -2395,6 +2417,8 @@ void fill_common(GemmArgs &a, const tw_plan *plan, const void *A, int64_t lda, v
     a.act = ep ? ep->activation : TW_ACT_NONE;
     a.store_through = 0;
     a.ticket = nullptr;
+    a.n_bal = 0;
+    a.rb_major = 0;
     a.n_arg_units = 0;
 }
 
@@ -2415,6 +2439,62 @@ void fill_queues(GemmArgs &a, const tw_plan *plan, int M, int bm, int piece, int
     a.n_own_items = a.n_own * a.n_all_u;
     a.n_tail_mblk = a.n_mblk - kXcd * a.n_own;
     a.n_tail_items = a.n_tail_mblk * a.n_all_u;
+}
+
+// Row blocks sized per column of the item matrix, for launches whose items do not fill the chip
+// once: with whole row blocks the launch lasts as long as an item of the tile with the most kept
+// rows, next to idle compute units and to items that end early.  Column u gets row blocks of
+// h_u rows, a multiple of 64 (whole 128-byte lines of a K-major row of 16-bit elements, whole
+// multiplying waves) of at most bm, so that steps_u * h_u is as even as the items allow while
+// all of them still fit the chip at once.  Returns false (and leaves `a` alone) where that gains
+// nothing: one column, every column at full height, more items than workgroups.
+bool balance_items(GemmArgs &a, const tw_plan *plan, int M, int bm, int64_t wgs)
+{
+    if (a.n_split != 1 || a.n_own != 0 || a.n_all_u > kBalColumns || a.n_pipe_u < 2 || bm < 128)
+        return false;
+    int steps[kBalColumns];
+    for (int u = 0; u < a.n_all_u; ++u)
+        steps[u] = u < a.n_pipe_u ? plan->h_units[u].k_pad / kBlockK : 0;
+    auto items_at = [&](int64_t cost, int32_t *rows) {
+        int64_t n = 0;
+        for (int u = 0; u < a.n_all_u; ++u) {
+            int h = bm;
+            if (steps[u] > 0)
+                h = (int)std::min<int64_t>(bm, std::max<int64_t>(64, cost / steps[u] / 64 * 64));
+            rows[u] = h;
+            n += (M + h - 1) / h;
+        }
+        return n;
+    };
+    // candidate costs: every steps_u * h; the smallest whose items fit
+    int64_t best = 0;
+    int32_t rows[kBalColumns], best_rows[kBalColumns];
+    for (int u = 0; u < a.n_pipe_u; ++u)
+        for (int h = 64; h <= bm; h += 64) {
+            const int64_t cost = (int64_t)steps[u] * h;
+            if ((best == 0 || cost < best) && items_at(cost, rows) <= wgs) {
+                best = cost;
+                std::copy(rows, rows + a.n_all_u, best_rows);
+            }
+        }
+    if (best == 0)
+        return false;
+    bool shorter = false;
+    for (int u = 0; u < a.n_pipe_u; ++u)
+        shorter |= best_rows[u] < bm;
+    if (!shorter)
+        return false;
+    a.n_bal = a.n_all_u;
+    int32_t first = 0;
+    for (int u = 0; u < a.n_all_u; ++u) {
+        a.bal_first[u] = first;
+        a.bal_rows[u] = best_rows[u];
+        first += (M + best_rows[u] - 1) / best_rows[u];
+    }
+    for (int u = a.n_all_u; u <= kBalColumns; ++u)
+        a.bal_first[u] = first;
+    a.n_tail_items = first;
+    return true;
 }
 
 // launches the K-major kernels with the counters at `ticket` (kTicketInts zeros)
@@ -2530,6 +2610,9 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
 
     const Choice c = choose_shape(plan, M, lda, ldc, beta != 0.0f);
     fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
+    a.rb_major = option(TW_OPT_XCD_QUEUES) == 2;
+    if (c.shape != TW_SHAPE_WIDE && !is_queueless_shape(c.shape) && option(TW_OPT_BALANCE) != 0)
+        balance_items(a, plan, M, kShapes[c.shape].bm, (int64_t)plan->cu_count * c.per_cu);
     if ((int64_t)a.n_all_u * a.n_mblk > kMaxItems)
         return fail(TW_ERR_SHAPE, "%lld work items (M=%d): a launch takes at most %lld",
                     (long long)a.n_all_u * a.n_mblk, M, (long long)kMaxItems);

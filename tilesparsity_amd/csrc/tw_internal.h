@@ -23,6 +23,7 @@ constexpr int kMaxUnitN = 128; // compact columns handled by one work item
 constexpr int kTicketSlots = 256;
 constexpr int kEagerSlots = 192;  // slots of eager launches; the rest serve launches recorded in graphs
 constexpr int kMaxArgUnits = 32;
+constexpr int kBalColumns = 8; // columns of the item matrix that may have row blocks of their own height
 
 // One schedulable piece of a tile: at most kMaxUnitN compact columns.
 // 48 bytes; read with scalar loads.
@@ -91,6 +92,13 @@ struct GemmArgs {
     int32_t act;          // TW_ACT_*
     int32_t store_through; // output stores write through to memory (large outputs) or stay in L2
     int32_t *ticket;      // kTicketInts counters, zero between launches
+    // Row blocks sized per column of the item matrix (n_bal > 0: one list of items for all
+    // queues, n_own == 0, n_tail_items items): column u has items of bal_rows[u] rows, the items
+    // bal_first[u] .. bal_first[u + 1] - 1 of the list.  See balance_items.
+    int32_t n_bal;
+    int32_t rb_major;     // the items no queue owns are dealt out row block after row block instead of column after column
+    int32_t bal_first[kBalColumns + 1];
+    int32_t bal_rows[kBalColumns];
     // Copy of `units` inside the kernel arguments for plans of at most kMaxArgUnits units
     // (n_arg_units == 0 otherwise): a workgroup then reads its first unit through the scalar
     // cache instead of waiting for a global load before it can fetch anything else.

@@ -306,7 +306,9 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  *   TW_OPT_XCD_QUEUES   1: one work queue per accelerator die, each owning whole row blocks of A
  *                       (the workgroups of a die then share those rows in their L2);
  *                       0: the work items are dealt out over the dies in turn; automatic: 0
- *                       unless nearly every tile keeps nearly every row (a 0 %-sparse plan)
+ *                       unless nearly every tile keeps nearly every row (a 0 %-sparse plan);
+ *                       2: dealt out over the dies in turn, row block after row block (all tiles
+ *                       of a row block before the next) instead of tile after tile
  * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
  * TWGEMM_PIECE and TWGEMM_XCD_QUEUES, read once. */
 #define TW_OPT_SHAPE 0
@@ -314,7 +316,7 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_PIECE 2
 #define TW_OPT_XCD_QUEUES 3
 #define TW_OPT_SPIN_LIMIT 4 /* polls a workgroup of tw_lstm_steps spends at a barrier before it gives up (default 2^20) */
-#define TW_OPT_BALANCE 5 /* 0: every tile in row blocks of the kernel's full height; automatic (1): a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows) */
+#define TW_OPT_BALANCE 5 /* 1: a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows); 0 and automatic: every tile in row blocks of the kernel's full height (the benchmark shapes run no faster with 1) */
 #define TW_N_OPTIONS 6
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */

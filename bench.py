@@ -30,11 +30,12 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 # this run: `traffic_source` in the line says which file, and for which kernel, they stand.
 # Keyed by the workload's own name.
 MEASURED_TRAFFIC = {
-    "vgg16_conv4_2_im2col": ((2 * 62061 + 11410) * 1024, "profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md (tw_gemm_ws_kernel 256x128)"),
+    "vgg16_conv4_2_im2col": ((2 * 62054 + 11282) * 1024, "profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md (tw_gemm_ws_kernel 256x128)"),
     "bert_base_ffn_in": ((2 * 7897 + 24576) * 1024, "profiles/tw_gemm_as_kernel__bert_base_ffn.md (tw_gemm_as_kernel 64 rows)"),
     "nmt_lstm_gates": ((2 * 3558.5 + 1024) * 1024, "profiles/tw_gemm_skinny_kernel__nmt_lstm_gates.md (tw_gemm_skinny_kernel)"),
     "imbalance_stress": ((2 * 908806 + 212608) * 1024, "profiles/tw_gemm_ws_kernel__imbalance_stress.md (tw_gemm_ws_kernel 512x64)"),
     "bert_large_ffn1_keep25": ((2 * 16649 + 65536) * 1024, "profiles/tw_gemm_as_kernel__bert_large_ffn1.md (tw_gemm_as_kernel 64 rows)"),
+    "bert_large_ffn1_keep10": ((2 * 12319 + 65536) * 1024, "profiles/tw_gemm_bs_kernel__bert_large_ffn1_90.md (tw_gemm_bs_kernel)"),
     "bert_large_ffn2_keep25": ((2 * 38143 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
 }
 
@@ -599,6 +600,9 @@ def main():
     ap.add_argument("--all", action="store_true", help="(kept for old command lines: every configuration runs by default)")
     ap.add_argument("--headline-only", action="store_true", help="skip the other configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--rows", type=int, default=None,
+                    help="launch the configuration's plan on its first ROWS rows of A only (how long "
+                         "an item takes with few of them on the chip); implies --headline-only")
     ap.add_argument("--producers", action="store_true",
                     help="benchmark the TW mask producers instead of the GEMM (one JSON line)")
     ap.add_argument("--prepass", action="store_true",
@@ -654,6 +658,14 @@ def main():
 
     two_streams = args.two_streams or full_report
     wl = make_workload(args.workload)
+    if args.rows is not None:
+        if not 0 < args.rows <= wl["M"]:
+            print("bench.py: --rows must be in 1 .. %d" % wl["M"], file=sys.stderr)
+            return 2
+        full_values, rows = wl["values"], args.rows
+        wl = dict(wl, M=rows, values=lambda: (lambda ab: (np.ascontiguousarray(ab[0][:rows]), ab[1]))(full_values()))
+        args.headline_only = True
+        two_streams = args.two_streams
     res, (A, B) = run_workload(wl, args.steps, args.warmup, torch, two_streams=two_streams)
     roof = dict(res["roofline"])
     out = {

@@ -317,7 +317,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_XCD_QUEUES 3
 #define TW_OPT_SPIN_LIMIT 4 /* polls a workgroup of tw_lstm_steps spends at a barrier before it gives up (default 2^20) */
 #define TW_OPT_BALANCE 5 /* 1: a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows); 0 and automatic: every tile in row blocks of the kernel's full height (the benchmark shapes run no faster with 1) */
-#define TW_N_OPTIONS 6
+#define TW_OPT_LDS_DMA 6 /* the 256-row streaming kernels (256 x 128, 256 x 64) with loads that write LDS directly: 0 never; 1 and automatic: wherever those shapes run */
+#define TW_N_OPTIONS 7
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
 #define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns */

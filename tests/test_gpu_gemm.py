@@ -597,8 +597,15 @@ def test_every_kernel_shape_agrees(tw, oracle, dtype):
                         C2, bits2 = run_gemm(tw, oracle, plan, A, dtype, N)
                         assert oracle.rel_error(C1[:, keep], ref[:, keep]) <= TOL[dtype], (shape, piece)
                         assert np.array_equal(bits1, bits2), (shape, piece)
+                        if shape in (S4, S6):
+                            # the 256-row kernels load straight into LDS by default; their
+                            # register-staged form gives the same bits
+                            tw.set_option(tw.OPT_LDS_DMA, 0)
+                            C3, bits3 = run_gemm(tw, oracle, plan, A, dtype, N)
+                            tw.set_option(tw.OPT_LDS_DMA, -1)
+                            assert np.array_equal(bits1, bits3), (shape, piece, "register-staged")
     finally:
-        for opt in (tw.OPT_SHAPE, tw.OPT_PIECE, tw.OPT_XCD_QUEUES):
+        for opt in (tw.OPT_SHAPE, tw.OPT_PIECE, tw.OPT_XCD_QUEUES, tw.OPT_LDS_DMA):
             tw.set_option(opt, -1)
 
 

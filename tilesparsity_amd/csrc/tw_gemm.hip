@@ -537,7 +537,7 @@ template <int NRD, int NMM, int I, bool READS> __device__ __forceinline__ void s
 //   BM = 512: 4 + 4 waves, each multiplying wave 128 rows (tiles of at most 64 kept columns).
 // The first loads of the next item are issued during the last step of the current one and
 // fly over its epilogue.
-template <int DT, int BM, int BN, int R>
+template <int DT, int BM, int BN, int R, bool DMA = false>
 __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(const GemmArgs p)
 {
     constexpr int NMW = BM == 128 ? 2 : 4;     // multiplying waves, and as many moving waves
@@ -554,10 +554,25 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
     constexpr int PASSES = RPW / RG;           // A loads per moving thread and step
     constexpr int BPASS = BN * BK / 8 / NPM;   // weight loads per moving thread and step
     constexpr int PITCH = BM + TW_A_PAD;
-    constexpr int ASTAGE = BK * PITCH, BSTAGE = BN * BK;
+    // DMA: the moving waves issue loads that write LDS directly.  A load of a wave (64 lanes x 16
+    // bytes) lands as 1 KB in one piece, so a stage of A is 32 slots of two rows of the step (the
+    // rows mw * 16 + ps and + 8 of moving wave mw's load ps: what one transposed read's lanes
+    // 0 - 31 and 32 - 63 address), 64 bytes of padding behind each slot so that the four slots a
+    // transposed read touches fall into four different groups of 16 banks; three stages, since a
+    // stage is written by loads issued two steps ahead instead of passing through registers.
+    constexpr int SLOTB = 1024 + 64; // bytes
+    constexpr int NST = DMA ? 3 : 2;
+    constexpr int ASTAGE = DMA ? (BK / 2) * SLOTB / 2 : BK * PITCH, BSTAGE = BN * BK;
     constexpr int CPITCH = BM + 4;
-    constexpr int PIPE = 2 * (ASTAGE + BSTAGE);
-    constexpr int SMEM = PIPE > BN * CPITCH ? PIPE : BN * CPITCH;
+    constexpr int PIPE = NST * (ASTAGE + BSTAGE);
+    // DMA: the stages lie one behind the other, each its rows of A followed by its weight, and the
+    // C tile of an item is staged 64 columns at a time in the stage its last step was multiplied
+    // from, so that the other two can already receive the first steps of the workgroup's next item
+    constexpr int STG = ASTAGE + BSTAGE;
+    constexpr int CROUNDS = DMA ? BN / 64 : 1;
+    static_assert(!DMA || 64 * CPITCH <= STG, "64 columns of the C tile fit one stage");
+    constexpr int SMEM = DMA ? PIPE : (PIPE > BN * CPITCH ? PIPE : BN * CPITCH);
+    static_assert(!DMA || BM == 256, "the direct-to-LDS form is laid out for 256-row items");
     static_assert(BK == kBlockK && KS == PKS, "one packed weight step per main-loop step");
     static_assert(CPR <= 64 && PASSES % 4 == 0 && BPASS >= 1 && BN <= NPM, "tile shape");
     using E = Elem<DT>;
@@ -572,8 +587,9 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
     const uint16_t *const A = reinterpret_cast<const uint16_t *>(p.A);
     uint16_t *const C = reinterpret_cast<uint16_t *>(p.C);
     const uint16_t *const Bp = reinterpret_cast<const uint16_t *>(p.Bp);
+    // (DMA: stage i holds its rows of A at sA + i * STG and its weight at sB + i * STG)
     uint16_t *const sA = smem;
-    uint16_t *const sB = smem + 2 * ASTAGE;
+    uint16_t *const sB = DMA ? smem + ASTAGE : smem + NST * ASTAGE;
 
     // this workgroup's queue
     const int qx = blockIdx.x % kXcd;
@@ -715,7 +731,202 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         }
     };
 
-    if (wave >= NMW) {
+    // (DMA) scatters round rd of a C tile staged at `ctile`: 64 columns at most.  By the multiplying
+    // waves alone where the moving waves are already loading the workgroup's next item (they must
+    // not have stores among their loads), else by all waves.
+    auto store_round = [&](const uint16_t *ctile, int rd, const UnitDev &u, int m0, int m_end, bool all) {
+        const int m_st = m0 + (tid % CPR) * 8;
+        const int jn = u.n_cnt - rd * 64 < 64 ? u.n_cnt - rd * 64 : 64;
+        for (int j = tid / CPR; j < jn; j += (all ? NT : NPM) / CPR) {
+            const int c = s_cols[rd * 64 + j];
+            const u32x2 lo = *reinterpret_cast<const u32x2 *>(ctile + j * CPITCH + (tid % CPR) * 8);
+            const u32x2 hi = *reinterpret_cast<const u32x2 *>(ctile + j * CPITCH + (tid % CPR) * 8 + 4);
+            u32x4 v;
+            v.x = lo.x;
+            v.y = lo.y;
+            v.z = hi.x;
+            v.w = hi.y;
+            store_chunk(C + (int64_t)c * p.ldc + m_st, v, m_st, m_end, p.store_through != 0);
+        }
+    };
+
+    if (wave >= NMW && DMA) {
+        // ================= moving waves, loads straight into LDS ===========================
+        // Lane (g, chunk) of moving wave mw fetches chunk `chunk` (8 consecutive m) of the kept
+        // rows mw * 16 + g * 8 + ps, ps = 0 .. 7, of a step: load ps of the wave fills slot
+        // mw * 8 + ps of the stage.  A row past the tile's list, a chunk past the item's rows and
+        // every load of a step past the item's last get an offset beyond the buffer and arrive
+        // as zeros.  Step j + 1 is issued in time slot j (its stage was multiplied two slots
+        // ago), step j is waited for at the slot's end: two steps in flight.  Every slot issues
+        // the same loads in the same order, so the waits are exact counts: behind the loads of
+        // step j are the two index loads and the twelve loads of the slot that follows.
+        if constexpr (DMA) {
+        constexpr uint32_t kGone = 0xFFFFFFF0u;
+        const int chunk = lane % CPR, g = lane / CPR;
+        const int mw = wave - NMW;
+        const int row0 = mw * RPW + g * PASSES;
+        const uint32_t lda_b = (uint32_t)p.lda * 2u;
+        typedef int i32x4 __attribute__((ext_vector_type(4)));
+        struct Idx {
+            i32x4 k[PASSES / 4];
+        };
+        const __amdgpu_buffer_rsrc_t a_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.A), 0, (int)p.a_bytes, 0x00020000);
+        const __amdgpu_buffer_rsrc_t b_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(p.Bp), 0, (int)p.b_bytes, 0x00020000);
+        TW_LDS(unsigned char) const lds_a = (TW_LDS(unsigned char))sA + mw * (PASSES * SLOTB);
+        TW_LDS(unsigned char) const lds_b = (TW_LDS(unsigned char))sB + mw * 1024;
+        // what the loads of an item's steps need
+        struct Ctx {
+            const char *k_base;
+            uint32_t m0b, b_pack_b;
+            uint32_t b_blk[BPASS]; // weight block of load bp (a block beyond the unit reads block 0), bytes into Bp
+            int k_left0, nsteps;
+            bool m_ok;
+        };
+        auto ctx_of = [&](const Item &it) {
+            Ctx c;
+            c.k_base = reinterpret_cast<const char *>(p.kept_k + it.u.kk_off) + row0 * 4;
+            c.m0b = (uint32_t)it.m0 * 2u;
+            c.m_ok = it.m0 + chunk * 8 < it.m_end;
+            c.k_left0 = it.u.k_kept - row0;
+            c.nsteps = it.u.k_pad / BK;
+#pragma unroll
+            for (int bp = 0; bp < BPASS; ++bp)
+                c.b_blk[bp] = (uint32_t)(it.u.b_off * 2) + (uint32_t)(it.u.nb0 + (bp < it.u.nb_cnt ? bp : 0)) * 4096u + mw * 1024u;
+            c.b_pack_b = (uint32_t)it.u.nblk * (PKS * 64 * 8 * 2);
+            return c;
+        };
+        auto load_idx = [&](const Ctx &c, int st, Idx &ix) { // (the list is padded: always in bounds)
+#pragma unroll
+            for (int i = 0; i < PASSES / 4; ++i)
+                ix.k[i] = *reinterpret_cast<const i32x4 *>(c.k_base + (int64_t)st * (BK * 4) + 16 * i);
+        };
+        // the BPASS + PASSES loads of step st of an item into stage `stage`
+        auto issue = [&](const Ctx &c, int st, int stage, const Idx &ix) {
+            const bool real = st < c.nsteps;
+            const uint32_t vb = real ? (uint32_t)lane * 16u : kGone;
+            const uint32_t sb = (real ? (uint32_t)st : 0u) * c.b_pack_b;
+#pragma unroll
+            for (int bp = 0; bp < BPASS; ++bp)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(b_rsrc, (TW_LDS(void))(lds_b + stage * (STG * 2) + bp * 4096),
+                                                         16, (int)vb, (int)(c.b_blk[bp] + sb), 0, 0);
+            const int k_left = real ? c.k_left0 - st * BK : 0;
+#pragma unroll
+            for (int ps = 0; ps < PASSES; ++ps) {
+                const uint32_t off = (ps < k_left && c.m_ok) ? (uint32_t)ix.k[ps >> 2][ps & 3] * lda_b + (uint32_t)chunk * 16u : kGone;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(a_rsrc, (TW_LDS(void))(lds_a + stage * (STG * 2) + ps * SLOTB),
+                                                         16, (int)off, (int)c.m0b, 0, 0);
+            }
+        };
+        // A time slot: the index loads of the step after next, then the loads of the next step
+        // into LDS (twelve at 128 columns), then the meeting, at which only those may still be
+        // in flight: the step before them has landed.  The loads into LDS are never removed or
+        // reordered among themselves; the index loads are kept ahead of them by a compiler barrier
+        // and are not counted on (the compiler drops those whose result nobody reads).  These
+        // waves issue no stores (a wave's loads and stores retire in order and share the counter).
+        auto fence = [&]() { asm volatile("" ::: "memory"); };
+        auto meet = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(BPASS + PASSES) : "memory"); };
+        Item cur = make_item(qi);
+        Item nxt = cur;
+        bool have_next = false;
+        int gs = 0;          // stage of the current item's step 0 is gs % NST: the steps of all items count on
+        bool primed = false; // the current item's steps 0 and 1 are already on their way (see below)
+        Idx i0, i1;
+        while (!is_end(cur)) {
+            if (!has_steps(cur)) {
+                nxt = claim();
+                have_next = true;
+            }
+            if (is_fill(cur)) {
+                zero_fill(cur);
+            } else {
+                const int nsteps = has_steps(cur) ? cur.u.k_pad / BK : 0;
+                bool next_primed = false;
+                if (nsteps > 0) {
+                    const Ctx c = ctx_of(cur);
+                    if (!primed) {
+                        load_idx(c, 0, i0);
+                        load_idx(c, 1, i1);
+                        fence();
+                        issue(c, 0, gs % NST, i0);
+                        fence();
+                        load_idx(c, 2, i0);
+                        fence();
+                        issue(c, 1, (gs + 1) % NST, i1);
+                    }
+                    meet(); // time slot 0: step 0 has landed
+                    if (!have_next) {
+                        nxt = published();
+                        have_next = true;
+                    }
+                    // time slots 1 .. nsteps - 2 issue the steps 2 .. nsteps - 1 (odd slots out
+                    // of i0, even ones out of i1)
+                    int j = 1;
+                    for (; j + 2 < nsteps; j += 2) {
+                        load_idx(c, j + 2, i1);
+                        fence();
+                        issue(c, j + 1, (gs + j + 1) % NST, i0);
+                        meet();
+                        load_idx(c, j + 3, i0);
+                        fence();
+                        issue(c, j + 2, (gs + j + 2) % NST, i1);
+                        meet();
+                    }
+                    if (j + 1 < nsteps) {
+                        issue(c, j + 1, (gs + j + 1) % NST, i0);
+                        meet();
+                        ++j;
+                    }
+                    if (nsteps >= 2) {
+                        // The last time slot has no step of this item left to issue.  If the next
+                        // item has steps, its steps 0 and 1 go out now and after the last
+                        // multiplication (the C tile is staged in the stage of this item's last
+                        // step, the other two are free): they fly over the epilogue, and the next
+                        // item finds itself as after its first loads.
+                        const bool chain = has_steps(nxt);
+                        if (chain) {
+                            const Ctx cn = ctx_of(nxt);
+                            load_idx(cn, 0, i0);
+                            load_idx(cn, 1, i1);
+                            fence();
+                            issue(cn, 0, (gs + nsteps) % NST, i0);
+                            meet();
+                            TW_LDS_BARRIER(); // end of the last time slot
+                            load_idx(cn, 2, i0);
+                            fence();
+                            issue(cn, 1, (gs + nsteps + 1) % NST, i1);
+                            next_primed = true;
+                        } else {
+                            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); // the last step has landed
+                            TW_LDS_BARRIER(); // end of the last time slot
+                        }
+                    } else {
+                        TW_LDS_BARRIER(); // end of the last time slot
+                    }
+                } else {
+                    TW_LDS_BARRIER(); // end of the last time slot
+                }
+                // the multiplying waves stage the C tile, 64 columns at a time; these waves help
+                // to store it unless they are loading the next item
+                const uint16_t *const ctile = smem + ((nsteps > 0 ? gs + nsteps - 1 : gs) % NST) * STG;
+#pragma unroll
+                for (int r = 0; r < CROUNDS; ++r) {
+                    TW_LDS_BARRIER(); // staged
+                    if (!next_primed)
+                        store_round(ctile, r, cur.u, cur.m0, cur.m_end, true);
+                    TW_LDS_BARRIER(); // stored
+                }
+                gs += nsteps;
+                primed = next_primed;
+            }
+            TW_LDS_BARRIER(); // LDS may be reused now
+            cur = nxt;
+            have_next = false;
+        }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // nothing on its way into LDS when the workgroup ends
+        }
+    } else if (wave >= NMW) {
         // ================= moving waves ===================================================
         // A load of a wave covers RG kept rows (CPR lanes of 16 bytes each per row); lane
         // (g, chunk) moves chunk `chunk` (8 consecutive m) of the rows
@@ -892,6 +1103,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         Item cur = make_item(qi);
         Item nxt = cur;
         bool have_next = false;
+        int gs = 0; // (DMA) stage of the current item's step 0 is gs % NST
         while (!is_end(cur)) {
             if (!has_steps(cur)) {
                 nxt = claim();
@@ -926,8 +1138,8 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                 for (int ni = 0; ni < NI; ++ni)
                     out_bias[ni] = p.bias ? p.bias[out_col[ni]] : 0.0f;
                 auto frags = [&](int s, int ks, u32x4(&af)[MI], u32x4(&bf)[NI]) {
-                    const uint16_t *const stA = sA + (s & 1) * ASTAGE;
-                    const uint16_t *const stB = sB + (s & 1) * BSTAGE;
+                    const uint16_t *const stA = DMA ? sA + ((gs + s) % NST) * STG : sA + (s & 1) * ASTAGE;
+                    const uint16_t *const stB = DMA ? sB + ((gs + s) % NST) * STG : sB + (s & 1) * BSTAGE;
 #pragma unroll
                     for (int mi = 0; mi < MI; ++mi) {
                         // ds_read_b64_tr_b16: 16 lanes read a 4(k) x 16(m) block; lane L addresses
@@ -935,10 +1147,13 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                         const int L = lane & 15;
                         const int row = ks * 16 + (lane >> 5) * 8 + (L >> 2);
                         const int col = wave * RW + mi * 32 + ((lane >> 4) & 1) * 16 + (L & 3) * 4;
-                        const uint16_t *q = stA + row * PITCH + col;
+                        // (DMA: row (ks, lane >> 5, L >> 2) is half lane >> 5 of slot ks * 8 + (L >> 2))
+                        constexpr int RSTEP = DMA ? SLOTB / 2 : PITCH; // from row r to row r + 1 of a group of eight
+                        const uint16_t *q = DMA ? stA + (ks * 8 + (L >> 2)) * (SLOTB / 2) + (lane >> 5) * BM + col
+                                                : stA + row * PITCH + col;
                         s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))q);
                         s16x4 hi =
-                            __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * PITCH));
+                            __builtin_amdgcn_ds_read_tr16_b64_v4i16((TW_LDS(s16x4))(q + 4 * RSTEP));
                         u32x2 l2 = __builtin_bit_cast(u32x2, lo), h2 = __builtin_bit_cast(u32x2, hi);
                         af[mi].x = l2.x;
                         af[mi].y = l2.y;
@@ -1010,65 +1225,74 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                     }
                     scale = 1.0f;
                 }
-                if (fused) {
-                    // bias and activation in fp32, one rounding; the activation is a compile-time
-                    // constant of each copy
-                    auto stage_fused = [&](auto act_tag) {
-                        constexpr int ACT = decltype(act_tag)::value;
+                // The C tile goes through LDS in CROUNDS rounds of RNI blocks of 32 columns: all of
+                // it at once into the pipeline's stages, or (DMA) 64 columns at a time into the
+                // stage of the item's last step.
+                constexpr int RNI = NI / CROUNDS;
+                uint16_t *const ctile = DMA ? smem + ((nsteps > 0 ? gs + nsteps - 1 : gs) % NST) * STG : smem;
+                auto stage_round = [&](auto round_tag) {
+                    constexpr int RD = decltype(round_tag)::value;
+                    if (fused) {
+                        // bias and activation in fp32, one rounding; the activation is a
+                        // compile-time constant of each copy
+                        auto stage_fused = [&](auto act_tag) {
+                            constexpr int ACT = decltype(act_tag)::value;
 #pragma unroll
-                        for (int ni = 0; ni < NI; ++ni) {
-                            const int j = ni * 32 + (lane & 31);
-                            const float bj = out_bias[ni];
+                            for (int ni = RD * RNI; ni < (RD + 1) * RNI; ++ni) {
+                                const int j = (ni - RD * RNI) * 32 + (lane & 31);
+                                const float bj = out_bias[ni];
+#pragma unroll
+                                for (int mi = 0; mi < MI; ++mi) {
+                                    const int mloc = wave * RW + mi * 32 + (lane >> 5) * 4;
+#pragma unroll
+                                    for (int r4 = 0; r4 < 4; ++r4) {
+                                        float v[4];
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e)
+                                            v[e] = tw_fp32_value(tw_activate(scale * acc[mi][ni][r4 * 4 + e] + bj, ACT));
+                                        u32x2 pk;
+                                        pk.x = E::to_bits(v[0]) | (E::to_bits(v[1]) << 16);
+                                        pk.y = E::to_bits(v[2]) | (E::to_bits(v[3]) << 16);
+                                        *reinterpret_cast<u32x2 *>(ctile + j * CPITCH + mloc + r4 * 8) = pk;
+                                    }
+                                }
+                            }
+                        };
+                        switch (p.act) {
+                        case TW_ACT_RELU:
+                            stage_fused(std::integral_constant<int, TW_ACT_RELU>());
+                            break;
+                        case TW_ACT_GELU:
+                            stage_fused(std::integral_constant<int, TW_ACT_GELU>());
+                            break;
+                        case TW_ACT_TANH:
+                            stage_fused(std::integral_constant<int, TW_ACT_TANH>());
+                            break;
+                        default:
+                            stage_fused(std::integral_constant<int, TW_ACT_NONE>());
+                            break;
+                        }
+                    } else {
+#pragma unroll
+                        for (int ni = RD * RNI; ni < (RD + 1) * RNI; ++ni) {
+                            const int j = (ni - RD * RNI) * 32 + (lane & 31); // compact column inside the round
 #pragma unroll
                             for (int mi = 0; mi < MI; ++mi) {
                                 const int mloc = wave * RW + mi * 32 + (lane >> 5) * 4;
 #pragma unroll
                                 for (int r4 = 0; r4 < 4; ++r4) {
-                                    float v[4];
-#pragma unroll
-                                    for (int e = 0; e < 4; ++e)
-                                        v[e] = tw_fp32_value(tw_activate(scale * acc[mi][ni][r4 * 4 + e] + bj, ACT));
                                     u32x2 pk;
-                                    pk.x = E::to_bits(v[0]) | (E::to_bits(v[1]) << 16);
-                                    pk.y = E::to_bits(v[2]) | (E::to_bits(v[3]) << 16);
-                                    *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
+                                    pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
+                                           (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
+                                    pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
+                                           (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
+                                    *reinterpret_cast<u32x2 *>(ctile + j * CPITCH + mloc + r4 * 8) = pk;
                                 }
                             }
                         }
-                    };
-                    switch (p.act) {
-                    case TW_ACT_RELU:
-                        stage_fused(std::integral_constant<int, TW_ACT_RELU>());
-                        break;
-                    case TW_ACT_GELU:
-                        stage_fused(std::integral_constant<int, TW_ACT_GELU>());
-                        break;
-                    case TW_ACT_TANH:
-                        stage_fused(std::integral_constant<int, TW_ACT_TANH>());
-                        break;
-                    default:
-                        stage_fused(std::integral_constant<int, TW_ACT_NONE>());
-                        break;
                     }
-                } else {
-#pragma unroll
-                    for (int ni = 0; ni < NI; ++ni) {
-                        const int j = ni * 32 + (lane & 31); // compact column inside the unit
-#pragma unroll
-                        for (int mi = 0; mi < MI; ++mi) {
-                            const int mloc = wave * RW + mi * 32 + (lane >> 5) * 4;
-#pragma unroll
-                            for (int r4 = 0; r4 < 4; ++r4) {
-                                u32x2 pk;
-                                pk.x = E::to_bits(scale * acc[mi][ni][r4 * 4 + 0]) |
-                                       (E::to_bits(scale * acc[mi][ni][r4 * 4 + 1]) << 16);
-                                pk.y = E::to_bits(scale * acc[mi][ni][r4 * 4 + 2]) |
-                                       (E::to_bits(scale * acc[mi][ni][r4 * 4 + 3]) << 16);
-                                *reinterpret_cast<u32x2 *>(smem + j * CPITCH + mloc + r4 * 8) = pk;
-                            }
-                        }
-                    }
-                }
+                };
+                stage_round(std::integral_constant<int, 0>());
                 if (wave == 0 && lane < 32) {
 #pragma unroll
                     for (int ni = 0; ni < NI; ++ni)
@@ -1077,8 +1301,23 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                 pick_up();
                 if (tid == 0 && announced)
                     asm volatile("" : "+v"(t_done)); // the count has returned: read it before the stores
-                TW_LDS_BARRIER(); // the C tile is staged
-                store_tile(u, m0, cur.m_end);
+                TW_LDS_BARRIER(); // the C tile (its first round) is staged
+                if constexpr (!DMA) {
+                    store_tile(u, m0, cur.m_end);
+                } else {
+                    // (the moving waves help unless they are loading the next item already)
+                    const bool all_store = !(nsteps >= 2 && has_steps(nxt));
+                    store_round(ctile, 0, u, m0, cur.m_end, all_store);
+                    TW_LDS_BARRIER(); // stored: the stage may be written again
+                    if constexpr (CROUNDS > 1) {
+                        stage_round(std::integral_constant<int, CROUNDS - 1>());
+                        TW_LDS_BARRIER(); // staged
+                        store_round(ctile, 1, u, m0, cur.m_end, all_store);
+                        TW_LDS_BARRIER(); // stored
+                    }
+                    static_assert(CROUNDS <= 2, "two rounds at most");
+                    gs += nsteps;
+                }
             }
             TW_LDS_BARRIER(); // LDS may be reused now
             cur = nxt;
@@ -2053,10 +2292,16 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
         hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 128, 32, TW_R_128x32>), dim3(grid), dim3(256), 0, s, a);
         break;
     case TW_SHAPE_256x64:
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 64, TW_R_256x64>), dim3(grid), dim3(512), 0, s, a);
+        if (a.lds_dma)
+            hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 64, TW_R_256x64, true>), dim3(grid), dim3(512), 0, s, a);
+        else
+            hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 64, TW_R_256x64>), dim3(grid), dim3(512), 0, s, a);
         break;
     default: // TW_SHAPE_256x128
-        hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128, TW_R_256x128>), dim3(grid), dim3(512), 0, s, a);
+        if (a.lds_dma)
+            hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128, TW_R_256x128, true>), dim3(grid), dim3(512), 0, s, a);
+        else
+            hipLaunchKernelGGL((tw_gemm_ws_kernel<DT, 256, 128, TW_R_256x128>), dim3(grid), dim3(512), 0, s, a);
         break;
     }
 }
@@ -2067,7 +2312,8 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
 static std::atomic<int> g_opt[TW_N_OPTIONS];
 static std::once_flag g_opt_once;
 static const char *const kOptEnv[TW_N_OPTIONS] = {"TWGEMM_SHAPE", "TWGEMM_WGS_PER_CU", "TWGEMM_PIECE",
-                                                  "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT", "TWGEMM_BALANCE"};
+                                                  "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT", "TWGEMM_BALANCE",
+                                                  "TWGEMM_LDS_DMA"};
 
 static bool option_in_range(int option, int value)
 {
@@ -2085,6 +2331,7 @@ static bool option_in_range(int option, int value)
     case TW_OPT_SPIN_LIMIT:
         return value >= 0;
     case TW_OPT_BALANCE:
+    case TW_OPT_LDS_DMA:
         return value == 0 || value == 1;
     }
     return false;
@@ -2164,6 +2411,11 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc,
     // units give 384 workgroups for 512 slots, and the kernel is then 1 us slower than the
     // A-stationary one (15 against 14), where 32 units (BERT-large FFN1 at 90 %) gain 12 %.
     const bool bs = bs_takes(plan, lda, ldc, reads_c) && width > 64 && M >= 2048 && bs_fill(plan, M) >= 0.9;
+    // Tiles of six steps and more on average, wide, with 256-row items for three quarters of the
+    // chip: the streaming 256 x 128 kernel, whose loads write LDS directly, is ahead of the panel
+    // (M 8192, K 1024, N 2048, half the rows kept: 28.4 against 33.2 us; BERT-large FFN1 at 50 %
+    // 47 against 52 - 58)
+    const bool long_tiles = ws_ok && width > 64 && plan->pipe_steps >= 6 * units && items(256, 128) * 4 >= 3 * cu;
     if (skinny) {
         c.shape = TW_SHAPE_SKINNY;
     } else if (bs) {
@@ -2171,7 +2423,7 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc,
     } else if (!ws_ok) {
         c.shape = TW_SHAPE_WIDE;
     } else if (as_ok(TW_SHAPE_AS64) && (M > 128 || plan->n_blocks >= 96) &&
-               (!plan->rows_shared || width <= 64 || items(256, 128) * 2 <= 3 * cu)) {
+               (!plan->rows_shared || width <= 64 || items(256, 128) * 2 <= 3 * cu) && !long_tiles) {
         // (a 0 %-sparse plan with many 256-row items is better off streaming with one queue per
         // die: M 12800, K 768, N 3072: 87 against 96 us)
         // 64-row panels where they still give three quarters of the compute units a workgroup
@@ -2201,9 +2453,10 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc,
         }
     } else if (width > 32) {
         c.piece = 64;
-        if (items(512, 64) * 5 >= 3 * cu) {
-            c.shape = TW_SHAPE_512x64;
-        } else if (items(256, 64) * 5 >= 3 * cu) {
+        // (256-row items, whose loads write LDS directly, are ahead of 512-row items wherever
+        // both fill the chip - M 2048, K 4096, N 4096, half the rows kept: 50 against 66 us; the
+        // stress shape 363 against 385 - and of 128-row items from a quarter of a chip of items on)
+        if (items(256, 64) * 4 >= cu) {
             c.shape = TW_SHAPE_256x64;
         } else if (items(128, 64) * 2 >= cu) {
             c.shape = TW_SHAPE_128x64;
@@ -2419,6 +2672,8 @@ void fill_common(GemmArgs &a, const tw_plan *plan, const void *A, int64_t lda, v
     a.ticket = nullptr;
     a.n_bal = 0;
     a.rb_major = 0;
+    a.lds_dma = 0;
+    a.a_bytes = a.b_bytes = 0;
     a.n_arg_units = 0;
 }
 
@@ -2611,6 +2866,13 @@ int gemm_impl(const tw_plan *plan, const void *A, int a_layout, int64_t lda, voi
     const Choice c = choose_shape(plan, M, lda, ldc, beta != 0.0f);
     fill_queues(a, plan, M, kShapes[c.shape].bm, c.piece, pruned_cols, c.xcd);
     a.rb_major = option(TW_OPT_XCD_QUEUES) == 2;
+    // 256-row items whose loads write LDS directly (measured faster on every shape tried, with
+    // one item per workgroup and with several)
+    if ((c.shape == TW_SHAPE_256x128 || c.shape == TW_SHAPE_256x64) && option(TW_OPT_LDS_DMA) != 0 && (uint64_t)plan->packed_elems * 2u < (1ull << 32)) {
+        a.lds_dma = 1;
+        a.a_bytes = (uint32_t)((uint64_t)plan->K * (uint64_t)lda * 2u); // (a chunk that holds row K - 1's last elements is read whole)
+        a.b_bytes = (uint32_t)((uint64_t)plan->packed_elems * 2u);
+    }
     // (a tuning switch, off unless asked for: measured on the benchmark shapes it changes nothing,
     // a step of an item takes as long at 192 rows as at 256)
     if (c.shape != TW_SHAPE_WIDE && !is_queueless_shape(c.shape) && option(TW_OPT_BALANCE) == 1)

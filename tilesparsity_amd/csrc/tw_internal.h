@@ -96,6 +96,10 @@ struct GemmArgs {
     // queues, n_own == 0, n_tail_items items): column u has items of bal_rows[u] rows, the items
     // bal_first[u] .. bal_first[u + 1] - 1 of the list.  See balance_items.
     int32_t n_bal;
+    // The 256 x 128 kernel in its direct-to-LDS form: bytes of A (K * lda elements) and
+    // of the packed weight, the sizes of the two buffers its loads are checked against.
+    int32_t lds_dma;
+    uint32_t a_bytes, b_bytes;
     int32_t rb_major;     // the items no queue owns are dealt out row block after row block instead of column after column
     int32_t bal_first[kBalColumns + 1];
     int32_t bal_rows[kBalColumns];
@@ -143,6 +147,7 @@ struct tw_plan {
     int n_halves = 0;   // pieces of 64 compact columns over all units (the skinny kernel's work per row block)
     bool rows_shared = false; // the tiles that keep rows keep nearly all of them (a dense or almost dense plan)
     int max_k_pad = 0;        // most kept rows of a tile, rounded up to whole steps
+    int64_t pipe_steps = 0;   // steps of 64 kept rows over all units that have any
     int cu_count = 0;
 };
 

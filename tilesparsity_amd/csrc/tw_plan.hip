@@ -639,8 +639,11 @@ int finalize_plan_geometry(tw_plan *p, hipStream_t s)
                      (int64_t)p->kept_k_idx.size() * 10 >= (int64_t)p->K * tiles_with_rows * 9;
     p->n_zero_tiles = (int)ztiles.size();
     p->max_k_pad = 0;
-    for (const UnitDev &u : units)
+    p->pipe_steps = 0;
+    for (const UnitDev &u : units) {
         p->max_k_pad = std::max(p->max_k_pad, u.k_pad);
+        p->pipe_steps += u.k_pad / kBlockK;
+    }
 
     // One device allocation for everything the plan owns besides lists that were compacted on
     // the device: [staged tables, uploaded with one copy][ticket slots][packed weight], the last

@@ -30,10 +30,11 @@ MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 # this run: `traffic_source` in the line says which file, and for which kernel, they stand.
 # Keyed by the workload's own name.
 MEASURED_TRAFFIC = {
-    "vgg16_conv4_2_im2col": ((2 * 62054 + 11282) * 1024, "profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md (tw_gemm_ws_kernel 256x128)"),
+    "vgg16_conv4_2_im2col": ((2 * 62014 + 11282) * 1024, "profiles/tw_gemm_ws_kernel__vgg16_conv4_2.md (tw_gemm_ws_kernel 256x128)"),
     "bert_base_ffn_in": ((2 * 7897 + 24576) * 1024, "profiles/tw_gemm_as_kernel__bert_base_ffn.md (tw_gemm_as_kernel 64 rows)"),
     "nmt_lstm_gates": ((2 * 3558.5 + 1024) * 1024, "profiles/tw_gemm_skinny_kernel__nmt_lstm_gates.md (tw_gemm_skinny_kernel)"),
-    "imbalance_stress": ((2 * 908806 + 212608) * 1024, "profiles/tw_gemm_ws_kernel__imbalance_stress.md (tw_gemm_ws_kernel 512x64)"),
+    "imbalance_stress": ((2 * 922921 + 209150) * 1024, "profiles/tw_gemm_ws_kernel__imbalance_stress.md (tw_gemm_ws_kernel 256x64)"),
+    "bert_large_ffn2_keep50": ((2 * 49480 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
     "bert_large_ffn1_keep25": ((2 * 16649 + 65536) * 1024, "profiles/tw_gemm_as_kernel__bert_large_ffn1.md (tw_gemm_as_kernel 64 rows)"),
     "bert_large_ffn1_keep10": ((2 * 12319 + 65536) * 1024, "profiles/tw_gemm_bs_kernel__bert_large_ffn1_90.md (tw_gemm_bs_kernel)"),
     "bert_large_ffn2_keep25": ((2 * 38143 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),

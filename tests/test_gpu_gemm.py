@@ -734,6 +734,70 @@ def test_row_blocks_sized_per_tile(tw, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("shape_bn", [128, 64])
+def test_streaming_kernel_several_items_per_workgroup(tw, oracle, dtype, shape_bn):
+    """The 256-row streaming kernels with more items than workgroups, so that every workgroup runs
+    several one after the other: the first steps of the next item are loaded over the epilogue of
+    the current one, and a full C tile (every column kept, 256 rows) is stored by the moving waves
+    during the next item's first time slot.  Tiles of 1 to 7 steps, one without kept rows, full
+    and partly kept columns, a ragged last row block: the same bits as the register-staged form of
+    the kernel (TW_OPT_LDS_DMA = 0) and as a second launch, within tolerance of the oracle, with
+    bias + activation and filled pruned columns as well."""
+    import torch
+    rng = np.random.default_rng(31337 + shape_bn)
+    G = shape_bn
+    n_tiles = 40 if G == 128 else 72
+    M, K, N = 2048 + 256 * 5 + 77, 448, n_tiles * G          # 14 row blocks, the last one ragged
+    A = rng.standard_normal((M, K)).astype(np.float32)
+    B = (rng.standard_normal((K, N)) * 0.05).astype(np.float32)
+    bias = rng.standard_normal(N).astype(np.float32)
+    tiles = []
+    for t in range(n_tiles):
+        kt = (64, 128, 200, 448, 0, 130, 70, 256)[t % 8]
+        nt = G if t % 3 else int(G * 0.8)
+        tiles.append(dict(col0=t * G, width=G,
+                          kept_k=np.sort(rng.choice(K, size=kt, replace=False)).astype(np.int32),
+                          kept_n=np.sort(rng.choice(G, size=nt, replace=False)).astype(np.int32)))
+    keep = kept_columns(tiles, N)
+    ref = reference(oracle, A, B, tiles, dtype)
+    dbias = torch.from_numpy(bias).cuda()
+    lda = ldc = round_up(M, 8)
+    At = np.zeros((K, lda), np.uint16)
+    At[:, :M] = oracle.cast_bits(A, dtype).reshape(M, K).T
+    dA = to_device_bits(At, At.shape)
+    shape = tw.SHAPE_256x128 if G == 128 else tw.SHAPE_256x64
+
+    def launch(plan, dma, pruned, with_bias, act):
+        dC = to_device_bits(np.full((N, ldc), SENTINEL, np.uint16), (N, ldc))
+        tw.set_option(tw.OPT_LDS_DMA, dma)
+        print("several items per workgroup:", G, dma, pruned, with_bias, act, dtype, flush=True)
+        assert plan.choice(M, lda, ldc)["shape"] == shape
+        plan.gemm(dA.data_ptr(), dC.data_ptr(), M, lda=lda, ldc=ldc, pruned_cols=pruned,
+                  bias_ptr=dbias.data_ptr() if with_bias else None, activation=act,
+                  stream=torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        return from_device_bits(dC)
+
+    try:
+        tw.set_option(tw.OPT_SHAPE, shape)
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            for (pruned, with_bias, act) in ((tw.PRUNED_UNTOUCHED, False, tw.ACT_NONE),
+                                             (tw.PRUNED_ZERO, True, tw.ACT_RELU)):
+                want = launch(plan, 0, pruned, with_bias, act)
+                for rep in range(2):
+                    got = launch(plan, 1, pruned, with_bias, act)
+                    assert np.array_equal(got, want), (rep, pruned, with_bias, act)
+                assert (want[:, M:] == SENTINEL).all()
+                if not with_bias:
+                    Cf = oracle.bits_to_f32(want[:, :M], dtype).reshape(N, M).T
+                    assert oracle.rel_error(Cf[:, keep], ref[:, keep]) <= TOL[dtype]
+                    assert (want[~keep] == SENTINEL).all()
+    finally:
+        tw.set_option(tw.OPT_SHAPE, -1)
+        tw.set_option(tw.OPT_LDS_DMA, -1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
 def test_256x64_shape_epilogues(tw, oracle, dtype):
     """The 256 x 64 streaming shape (64-wide tiles of plans with few items) with every epilogue:
     alpha / beta, bias + activation, filled pruned columns, both queue layouts and both piece

@@ -731,6 +731,11 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         }
     };
 
+    // (DMA) the moving waves store this item's C tile during the next item's first time slot:
+    // a full tile (no lane, no column to skip) followed by an item of two steps or more
+    auto defer_stores = [&](const Item &it, const Item &next) {
+        return it.u.n_cnt == BN && it.m_end - it.m0 == BM && has_steps(next) && next.u.k_pad >= 2 * BK;
+    };
     // (DMA) scatters round rd of a C tile staged at `ctile`: 64 columns at most.  By the multiplying
     // waves alone where the moving waves are already loading the workgroup's next item (they must
     // not have stores among their loads), else by all waves.
@@ -827,12 +832,76 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         // waves issue no stores (a wave's loads and stores retire in order and share the counter).
         auto fence = [&]() { asm volatile("" ::: "memory"); };
         auto meet = [&]() { asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(BPASS + PASSES) : "memory"); };
+        // Deferred stores.  Where a full C tile (every column kept, 256 rows) is followed by
+        // another item of this workgroup, these waves take the staged tile out of LDS into
+        // registers (8 x 16 bytes a lane and round) and store it during the next item's first
+        // time slot, so that the multiplying waves go straight on: the chip's stores then run
+        // beside the next item's products instead of between two items.  The stores come BEHIND
+        // the slot's loads in the wave's queue: the meetings of that slot and the next count them
+        // in (the step waited for is older than they are), and by the slot after, two steps
+        // later, memory has acknowledged them.  Their number is fixed (a full tile has no lane
+        // and no column to skip), so the counts stay exact.
+        constexpr int NDS = 8 * CROUNDS; // stores a lane defers
+        auto meet_wide = [&](bool wide) {
+            if (wide)
+                asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(BPASS + PASSES + NDS) : "memory");
+            else
+                meet();
+        };
+        u32x2 dlo[NDS], dhi[NDS]; // the deferred tile: column pt / CPR + 8 i of round r, 8 rows m from m_st on
+        int dcol[NDS];
+        uint16_t *d_c = C;        // C + the lane's first row of the deferred tile
+        bool deferred = false;
+        const int pt = tid - NPM;
+        auto take_round = [&](const uint16_t *ctile, int rd) {
+            // LDS reads in asm: a C++ read would make the compiler wait for every load into LDS
+            // that is on its way (it cannot tell that those go to other stages)
+            const uint32_t a0 = (uint32_t)(uintptr_t)(TW_LDS(const uint16_t))(ctile + (pt / CPR) * CPITCH + (pt % CPR) * 8);
+            const uint32_t c0 = (uint32_t)(uintptr_t)(TW_LDS(const int))(s_cols + rd * 64 + pt / CPR);
+#pragma unroll
+            for (int i = 0; i < 8; i += 4) {
+                asm volatile("ds_read_b64 %0, %8 offset:%9\n\tds_read_b64 %1, %8 offset:%10\n\t"
+                             "ds_read_b64 %2, %8 offset:%11\n\tds_read_b64 %3, %8 offset:%12\n\t"
+                             "ds_read_b64 %4, %8 offset:%13\n\tds_read_b64 %5, %8 offset:%14\n\t"
+                             "ds_read_b64 %6, %8 offset:%15\n\tds_read_b64 %7, %8 offset:%16\n\t"
+                             "s_waitcnt lgkmcnt(0)"
+                             : "=&v"(dlo[rd * 8 + i]), "=&v"(dhi[rd * 8 + i]), "=&v"(dlo[rd * 8 + i + 1]), "=&v"(dhi[rd * 8 + i + 1]),
+                               "=&v"(dlo[rd * 8 + i + 2]), "=&v"(dhi[rd * 8 + i + 2]), "=&v"(dlo[rd * 8 + i + 3]), "=&v"(dhi[rd * 8 + i + 3])
+                             : "v"(a0), "n"((i + 0) * 8 * CPITCH * 2), "n"((i + 0) * 8 * CPITCH * 2 + 8),
+                               "n"((i + 1) * 8 * CPITCH * 2), "n"((i + 1) * 8 * CPITCH * 2 + 8),
+                               "n"((i + 2) * 8 * CPITCH * 2), "n"((i + 2) * 8 * CPITCH * 2 + 8),
+                               "n"((i + 3) * 8 * CPITCH * 2), "n"((i + 3) * 8 * CPITCH * 2 + 8)
+                             : "memory");
+            }
+            asm volatile("ds_read_b32 %0, %8\n\tds_read_b32 %1, %8 offset:32\n\tds_read_b32 %2, %8 offset:64\n\t"
+                         "ds_read_b32 %3, %8 offset:96\n\tds_read_b32 %4, %8 offset:128\n\tds_read_b32 %5, %8 offset:160\n\t"
+                         "ds_read_b32 %6, %8 offset:192\n\tds_read_b32 %7, %8 offset:224\n\ts_waitcnt lgkmcnt(0)"
+                         : "=&v"(dcol[rd * 8 + 0]), "=&v"(dcol[rd * 8 + 1]), "=&v"(dcol[rd * 8 + 2]), "=&v"(dcol[rd * 8 + 3]),
+                           "=&v"(dcol[rd * 8 + 4]), "=&v"(dcol[rd * 8 + 5]), "=&v"(dcol[rd * 8 + 6]), "=&v"(dcol[rd * 8 + 7])
+                         : "v"(c0)
+                         : "memory");
+        };
+        auto store_deferred = [&]() {
+#pragma unroll
+            for (int i = 0; i < NDS; ++i) {
+                u32x4 v;
+                v.x = dlo[i].x;
+                v.y = dlo[i].y;
+                v.z = dhi[i].x;
+                v.w = dhi[i].y;
+                uint16_t *const dst = d_c + (int64_t)dcol[i] * p.ldc;
+                if (p.store_through)
+                    asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+                else
+                    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(dst), "v"(v) : "memory");
+            }
+        };
         Item cur = make_item(qi);
         Item nxt = cur;
         bool have_next = false;
         int gs = 0;          // stage of the current item's step 0 is gs % NST: the steps of all items count on
         bool primed = false; // the current item's steps 0 and 1 are already on their way (see below)
-        Idx i0, i1;
+        Idx i0, i1, n0, n1;
         while (!is_end(cur)) {
             if (!has_steps(cur)) {
                 nxt = claim();
@@ -855,10 +924,22 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                         fence();
                         issue(c, 1, (gs + 1) % NST, i1);
                     }
-                    meet(); // time slot 0: step 0 has landed
+                    if (deferred)
+                        store_deferred();
+                    meet_wide(deferred); // time slot 0: step 0 has landed
                     if (!have_next) {
                         nxt = published();
                         have_next = true;
+                    }
+                    // the next item's first index words, for the loads that the last time slot
+                    // issues on its behalf: fetched now, so that nobody waits for them there
+                    const bool chain = nsteps >= 2 && has_steps(nxt);
+                    Ctx cn = c;
+                    if (chain) {
+                        cn = ctx_of(nxt);
+                        load_idx(cn, 0, n0);
+                        load_idx(cn, 1, n1);
+                        fence();
                     }
                     // time slots 1 .. nsteps - 2 issue the steps 2 .. nsteps - 1 (odd slots out
                     // of i0, even ones out of i1)
@@ -867,7 +948,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                         load_idx(c, j + 2, i1);
                         fence();
                         issue(c, j + 1, (gs + j + 1) % NST, i0);
-                        meet();
+                        meet_wide(deferred && j == 1);
                         load_idx(c, j + 3, i0);
                         fence();
                         issue(c, j + 2, (gs + j + 2) % NST, i1);
@@ -875,7 +956,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                     }
                     if (j + 1 < nsteps) {
                         issue(c, j + 1, (gs + j + 1) % NST, i0);
-                        meet();
+                        meet_wide(deferred && j == 1);
                         ++j;
                     }
                     if (nsteps >= 2) {
@@ -884,18 +965,13 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                         // multiplication (the C tile is staged in the stage of this item's last
                         // step, the other two are free): they fly over the epilogue, and the next
                         // item finds itself as after its first loads.
-                        const bool chain = has_steps(nxt);
                         if (chain) {
-                            const Ctx cn = ctx_of(nxt);
-                            load_idx(cn, 0, i0);
-                            load_idx(cn, 1, i1);
-                            fence();
-                            issue(cn, 0, (gs + nsteps) % NST, i0);
-                            meet();
+                            issue(cn, 0, (gs + nsteps) % NST, n0);
+                            meet_wide(deferred && j == 1);
                             TW_LDS_BARRIER(); // end of the last time slot
                             load_idx(cn, 2, i0);
                             fence();
-                            issue(cn, 1, (gs + nsteps + 1) % NST, i1);
+                            issue(cn, 1, (gs + nsteps + 1) % NST, n1);
                             next_primed = true;
                         } else {
                             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory"); // the last step has landed
@@ -910,12 +986,17 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                 // the multiplying waves stage the C tile, 64 columns at a time; these waves help
                 // to store it unless they are loading the next item
                 const uint16_t *const ctile = smem + ((nsteps > 0 ? gs + nsteps - 1 : gs) % NST) * STG;
+                deferred = next_primed && defer_stores(cur, nxt);
+                if (deferred)
+                    d_c = C + cur.m0 + (pt % CPR) * 8;
 #pragma unroll
                 for (int r = 0; r < CROUNDS; ++r) {
                     TW_LDS_BARRIER(); // staged
-                    if (!next_primed)
+                    if (deferred)
+                        take_round(ctile, r);
+                    else if (!next_primed)
                         store_round(ctile, r, cur.u, cur.m0, cur.m_end, true);
-                    TW_LDS_BARRIER(); // stored
+                    TW_LDS_BARRIER(); // stored, or taken
                 }
                 gs += nsteps;
                 primed = next_primed;
@@ -1306,13 +1387,17 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                     store_tile(u, m0, cur.m_end);
                 } else {
                     // (the moving waves help unless they are loading the next item already)
-                    const bool all_store = !(nsteps >= 2 && has_steps(nxt));
-                    store_round(ctile, 0, u, m0, cur.m_end, all_store);
-                    TW_LDS_BARRIER(); // stored: the stage may be written again
+                    const bool chained = nsteps >= 2 && has_steps(nxt);
+                    const bool all_store = !chained;
+                    const bool deferred = chained && defer_stores(cur, nxt);
+                    if (!deferred)
+                        store_round(ctile, 0, u, m0, cur.m_end, all_store);
+                    TW_LDS_BARRIER(); // stored (or taken by the moving waves): the stage may be written again
                     if constexpr (CROUNDS > 1) {
                         stage_round(std::integral_constant<int, CROUNDS - 1>());
                         TW_LDS_BARRIER(); // staged
-                        store_round(ctile, 1, u, m0, cur.m_end, all_store);
+                        if (!deferred)
+                            store_round(ctile, 1, u, m0, cur.m_end, all_store);
                         TW_LDS_BARRIER(); // stored
                     }
                     static_assert(CROUNDS <= 2, "two rounds at most");

@@ -2495,11 +2495,14 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc,
     // Its workgroups (unit x range of rows) have to fill the chip's slots evenly: BERT-base's 24
     // units give 384 workgroups for 512 slots, and the kernel is then 1 us slower than the
     // A-stationary one (15 against 14), where 32 units (BERT-large FFN1 at 90 %) gain 12 %.
-    const bool bs = bs_takes(plan, lda, ldc, reads_c) && width > 64 && M >= 2048 && bs_fill(plan, M) >= 0.9;
+    // With K = 512 the panel of A is small and the A-stationary kernel stays ahead (M 16384, N 4096:
+    // 43 against 49 - 54 us), so the kernel is taken from K = 1024 on.
+    const bool bs = bs_takes(plan, lda, ldc, reads_c) && width > 64 && M >= 2048 && plan->K >= 1024 && bs_fill(plan, M) >= 0.9;
     // Tiles of six steps and more on average, wide, with 256-row items for three quarters of the
     // chip: the streaming 256 x 128 kernel, whose loads write LDS directly, is ahead of the panel
     // (M 8192, K 1024, N 2048, half the rows kept: 28.4 against 33.2 us; BERT-large FFN1 at 50 %
-    // 47 against 52 - 58)
+    // 47 against 55; at four steps the two are level: BERT-large FFN1 at 75 % 34 against 34 - 37,
+    // random tiles of K 1024 with a quarter of the rows kept 39 against 36)
     const bool long_tiles = ws_ok && width > 64 && plan->pipe_steps >= 6 * units && items(256, 128) * 4 >= 3 * cu;
     if (skinny) {
         c.shape = TW_SHAPE_SKINNY;

@@ -783,6 +783,7 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         TW_LDS(unsigned char) const lds_b = (TW_LDS(unsigned char))sB + mw * 1024;
         // what the loads of an item's steps need
         struct Ctx {
+            const int32_t *k_list; // the tile's padded list of kept rows (uniform)
             const char *k_base;
             uint32_t m0b, b_pack_b;
             uint32_t b_blk[BPASS]; // weight block of load bp (a block beyond the unit reads block 0), bytes into Bp
@@ -791,7 +792,8 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
         };
         auto ctx_of = [&](const Item &it) {
             Ctx c;
-            c.k_base = reinterpret_cast<const char *>(p.kept_k + it.u.kk_off) + row0 * 4;
+            c.k_list = p.kept_k + it.u.kk_off;
+            c.k_base = reinterpret_cast<const char *>(c.k_list) + row0 * 4;
             c.m0b = (uint32_t)it.m0 * 2u;
             c.m_ok = it.m0 + chunk * 8 < it.m_end;
             c.k_left0 = it.u.k_kept - row0;
@@ -806,6 +808,17 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
 #pragma unroll
             for (int i = 0; i < PASSES / 4; ++i)
                 ix.k[i] = *reinterpret_cast<const i32x4 *>(c.k_base + (int64_t)st * (BK * 4) + 16 * i);
+        };
+        // The same words through the scalar cache (the wave's sixteen rows of the step, of which a
+        // lane picks its eight): for the next item's first steps, whose index words are fetched
+        // while this item's loads are in flight.  A vector load there would make the compiler wait
+        // for all of those first (it cannot tell, around the loop over the items, that the
+        // registers it is about to overwrite are no longer being loaded into).
+        auto load_idx_scalar = [&](const Ctx &c, int st, Idx &ix) {
+            const auto *kp = (const __attribute__((address_space(4))) int32_t *)(uintptr_t)(c.k_list + st * BK + mw * RPW);
+#pragma unroll
+            for (int e = 0; e < PASSES; ++e)
+                ix.k[e >> 2][e & 3] = g ? kp[PASSES + e] : kp[e];
         };
         // the BPASS + PASSES loads of step st of an item into stage `stage`
         auto issue = [&](const Ctx &c, int st, int stage, const Idx &ix) {
@@ -937,9 +950,8 @@ __global__ void __launch_bounds__(BM == 128 ? 256 : 512, 2) tw_gemm_ws_kernel(co
                     Ctx cn = c;
                     if (chain) {
                         cn = ctx_of(nxt);
-                        load_idx(cn, 0, n0);
-                        load_idx(cn, 1, n1);
-                        fence();
+                        load_idx_scalar(cn, 0, n0);
+                        load_idx_scalar(cn, 1, n1);
                     }
                     // time slots 1 .. nsteps - 2 issue the steps 2 .. nsteps - 1 (odd slots out
                     // of i0, even ones out of i1)

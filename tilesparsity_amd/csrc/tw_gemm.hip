@@ -2515,7 +2515,12 @@ static Choice choose_shape(const tw_plan *plan, int M, int64_t lda, int64_t ldc,
     // (M 8192, K 1024, N 2048, half the rows kept: 28.4 against 33.2 us; BERT-large FFN1 at 50 %
     // 47 against 55; at four steps the two are level: BERT-large FFN1 at 75 % 34 against 34 - 37,
     // random tiles of K 1024 with a quarter of the rows kept 39 against 36)
-    const bool long_tiles = ws_ok && width > 64 && plan->pipe_steps >= 6 * units && items(256, 128) * 4 >= 3 * cu;
+    // (only where the 256-row items come out even over the workgroups: 600 items on 256 are three
+    // rounds for 2.3 rounds of work, and the panel kernel wins: M 12800, K 768, N 3072 with 12 tiles
+    // of 384 kept rows 28.3 against 32.2 us)
+    const int64_t it256 = items(256, 128);
+    const bool long_tiles = ws_ok && width > 64 && plan->pipe_steps >= 6 * units && it256 * 4 >= 3 * cu &&
+                            it256 * 10 >= (it256 + cu - 1) / cu * cu * 9;
     if (skinny) {
         c.shape = TW_SHAPE_SKINNY;
     } else if (bs) {

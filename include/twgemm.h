@@ -309,8 +309,13 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  *                       unless nearly every tile keeps nearly every row (a 0 %-sparse plan);
  *                       2: dealt out over the dies in turn, row block after row block (all tiles
  *                       of a row block before the next) instead of tile after tile
+ *   TW_OPT_SPIN_LIMIT   polls a workgroup of tw_lstm_steps spends at a barrier before it gives up
+ *   TW_OPT_BALANCE      1: row blocks sized per tile where the items would not fill the chip once
+ *   TW_OPT_LDS_DMA      0: the 256-row streaming kernels stage their loads through registers
+ *                       instead of writing LDS directly (same results, bit for bit)
  * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
- * TWGEMM_PIECE and TWGEMM_XCD_QUEUES, read once. */
+ * TWGEMM_PIECE, TWGEMM_XCD_QUEUES, TWGEMM_SPIN_LIMIT, TWGEMM_BALANCE and TWGEMM_LDS_DMA, read
+ * once. */
 #define TW_OPT_SHAPE 0
 #define TW_OPT_WGS_PER_CU 1
 #define TW_OPT_PIECE 2
@@ -321,11 +326,11 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_N_OPTIONS 7
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
-#define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns */
+#define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns (forced only: 256 x 64 is ahead) */
 #define TW_SHAPE_128x64 3  /* wave-specialised, 128 x 64 */
-#define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU */
+#define TW_SHAPE_256x128 4 /* wave-specialised, 256 x 128, one workgroup per CU, loads straight into LDS */
 #define TW_SHAPE_128x32 5  /* wave-specialised, 128 x 32: skinny M */
-#define TW_SHAPE_256x64 6  /* wave-specialised, 256 x 64 */
+#define TW_SHAPE_256x64 6  /* wave-specialised, 256 x 64, loads straight into LDS */
 #define TW_SHAPE_AS64 7    /* A-stationary, 64 rows of all K in LDS: K up to 1064, beta == 0 */
 #define TW_SHAPE_AS32 8    /* A-stationary, 32 rows: K up to 2128, beta == 0 */
 #define TW_SHAPE_SKINNY 9  /* 64 rows x 32 columns per workgroup, the kept rows split over its waves: few rows of A */

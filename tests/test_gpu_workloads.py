@@ -185,6 +185,46 @@ def test_config5_imbalance_stress(tw, oracle):
     check_workload(tw, oracle, wl)
 
 
+@pytest.mark.parametrize("name", ["vgg16_conv4_2", "bert_large_ffn2_75", "bert_large_ffn1_50"])
+def test_direct_loads_repeat_under_back_to_back_launches(tw, name):
+    """The 256 x 128 kernel with loads that write LDS directly relies on exact counts of the loads
+    in flight.  At full size, with launches queued back to back (a launch then starts while the
+    memory system is still busy with its predecessor's stores, which is when a count that is one
+    too generous shows), every launch gives the bits of the register-staged form of the kernel:
+    one item per workgroup (VGG16 conv4_2, BERT-large FFN2) and four chained items with deferred
+    stores (BERT-large FFN1)."""
+    import torch
+    from tilesparsity_amd import workloads
+    wl = {"vgg16_conv4_2": workloads.vgg16_conv4_2, "bert_large_ffn2_75": lambda: workloads.bert_large_ffn(2, 0.25),
+          "bert_large_ffn1_50": lambda: workloads.bert_large_ffn(1, 0.50)}[name]()
+    M, K, N, dtype, tiles = wl["M"], wl["K"], wl["N"], wl["dtype"], wl["tiles"]
+    A, B = wl["values"]()
+    tdt = torch.float16 if dtype == "f16" else torch.bfloat16
+    At = torch.from_numpy(A).cuda().to(tdt).t().contiguous()
+    s = torch.cuda.current_stream().cuda_stream
+    try:
+        tw.set_option(tw.OPT_SHAPE, tw.SHAPE_256x128)
+        with tw.Plan.create(K, N, dtype, tiles, B) as plan:
+            tw.set_option(tw.OPT_LDS_DMA, 0)
+            want = torch.zeros((N, M), dtype=torch.int16, device="cuda")
+            plan.gemm(At.data_ptr(), want.data_ptr(), M, stream=s)
+            torch.cuda.synchronize()
+            tw.set_option(tw.OPT_LDS_DMA, 1)
+            outs = [torch.zeros((N, M), dtype=torch.int16, device="cuda") for _ in range(3)]
+            for rep in range(8):
+                print("direct loads, back to back:", name, rep, flush=True)
+                for c in outs:
+                    c.zero_()
+                for i in range(9):
+                    plan.gemm(At.data_ptr(), outs[i % 3].data_ptr(), M, stream=s)
+                torch.cuda.synchronize()
+                for c in outs:
+                    assert torch.equal(c, want), (name, rep)
+    finally:
+        tw.set_option(tw.OPT_SHAPE, -1)
+        tw.set_option(tw.OPT_LDS_DMA, -1)
+
+
 def test_cpp_driver_reference_command_line():
     """The C++ perf driver with the reference's command line (`./test_basic_nn M N K N_kept K_kept`,
     StreamMaskedGEMM/README.md:12-13) at a reduced M: its three self-checks (fused == gather /

@@ -36,10 +36,12 @@ MEASURED_TRAFFIC = {
     "bert_base_ffn_in": ((2 * 7897 + 24576) * 1024, "profiles/tw_gemm_as_kernel__bert_base_ffn.md (tw_gemm_as_kernel 64 rows)"),
     "nmt_lstm_gates": ((2 * 3558.5 + 1024) * 1024, "profiles/tw_gemm_skinny_kernel__nmt_lstm_gates.md (tw_gemm_skinny_kernel)"),
     "imbalance_stress": ((2 * 922921 + 209150) * 1024, "profiles/tw_gemm_ws_kernel__imbalance_stress.md (tw_gemm_ws_kernel 256x64)"),
+    "bert_large_ffn1_keep50": ((2 * 25220 + 65570) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn1_50.md (tw_gemm_ws_kernel 256x128)"),
+    "bert_large_ffn2_keep10": ((2 * 22280 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
     "bert_large_ffn2_keep50": ((2 * 49480 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
     "bert_large_ffn1_keep25": ((2 * 16649 + 65536) * 1024, "profiles/tw_gemm_as_kernel__bert_large_ffn1.md (tw_gemm_as_kernel 64 rows)"),
     "bert_large_ffn1_keep10": ((2 * 12319 + 65536) * 1024, "profiles/tw_gemm_bs_kernel__bert_large_ffn1_90.md (tw_gemm_bs_kernel)"),
-    "bert_large_ffn2_keep25": ((2 * 38143 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
+    "bert_large_ffn2_keep25": ((2 * 38160 + 16400) * 1024, "profiles/tw_gemm_ws_kernel__bert_large_ffn2.md (tw_gemm_ws_kernel 256x128)"),
 }
 
 

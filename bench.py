@@ -230,7 +230,7 @@ def time_nmt_recurrence(wl, steps, torch):
         start.record(torch.cuda.current_stream())
         plan.lstm_steps(steps, seq.data_ptr(), M, cell.data_ptr(), bias_ptr=bias.data_ptr(), stream=s)
         stop.record(torch.cuda.current_stream())
-        plan.lstm_steps_status(s)      # waits, and raises if the launch gave up at a barrier
+        plan.lstm_steps_status(s)      # waits, and raises if the launch gave up
         ts.append(start.elapsed_time(stop) * 1e-3 / steps)
     out.append(float(np.median(ts[1:])))
     plan.destroy()

@@ -309,7 +309,7 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  *                       unless nearly every tile keeps nearly every row (a 0 %-sparse plan);
  *                       2: dealt out over the dies in turn, row block after row block (all tiles
  *                       of a row block before the next) instead of tile after tile
- *   TW_OPT_SPIN_LIMIT   polls a workgroup of tw_lstm_steps spends at a barrier before it gives up
+ *   TW_OPT_SPIN_LIMIT   loads a wave of tw_lstm_steps spends looking for a step's h before it gives up
  *   TW_OPT_BALANCE      1: row blocks sized per tile where the items would not fill the chip once
  *   TW_OPT_LDS_DMA      0: the 256-row streaming kernels stage their loads through registers
  *                       instead of writing LDS directly (same results, bit for bit)
@@ -320,7 +320,7 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_WGS_PER_CU 1
 #define TW_OPT_PIECE 2
 #define TW_OPT_XCD_QUEUES 3
-#define TW_OPT_SPIN_LIMIT 4 /* polls a workgroup of tw_lstm_steps spends at a barrier before it gives up (default 2^20) */
+#define TW_OPT_SPIN_LIMIT 4 /* loads a wave of tw_lstm_steps spends looking for a step's h before it gives up (default 2^20) */
 #define TW_OPT_BALANCE 5 /* 1: a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows); 0 and automatic: every tile in row blocks of the kernel's full height (the benchmark shapes run no faster with 1) */
 #define TW_OPT_LDS_DMA 6 /* the 256-row streaming kernels (256 x 128, 256 x 64) with loads that write LDS directly: 0 never; 1 and automatic: wherever those shapes run */
 #define TW_N_OPTIONS 7
@@ -427,17 +427,20 @@ int tw_lstm_step(const tw_plan *plan, const void *A, int64_t lda, int M, const f
  * there.
  * Plans the fused step takes, with tiles of at most 512 kept rows and (H / 32) x ceil(M / 32)
  * no larger than the number of compute units, run as ONE persistent launch: weights, row
- * numbers, bias and cell state stay in registers, the workgroups meet at a barrier in device
- * memory between two steps.  That barrier needs every workgroup of the launch resident at
- * once; its polls are bounded (TW_OPT_SPIN_LIMIT), and a launch that gives up (the GPU was
- * shared with other work) sets a status word and drains: tw_lstm_steps_status then returns
- * TW_ERR_DEVICE.  Every other plan, and T == 1, runs as T calls of tw_lstm_step (gates_ws as
- * there).  Asynchronous on `stream`; at most 192 such launches of one plan in flight. */
+ * numbers, bias and cell state stay in registers, and the workgroups hand the rows of h to each
+ * other through A itself: the call first fills the rows of h of A_1 .. A_(T-1) (rows m < M) with
+ * the 16-bit pattern 0xFFFF, a step's stores go through to memory, and a workgroup that needs
+ * rows of h_t loads them until none shows the pattern (an h_t whose 16 bits come out as 0xFFFF, a
+ * NaN, is stored as 0xFFFE).  That needs every workgroup of the launch resident at once; the
+ * number of loads a wave spends looking is bounded (TW_OPT_SPIN_LIMIT), and a launch in which a
+ * wave gives up (the GPU was shared with other work) sets a status word and drains:
+ * tw_lstm_steps_status then returns TW_ERR_DEVICE.  Every other plan, and T == 1, runs as T
+ * calls of tw_lstm_step (gates_ws as there).  Asynchronous on `stream`. */
 int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, int64_t a_step, int M,
                   const float *bias, float forget_bias, float *c, int64_t ldc, void *gates_ws,
                   int64_t ldg, void *stream);
-/* Waits for `stream` and returns TW_ERR_DEVICE if a tw_lstm_steps launch of the plan gave up at
- * its barrier since the last call (and clears that), else TW_OK. */
+/* Waits for `stream` and returns TW_ERR_DEVICE if a tw_lstm_steps launch of the plan gave up
+ * waiting for a step's h since the last call (and clears that), else TW_OK. */
 int tw_lstm_steps_status(const tw_plan *plan, void *stream);
 
 /* ---- TW mask producers ---------------------------------------------------------------

@@ -305,7 +305,7 @@ def _oracle_recurrence(oracle, W, bias, tiles, xs, h0, c0, dtype):
                                               (120, 1024, 1024, 128, 0.25, 4)])  # the NMT cell
 def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
     """tw_lstm_steps: T time steps in one persistent launch (weights, row numbers and the cell state
-    stay in registers; a barrier in device memory between the steps).  Every h_t and the final c
+    stay in registers; the rows of h are handed from step to step through memory).  Every h_t and the final c
     against the oracle's recurrence (2 x the GEMM tolerance: errors of h feed the next step), within
     the same bound of T calls of tw_lstm_step, the same bits on a second launch, nothing written beyond
     M or into the rows of x, and a clean status."""
@@ -319,14 +319,22 @@ def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
     s = torch.cuda.current_stream().cuda_stream
     outs = []
     with tw.Plan.create(K, 4 * H, dtype, tiles, W) as plan:
-        for mode in ("steps", "steps", "single"):
+        for mode in ("steps", "steps", "single", "reuse"):
             dA = to_device_bits(A, A.shape)
             dC = torch.from_numpy(c.copy()).cuda()
             print("multi-step launch:", mode, M, I, H, G, T, dtype, flush=True)
-            if mode == "steps":
+            if mode == "reuse":
+                # the same buffers once more after a launch from another cell state: nothing of that
+                # launch's h may be read again (its rows of h linger in the caches)
+                dC.add_(0.75)
                 plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld,
                                 bias_ptr=dbias.data_ptr(), stream=s)
-                plan.lstm_steps_status(s)          # waits; raises if a barrier gave up
+                dA.copy_(to_device_bits(A, A.shape))
+                dC.copy_(torch.from_numpy(c.copy()).cuda())
+            if mode in ("steps", "reuse"):
+                plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld,
+                                bias_ptr=dbias.data_ptr(), stream=s)
+                plan.lstm_steps_status(s)          # waits; raises if a wave gave up
             else:
                 for t in range(T):
                     plan.lstm_step(dA[t].data_ptr(), M, dC.data_ptr(), dC.data_ptr(),
@@ -346,6 +354,7 @@ def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
     # (the two kernels' cell arithmetic is contracted into fused multiply-adds differently, and a
     # last-bit difference of h_t then feeds every later step)
     assert np.array_equal(a_bits, outs[1][0]) and np.array_equal(c_out, outs[1][1])
+    assert np.array_equal(a_bits, outs[3][0]) and np.array_equal(c_out, outs[3][1])
     single_h = oracle.bits_to_f32(np.ascontiguousarray(outs[2][0][1:, I:, :M]), dtype)
     steps_h = oracle.bits_to_f32(np.ascontiguousarray(a_bits[1:, I:, :M]), dtype)
     assert oracle.rel_error(steps_h, single_h) <= 2 * TOL[dtype]
@@ -354,9 +363,9 @@ def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
 
 
 def test_multi_step_launch_gives_up_cleanly(tw, oracle):
-    """The barrier's polls are bounded.  With no polls allowed at all a workgroup gives up at its
-    first barrier unless it happens to arrive last; every workgroup then leaves normally, the call
-    after it reports TW_ERR_DEVICE once, and the plan works again afterwards."""
+    """The loads a wave spends looking for a step's h are bounded.  With none allowed at all every
+    wave that needs rows of h gives up at the second step; every workgroup then leaves normally,
+    the call after it reports TW_ERR_DEVICE once, and the plan works again afterwards."""
     import torch
     rng = np.random.default_rng(5)
     M, I, H, G, T, dtype = 128, 64, 256, 128, 4, "f16"

@@ -346,24 +346,30 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_step_kernel(const 
 // step above (workgroup = 32 hidden units x 32 rows, wave = one gate and every second step of 64
 // kept rows), but the weight fragments, the row offsets, the bias and the cell state of a
 // workgroup are fetched once and stay in registers for all T steps; per step a workgroup reads
-// its rows of A_t = [x_t ; h_(t-1)], multiplies, applies the cell, writes its piece of h_t into
-// the rows of A_(t+1), and meets all other workgroups at a barrier in device memory before it
-// reads the rows of h of A_(t+1).  The rows of x of A_(t+1) do not wait: the steps of a tile's
-// kept rows that hold nothing else are fetched and multiplied while the barrier fills.
+// its rows of A_t = [x_t ; h_(t-1)], multiplies, applies the cell and writes its piece of h_t into
+// the rows of A_(t+1).  No barrier between the steps: the data is its own flag.
+//   hand-over: a launch before this one fills the rows of h of A_1 .. A_(T-1) (rows m below M)
+//           with the 16-bit pattern 0xFFFF, which no step ever stores (a NaN of that pattern is
+//           stored as 0xFFFE).  A wave that needs rows of h loads them and looks at what came: a
+//           piece that still shows the pattern has not been written yet, and the wave loads its
+//           rows again.  So a step costs one store's way to memory and one load's way back, not
+//           the round trips of a counter on top of them.  The rows of x of A_(t+1) do not wait:
+//           the steps of a tile's kept rows that hold nothing else are fetched with the rows of h
+//           of A_t and multiplied before the wave looks for h_t.
 //   coherence: h crosses from one die to another between two steps.  Its stores write through
 //           (sc0 sc1) and the loads of steps that hold rows of h bypass the die's L2 (sc0 sc1), so
 //           no cache is written back or invalidated inside the launch.
-//   barrier: one counter; a workgroup waits for its own stores, adds one and polls until the
-//           counter has reached (t + 1) x workgroups.  The poll is bounded: a workgroup that runs
-//           out of polls (the launch does not fit the chip next to whatever else runs there, so
-//           some workgroup never started) sets the status word and leaves; every other
-//           workgroup then runs out of polls too, and the host reports the launch as failed.
+//   bounds: the number of loads a wave spends on one step's rows is bounded.  A wave that runs out
+//           (the launch does not fit the chip next to whatever else runs there, so some
+//           workgroup never started) sets the status word, stops looking and runs its remaining
+//           steps on whatever it reads; the host reports the launch as failed.
 //   edges:  A_t is addressed through a buffer descriptor; the padding of a list of kept rows and
 //           rows m beyond M get an offset beyond the buffer, for which the hardware delivers
-//           zeros.
+//           zeros.  Elements m >= M inside a 16-byte piece are the caller's and are not looked at.
 constexpr int kSeqSteps = 4; // steps of 64 kept rows a wave holds in registers: tiles of at most 512 kept rows
 constexpr int kSeqRsrcFlags = 0x00020000;
 constexpr int kSeqAuxCoherent = 1 | 16; // sc0 sc1
+constexpr uint32_t kSeqUnwritten = 0xFFFFu; // 16-bit fill pattern of rows of h that no step has stored yet
 
 struct LstmSeqArgs {
     const void *A;
@@ -371,8 +377,7 @@ struct LstmSeqArgs {
     const void *Bp;
     const float *bias;
     float *c;
-    int32_t *sync;   // arrivals at the barrier: zero at the start
-    int32_t *status; // set to 1 by a workgroup that gave up
+    int32_t *status; // set to 1 by a wave that gave up
     int64_t lda, a_step, ldc;
     int32_t M, H, K, T;
     float forget_bias;
@@ -394,12 +399,10 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
     constexpr int STEPB = kBlockK * PITCH;
     constexpr int RPT = RB / 16;      // rows of a hidden unit a thread applies the cell to
     __shared__ __align__(16) unsigned char smem[kLstmWaves * kLstmStage];
-    __shared__ int s_ok;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int gate = wave >> 1, kh = wave & 1;
     const int hb = blockIdx.x, m0 = blockIdx.y * RB;
-    const int n_wgs = gridDim.x * gridDim.y;
     const LstmBlk blk = p.blk[hb * 4 + gate];
     const int nsteps = (blk.k_kept + kBlockK - 1) / kBlockK;
     unsigned char *const stage = smem + wave * kLstmStage;
@@ -410,6 +413,7 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
     const bool m_ok = m0 + ch * 8 < p.M;
     u32x4 bq[kSeqSteps][4];
     uint32_t voff[kSeqSteps][LPS];
+    uint32_t h_loads = 0; // bit i * LPS + r: load r of step i fetches a row of h
     {
         TW_GLOBAL(const unsigned char) const bsrc = (TW_GLOBAL(const unsigned char))p.Bp + blk.b_first + lane * 16;
         int rows[kSeqSteps][LPS];
@@ -431,7 +435,16 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
                 voff[i][r] = (kk < blk.k_kept && m_ok)
                                  ? (uint32_t)rows[i][r] * ((uint32_t)p.lda * 2u) + (uint32_t)(m0 + ch * 8) * 2u
                                  : 0xFFFFFFF0u;
+                if (kk < blk.k_kept && m_ok && rows[i][r] >= p.K - p.H)
+                    h_loads |= 1u << (i * LPS + r);
             }
+    }
+    // the elements of this lane's 16-byte piece that lie below M, as masks of its four words
+    uint32_t below_m[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const int m = m0 + ch * 8 + 2 * d;
+        below_m[d] = (m < p.M ? 0xFFFFu : 0u) | (m + 1 < p.M ? 0xFFFF0000u : 0u);
     }
     const int my_steps = nsteps > kh ? (nsteps - kh + 1) / 2 : 0; // <= kSeqSteps (host check)
     // The first n_pre of this wave's steps hold rows of x only (a list of kept rows ascends, and
@@ -520,13 +533,80 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     };
 
+    // the word lane l looks at before it fetches rows of h: the last one workgroup (l, this row
+    // block) stores, hidden unit 32 l + 31, the last two rows m of the block below M
+    const int probe_m = m0 + ((min(p.M - m0, RB) - 1) & ~1);
+    const uint32_t probe_off = lane < (int)gridDim.x
+                                   ? (uint32_t)(p.K - p.H + 32 * lane + 31) * ((uint32_t)p.lda * 2u) + (uint32_t)probe_m * 2u
+                                   : 0xFFFFFFF0u; // (beyond the buffer: zeros)
+    const uint32_t probe_mask = probe_m + 1 < p.M ? 0xFFFFFFFFu : 0xFFFFu;
+    // whether a piece of this wave's rows of h of a step still shows the fill pattern
+    auto unwritten = [&]() {
+        uint32_t bad = 0;
+#pragma unroll
+        for (int i = 0; i < kSeqSteps; ++i)
+            if (i >= n_pre && i < my_steps) {
+#pragma unroll
+            for (int r = 0; r < LPS; ++r) {
+                const uint32_t w[4] = {av[i][r].x, av[i][r].y, av[i][r].z, av[i][r].w};
+                uint32_t hit = 0;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) {
+                    const uint32_t x = ~(w[d] & below_m[d]); // a 16-bit half of zeros: all ones below M
+                    hit |= (x - 0x00010001u) & ~x & 0x80008000u;
+                }
+                bad |= (h_loads >> (i * LPS + r)) & 1u ? hit : 0u;
+            }
+            }
+        return __builtin_amdgcn_ballot_w64(bad != 0) != 0;
+    };
+
     clear();
     load_steps(0, 0, n_pre, false);
     multiply_steps(0, n_pre);
+    bool gave_up = false;
     for (int t = 0; t < p.T; ++t) {
-        // ---- the steps that hold rows of h (of the step before: behind the barrier); the next
-        // step's rows of x leave right behind them, so that one trip to memory covers both
-        load_steps(t, n_pre, my_steps, true);
+        // ---- the steps that hold rows of h (of the step before).  For t > 0 the wave
+        // first looks at one word of every workgroup that writes rows it needs (the last one
+        // each of them stores, past the caches) until none shows the fill pattern, then fetches
+        // its rows through the L2 like any others (the 16 workgroups of a die ask for the same
+        // lines), and falls back to loads past the L2 for what still shows the pattern: a line
+        // another workgroup of the die fetched too early.
+        bool look = t > 0 && !gave_up && h_loads != 0; // (A_0 holds the caller's h)
+        int left = p.spin_limit;
+        if (look) {
+            const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<uint16_t *>(A0 + (int64_t)t * p.a_step), 0, (int)p.a_bytes, kSeqRsrcFlags);
+            for (;;) {
+                if (left <= 0)
+                    break;
+                --left;
+                const uint32_t w = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)probe_off, 0, kSeqAuxCoherent);
+                const uint32_t x = ~(w & probe_mask);
+                const bool fresh = ((x - 0x00010001u) & ~x & 0x80008000u) != 0;
+                if (__builtin_amdgcn_ballot_w64(fresh) == 0)
+                    break;
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        load_steps(t, n_pre, my_steps, false);
+        if (look) {
+            for (;;) {
+                if (left <= 0) {
+                    gave_up = true;
+                    if (lane == 0)
+                        __hip_atomic_store(p.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    break;
+                }
+                if (!unwritten())
+                    break;
+                --left;
+                __builtin_amdgcn_s_sleep(1);
+                load_steps(t, n_pre, my_steps, true);
+            }
+        }
+        // the next step's rows of x leave now: they travel while this step is multiplied and
+        // the cell applied (together with the rows of h they would only hold those up)
         if (t + 1 < p.T)
             load_steps(t + 1, 0, n_pre, false);
         multiply_steps(n_pre, my_steps);
@@ -552,43 +632,30 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
 #pragma unroll
             for (int e = 0; e < RPT; ++e)
                 cell_update(pre[0][e], pre[1][e], pre[2][e], pre[3][e], p.forget_bias, c2[e], h2[e]);
-            // h_t into the rows of A_(t+1) that hold h; written through, for the other dies
+            // h_t into the rows of A_(t+1) that hold h; written through, for the other dies.  The
+            // fill pattern is never stored: it would read as "not written yet".
             uint16_t *const hdst = const_cast<uint16_t *>(A0) + (int64_t)(t + 1) * p.a_step +
                                    (int64_t)(p.K - p.H + hu) * p.lda + m0 + mt;
+            uint32_t h16[RPT];
+#pragma unroll
+            for (int e = 0; e < RPT; ++e) {
+                h16[e] = to16(h2[e], DT);
+                h16[e] = h16[e] == kSeqUnwritten ? kSeqUnwritten - 1u : h16[e];
+            }
             if (RPT == 2 && row_ok[RPT - 1]) {
-                const uint32_t w = (uint32_t)to16(h2[0], DT) | ((uint32_t)to16(h2[RPT - 1], DT) << 16);
+                const uint32_t w = h16[0] | (h16[RPT - 1] << 16);
                 asm volatile("global_store_dword %0, %1, off sc0 sc1" ::"v"(hdst), "v"(w) : "memory");
             } else if (row_ok[0]) {
-                const uint32_t w = to16(h2[0], DT);
+                const uint32_t w = h16[0];
                 asm volatile("global_store_short %0, %1, off sc0 sc1" ::"v"(hdst), "v"(w) : "memory");
             }
         }
         if (t + 1 == p.T)
             break;
-        // ---- the barrier between two steps, with the next step's rows of x multiplied on the way
+        // ---- the next step's rows of x, multiplied while h_t travels
         clear();
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this thread's piece of h is out
-        __syncthreads();                                  // (and the partial sums have been read)
-        if (tid == 0)
-            __hip_atomic_fetch_add(p.sync, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads(); // the partial sums have been read: the stages may be written again
         multiply_steps(0, n_pre);
-        if (tid == 0) {
-            const int target = (t + 1) * n_wgs;
-            int ok = 0;
-            for (int polls = p.spin_limit; polls > 0; --polls) {
-                if (__hip_atomic_load(p.sync, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) >= target) {
-                    ok = 1;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(1);
-            }
-            if (!ok)
-                __hip_atomic_store(p.status, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            s_ok = ok;
-        }
-        __syncthreads();
-        if (!s_ok)
-            return; // every other workgroup runs out of polls as well: the grid drains
     }
 #pragma unroll
     for (int e = 0; e < RPT; ++e)
@@ -596,10 +663,24 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
             p.c[(int64_t)hu * p.ldc + m0 + mt + e] = c2[e];
 }
 
-__global__ void clear_sync_kernel(int32_t *sync)
+// Fills the rows of h of A_1 .. A_(T-1), rows m below M, with the pattern tw_lstm_steps_kernel
+// takes for "not written yet".  One thread per 16-byte piece (8 rows m) of a row.
+__global__ void lstm_mark_unwritten_kernel(uint16_t *A, int64_t lda, int64_t a_step, int M, int H, int K, int T)
 {
-    if (threadIdx.x < 16)
-        sync[threadIdx.x] = 0;
+    const int pieces = (M + 7) / 8;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)(T - 1) * H * pieces)
+        return;
+    const int pc = (int)(i % pieces);
+    const int64_t row = i / pieces;
+    uint16_t *const dst = A + (row / H + 1) * a_step + (int64_t)(K - H + row % H) * lda + pc * 8;
+    if (pc * 8 + 8 <= M) {
+        const uint32_t w = kSeqUnwritten | (kSeqUnwritten << 16);
+        *reinterpret_cast<u32x4 *>(dst) = u32x4{w, w, w, w};
+    } else {
+        for (int e = 0; pc * 8 + e < M; ++e)
+            dst[e] = (uint16_t)kSeqUnwritten;
+    }
 }
 
 // what tw_lstm_step and tw_lstm_steps have in common: whether the fused kernels take the plan
@@ -763,10 +844,7 @@ extern "C" int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, i
     a.Bp = plan->d_Bp;
     a.bias = bias;
     a.c = c;
-    // a ticket slot of the plan holds the barrier's counter; the word behind the slots its status
-    const unsigned slot = __atomic_fetch_add(&plan->next_slot, 1u, __ATOMIC_RELAXED) % (unsigned)kEagerSlots;
-    a.sync = plan->d_tickets + kTicketInts * slot;
-    a.status = plan->d_tickets + kTicketInts * kTicketSlots;
+    a.status = plan->d_tickets + kTicketInts * kTicketSlots; // the word behind the plan's ticket slots
     a.lda = lda;
     a.a_step = a_step;
     a.ldc = ldc;
@@ -779,8 +857,12 @@ extern "C" int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, i
     a.spin_limit = limit >= 0 ? limit : (1 << 20);
     a.a_bytes = (uint32_t)((uint64_t)K * (uint64_t)lda * 2u);
     lstm_fill_blocks(plan, H, a.blk);
-    // (a kernel, not a memset: the call may be recorded into a graph)
-    hipLaunchKernelGGL(clear_sync_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, a.sync);
+    // the rows of h the steps will hand to each other start out as "not written yet"
+    if (T > 1) {
+        const int64_t n = (int64_t)(T - 1) * H * ((M + 7) / 8);
+        hipLaunchKernelGGL(lstm_mark_unwritten_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                           A16, lda, a_step, M, H, K, T);
+    }
     const dim3 grid((unsigned)(H / 32), (unsigned)row_blocks), block(64 * kLstmWaves);
     if (plan->dtype == TW_F16)
         hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_F16, 32>), grid, block, 0, (hipStream_t)stream, a);
@@ -803,8 +885,8 @@ extern "C" int tw_lstm_steps_status(const tw_plan *plan, void *stream)
     if (v == 0)
         return TW_OK;
     TW_HIP(hipMemset(word, 0, sizeof v));
-    return fail(TW_ERR_DEVICE, "a multi-step LSTM launch of this plan gave up at its barrier (its workgroups were not all "
-                               "resident at once); h and c of that call are undefined");
+    return fail(TW_ERR_DEVICE, "a multi-step LSTM launch of this plan gave up waiting for a step's h (its workgroups were not "
+                               "all resident at once); h and c of that call are undefined");
 }
 
 extern "C" int tw_lstm_gates(int M, int H, int dtype, const void *gates, int64_t ldg,

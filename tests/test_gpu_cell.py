@@ -362,6 +362,49 @@ def test_multi_step_launch(tw, oracle, dtype, M, I, H, G, k_keep, T):
     assert np.array_equal(outs[2][0][:, :I, :], A[:, :I, :])
 
 
+def test_multi_step_launch_in_a_graph(tw, oracle):
+    """tw_lstm_steps records into a HIP graph (its fill of the rows of h is a kernel, not a memset):
+    the graph is replayed four times on inputs restored in between, with eager launches of the same
+    plan between the replays, and every replay gives the eager call's bits."""
+    import torch
+    rng = np.random.default_rng(77)
+    M, I, H, G, T, dtype = 96, 128, 256, 128, 5, "bf16"
+    K, ld = I + H, 96
+    W, bias, tiles, xs, h0, c0, A, c = _sequence_problem(rng, oracle, M, I, H, G, 0.4, T, dtype, ld)
+    dbias = torch.from_numpy(bias).cuda()
+    s = torch.cuda.Stream()
+    with tw.Plan.create(K, 4 * H, dtype, tiles, W) as plan:
+        with torch.cuda.stream(s):
+            A0, C0 = to_device_bits(A, A.shape), torch.from_numpy(c.copy()).cuda()
+            dA, dC = A0.clone(), C0.clone()
+            other_a, other_c = A0.clone(), C0.clone()
+
+            def steps(a, cc):
+                plan.lstm_steps(T, a.data_ptr(), M, cc.data_ptr(), lda=ld, a_step=K * ld, ldc=ld,
+                                bias_ptr=dbias.data_ptr(), stream=s.cuda_stream)
+            print("multi-step launch, eager then in a graph", flush=True)
+            steps(dA, dC)
+            plan.lstm_steps_status(s.cuda_stream)
+            want_a, want_c = dA.clone(), dC.clone()
+            dA.copy_(A0)
+            dC.copy_(C0)
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=s):
+                steps(dA, dC)
+            for rep in range(4):
+                dA.copy_(A0)
+                dC.copy_(C0)
+                other_c.copy_(C0 + rep)              # eager work of the same plan between the replays
+                steps(other_a, other_c)
+                s.synchronize()
+                g.replay()
+                plan.lstm_steps_status(s.cuda_stream)
+                assert torch.equal(dA, want_a) and torch.equal(dC, want_c), rep
+    want_h, want_cc = _oracle_recurrence(oracle, W, bias, tiles, xs, h0, c0, dtype)
+    got = oracle.bits_to_f32(np.ascontiguousarray(from_device_bits(want_a)[T, I:, :M]), dtype).reshape(H, M).T
+    assert oracle.rel_error(got, want_h[-1]) <= 2 * TOL[dtype]
+
+
 def test_multi_step_launch_gives_up_cleanly(tw, oracle):
     """The loads a wave spends looking for a step's h are bounded.  With none allowed at all every
     wave that needs rows of h gives up at the second step; every workgroup then leaves normally,

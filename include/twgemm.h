@@ -313,9 +313,12 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
  *   TW_OPT_BALANCE      1: row blocks sized per tile where the items would not fill the chip once
  *   TW_OPT_LDS_DMA      0: the 256-row streaming kernels stage their loads through registers
  *                       instead of writing LDS directly (same results, bit for bit)
+ *   TW_OPT_LSTM_LOOK    0: a wave of tw_lstm_steps fetches a step's rows of h at once, past the
+ *                       caches, and again until they are all there, instead of first looking at
+ *                       one word of every workgroup that writes them (same results, slower)
  * Initial values come from the environment variables TWGEMM_SHAPE, TWGEMM_WGS_PER_CU,
- * TWGEMM_PIECE, TWGEMM_XCD_QUEUES, TWGEMM_SPIN_LIMIT, TWGEMM_BALANCE and TWGEMM_LDS_DMA, read
- * once. */
+ * TWGEMM_PIECE, TWGEMM_XCD_QUEUES, TWGEMM_SPIN_LIMIT, TWGEMM_BALANCE, TWGEMM_LDS_DMA and
+ * TWGEMM_LSTM_LOOK, read once. */
 #define TW_OPT_SHAPE 0
 #define TW_OPT_WGS_PER_CU 1
 #define TW_OPT_PIECE 2
@@ -323,7 +326,8 @@ int tw_gemm_staged(const tw_plan *plan, const void *A, int a_layout, int64_t lda
 #define TW_OPT_SPIN_LIMIT 4 /* loads a wave of tw_lstm_steps spends looking for a step's h before it gives up (default 2^20) */
 #define TW_OPT_BALANCE 5 /* 1: a launch whose items would not fill the chip once gives the tiles with more kept rows lower row blocks (multiples of 64 rows); 0 and automatic: every tile in row blocks of the kernel's full height (the benchmark shapes run no faster with 1) */
 #define TW_OPT_LDS_DMA 6 /* the 256-row streaming kernels (256 x 128, 256 x 64) with loads that write LDS directly: 0 never; 1 and automatic: wherever those shapes run */
-#define TW_N_OPTIONS 7
+#define TW_OPT_LSTM_LOOK 7 /* tw_lstm_steps: 1 and automatic: a wave looks at one word per writing workgroup before it fetches a step's rows of h; 0: it fetches the rows themselves until none shows the fill pattern */
+#define TW_N_OPTIONS 8
 #define TW_SHAPE_WIDE 0    /* 256 x 128 items, 64-bit row addressing (operands beyond 4 GiB) */
 #define TW_SHAPE_128x128 1 /* wave-specialised, 128 rows x 128 columns, two workgroups per CU */
 #define TW_SHAPE_512x64 2  /* wave-specialised, 512 x 64: tiles of at most 64 kept columns (forced only: 256 x 64 is ahead) */

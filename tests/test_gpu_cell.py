@@ -405,6 +405,38 @@ def test_multi_step_launch_in_a_graph(tw, oracle):
     assert oracle.rel_error(got, want_h[-1]) <= 2 * TOL[dtype]
 
 
+def test_multi_step_launch_without_the_first_look(tw, oracle):
+    """TW_OPT_LSTM_LOOK = 0: the waves fetch a step's rows of h at once and again until none shows
+    the fill pattern (the path a wave otherwise takes only for a line that was fetched too early).
+    Same bits as the default form."""
+    import torch
+    rng = np.random.default_rng(78)
+    M, I, H, G, T, dtype = 120, 192, 512, 128, 6, "f16"
+    K, ld = I + H, 120
+    W, bias, tiles, xs, h0, c0, A, c = _sequence_problem(rng, oracle, M, I, H, G, 0.3, T, dtype, ld)
+    dbias = torch.from_numpy(bias).cuda()
+    s = torch.cuda.current_stream().cuda_stream
+    outs = []
+    with tw.Plan.create(K, 4 * H, dtype, tiles, W) as plan:
+        try:
+            for look in (-1, 0, 0):
+                tw.set_option(tw.OPT_LSTM_LOOK, look)
+                dA = to_device_bits(A, A.shape)
+                dC = torch.from_numpy(c.copy()).cuda()
+                print("multi-step launch, first look", look, flush=True)
+                plan.lstm_steps(T, dA.data_ptr(), M, dC.data_ptr(), lda=ld, a_step=K * ld, ldc=ld,
+                                bias_ptr=dbias.data_ptr(), stream=s)
+                plan.lstm_steps_status(s)
+                outs.append((from_device_bits(dA).copy(), dC.cpu().numpy().copy()))
+        finally:
+            tw.set_option(tw.OPT_LSTM_LOOK, -1)
+    for a_bits, c_out in outs[1:]:
+        assert np.array_equal(a_bits, outs[0][0]) and np.array_equal(c_out, outs[0][1])
+    want_h, want_c = _oracle_recurrence(oracle, W, bias, tiles, xs, h0, c0, dtype)
+    got = oracle.bits_to_f32(np.ascontiguousarray(outs[0][0][T, I:, :M]), dtype).reshape(H, M).T
+    assert oracle.rel_error(got, want_h[-1]) <= 2 * TOL[dtype]
+
+
 def test_multi_step_launch_gives_up_cleanly(tw, oracle):
     """The loads a wave spends looking for a step's h are bounded.  With none allowed at all every
     wave that needs rows of h gives up at the second step; every workgroup then leaves normally,

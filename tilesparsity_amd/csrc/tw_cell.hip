@@ -388,8 +388,9 @@ struct LstmSeqArgs {
 };
 static_assert(sizeof(LstmSeqArgs) <= 4096, "kernel arguments");
 
-// RB rows m of A per workgroup (32 is what the launch uses).
-template <int DT, int RB>
+// RB rows m of A per workgroup (32 is what the launch uses).  LOOK false: without the first look at
+// one word per writing workgroup (the fall-back path alone; TW_OPT_LSTM_LOOK = 0).
+template <int DT, int RB, bool LOOK>
 __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const LstmSeqArgs p)
 {
     static_assert(RB == 32 || RB == 16, "rows of a workgroup");
@@ -574,7 +575,7 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
         // another workgroup of the die fetched too early.
         bool look = t > 0 && !gave_up && h_loads != 0; // (A_0 holds the caller's h)
         int left = p.spin_limit;
-        if (look) {
+        if (look && LOOK) {
             const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<uint16_t *>(A0 + (int64_t)t * p.a_step), 0, (int)p.a_bytes, kSeqRsrcFlags);
             for (;;) {
@@ -589,7 +590,7 @@ __global__ void __launch_bounds__(64 * kLstmWaves, 1) tw_lstm_steps_kernel(const
                 __builtin_amdgcn_s_sleep(1);
             }
         }
-        load_steps(t, n_pre, my_steps, false);
+        load_steps(t, n_pre, my_steps, !LOOK && look); // (without the first look: past the caches at once)
         if (look) {
             for (;;) {
                 if (left <= 0) {
@@ -864,10 +865,18 @@ extern "C" int tw_lstm_steps(const tw_plan *plan, int T, void *A, int64_t lda, i
                            A16, lda, a_step, M, H, K, T);
     }
     const dim3 grid((unsigned)(H / 32), (unsigned)row_blocks), block(64 * kLstmWaves);
-    if (plan->dtype == TW_F16)
-        hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_F16, 32>), grid, block, 0, (hipStream_t)stream, a);
-    else
-        hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_BF16, 32>), grid, block, 0, (hipStream_t)stream, a);
+    const bool first_look = get_option(TW_OPT_LSTM_LOOK) != 0;
+    if (plan->dtype == TW_F16) {
+        if (first_look)
+            hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_F16, 32, true>), grid, block, 0, (hipStream_t)stream, a);
+        else
+            hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_F16, 32, false>), grid, block, 0, (hipStream_t)stream, a);
+    } else {
+        if (first_look)
+            hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_BF16, 32, true>), grid, block, 0, (hipStream_t)stream, a);
+        else
+            hipLaunchKernelGGL((tw_lstm_steps_kernel<TW_BF16, 32, false>), grid, block, 0, (hipStream_t)stream, a);
+    }
     TW_HIP(hipGetLastError());
     return TW_OK;
 }

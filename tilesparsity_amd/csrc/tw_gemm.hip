@@ -2404,13 +2404,12 @@ template <int DT> static void launch_kmajor(int shape, const GemmArgs &a, int gr
 }
 
 // Process-wide tuning switches (tw_set_option); -1 = automatic.  The environment variables
-// TWGEMM_SHAPE, TWGEMM_WGS_PER_CU, TWGEMM_PIECE and TWGEMM_XCD_QUEUES give their initial values
-// and are read once.
+// named in kOptEnv give their initial values and are read once.
 static std::atomic<int> g_opt[TW_N_OPTIONS];
 static std::once_flag g_opt_once;
 static const char *const kOptEnv[TW_N_OPTIONS] = {"TWGEMM_SHAPE", "TWGEMM_WGS_PER_CU", "TWGEMM_PIECE",
                                                   "TWGEMM_XCD_QUEUES", "TWGEMM_SPIN_LIMIT", "TWGEMM_BALANCE",
-                                                  "TWGEMM_LDS_DMA"};
+                                                  "TWGEMM_LDS_DMA", "TWGEMM_LSTM_LOOK"};
 
 static bool option_in_range(int option, int value)
 {
@@ -2429,6 +2428,7 @@ static bool option_in_range(int option, int value)
         return value >= 0;
     case TW_OPT_BALANCE:
     case TW_OPT_LDS_DMA:
+    case TW_OPT_LSTM_LOOK:
         return value == 0 || value == 1;
     }
     return false;

@@ -24,7 +24,7 @@ F16, BF16 = 0, 1
 KMAJOR, ROWMAJOR = 0, 1
 PRUNED_UNTOUCHED, PRUNED_ZERO = 0, 1
 ACT_NONE, ACT_RELU, ACT_GELU, ACT_TANH = 0, 1, 2, 3
-OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES, OPT_SPIN_LIMIT, OPT_BALANCE, OPT_LDS_DMA = 0, 1, 2, 3, 4, 5, 6
+OPT_SHAPE, OPT_WGS_PER_CU, OPT_PIECE, OPT_XCD_QUEUES, OPT_SPIN_LIMIT, OPT_BALANCE, OPT_LDS_DMA, OPT_LSTM_LOOK = 0, 1, 2, 3, 4, 5, 6, 7
 SHAPE_AS64, SHAPE_AS32, SHAPE_SKINNY, SHAPE_BS = 7, 8, 9, 10
 SHAPE_WIDE, SHAPE_128x128, SHAPE_512x64, SHAPE_128x64, SHAPE_256x128, SHAPE_128x32, SHAPE_256x64 = range(7)
 SHAPE_NAMES = ("tw_gemm_kmajor_kernel 256x128", "tw_gemm_ws_kernel 128x128", "tw_gemm_ws_kernel 512x64",
